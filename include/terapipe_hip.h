@@ -1,0 +1,163 @@
+/*
+ * C ABI of libterapipe_hip.so -- the MI355X (gfx950) kernels behind the sliced GPT-layer hot path.
+ *
+ * The reference (zhuohan123/terapipe) is pure Python on PyTorch and has no FFI layer; each entry
+ * point below replaces the ATen call(s) the reference makes at the cited lines.  Conventions:
+ *   - every pointer is a raw device pointer owned by the caller (PyTorch owns all memory); the
+ *     library never allocates or frees device memory and keeps no state between calls
+ *     (exception, stated at its declaration: none in this version);
+ *   - `stream` is a hipStream_t passed as void*; launches are asynchronous on it, no internal syncs;
+ *   - every function returns 0 on success or a tp_status code; tp_last_error() gives the message of
+ *     the calling thread's last failure.  Nothing throws, nothing aborts;
+ *   - dtype is a tp_dtype; fp16/bf16 compute with fp32 accumulation on MFMA, fp32 uses fp32 MFMA.
+ *   - rows of every matrix are contiguous; leading dimensions and the contiguous extents must be
+ *     multiples of 16 bytes worth of elements (8 for fp16/bf16, 4 for fp32) and pointers 16-byte aligned.
+ */
+#ifndef TERAPIPE_HIP_H_
+#define TERAPIPE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { TP_F32 = 0, TP_F16 = 1, TP_BF16 = 2 } tp_dtype;
+
+typedef enum {
+    TP_OK = 0,
+    TP_ERR_ARG = 1,         /* null pointer, bad shape, misalignment */
+    TP_ERR_UNSUPPORTED = 2, /* shape or dtype outside what the kernels cover */
+    TP_ERR_WORKSPACE = 3,   /* workspace missing or too small */
+    TP_ERR_LAUNCH = 4       /* HIP reported a launch error */
+} tp_status;
+
+int tp_version(void);
+const char* tp_last_error(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * LayerNorm over the last dimension of x[M, E]  (replaces nn.LayerNorm at transformer_models.py:275
+ * and :280; modules built at :323, :325).  Statistics in fp32; mean/rstd [M] are saved for backward.
+ */
+int tp_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
+                     float* rstd, int M, int E, float eps, int dtype, void* stream);
+
+/* Backward of the above fused with the residual-path add that follows it in the layer
+ * (transformer_models.py:277, :284 are `x += y`, so the gradient of the LayerNorm input is
+ * LN'(dy) + dres).  dres may be NULL.  The parameter gradients are ADDED into fp32 accumulators:
+ *   dgamma_acc[E] += sum_m dy * xhat,   dbeta_acc[E] += sum_m dy,
+ *   colsum_dres_acc[E] += sum_m dres    (NULL to skip; this is the bias gradient of the
+ *                                        row-parallel linear whose output fed the residual add),
+ *   colsum_dx_acc[E]  += sum_m dx       (NULL to skip; bias gradient of the linear that produced
+ *                                        the LayerNorm's input branch).
+ */
+int tp_layernorm_bwd(const void* dy, const void* x, const float* mean, const float* rstd,
+                     const void* gamma, const void* dres, void* dx, float* dgamma_acc,
+                     float* dbeta_acc, float* colsum_dres_acc, float* colsum_dx_acc, int M, int E,
+                     int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * GEMMs that mpu.ColumnParallelLinear / RowParallelLinear reduce to at tensor-parallel size 1
+ * (F.linear at mpu/layers.py:256 and :335, and their autograd backward), with the elementwise work
+ * around them fused into the epilogue.
+ */
+typedef enum {
+    TP_GEMM_NT = 0, /* C[M,N] = A[M,K] . B[N,K]^T   forward  Y = X W^T        (W stored [out,in]) */
+    TP_GEMM_NN = 1, /* C[M,N] = A[M,K] . B[K,N]     data grad dX = dY W                          */
+    TP_GEMM_TN = 2  /* C[M,N] = A[K,M]^T . B[K,N]   weight grad dW = dY^T X                      */
+} tp_gemm_op;
+
+typedef enum {
+    TP_EPI_STORE = 0,         /* C = acc                                                            */
+    TP_EPI_ACCUMULATE = 1,    /* C += acc            (parameter .grad accumulation across slices)   */
+    TP_EPI_BIAS = 2,          /* C = acc + bias[n]   (ColumnParallelLinear, mpu/layers.py:256)      */
+    TP_EPI_BIAS_RELU = 3,     /* C = relu(acc + bias[n])   (fc1 + relu_, transformer_models.py:282) */
+    TP_EPI_BIAS_GELU = 4,     /* C = gelu_erf(acc + bias[n]); aux_out (if set) = acc + bias[n]      */
+    TP_EPI_BIAS_RESIDUAL = 5, /* C = acc + bias[n] + residual[m,n] (RowParallelLinear bias add
+                                 mpu/layers.py:346-347 + `x += y` transformer_models.py:277, :284)  */
+    TP_EPI_QKV_SCATTER = 6,   /* in_proj output split per head into q (scaled), k, v and written
+                                 straight to q[B*H,T,Dh] and rows [P, P+T) of the K/V caches
+                                 (transformer_models.py:217-219 and _AssignCache.forward :181-184)  */
+    TP_EPI_RELU_GRAD = 7,     /* C = acc * (aux[m,n] > 0)   backward of relu_ on its saved output   */
+    TP_EPI_GELU_GRAD = 8      /* C = acc * gelu_erf'(aux[m,n])   aux = saved pre-activation         */
+} tp_gemm_epilogue;
+
+typedef struct tp_gemm_desc {
+    int32_t op;       /* tp_gemm_op */
+    int32_t dtype;    /* tp_dtype of A, B, C, bias, residual, aux, q, caches */
+    int32_t epilogue; /* tp_gemm_epilogue */
+    int32_t M, N, K;
+    const void* A; int64_t lda;
+    const void* B; int64_t ldb;
+    void* C; int64_t ldc;               /* unused by TP_EPI_QKV_SCATTER */
+    const void* bias;                   /* [N] */
+    const void* residual; int64_t ldr;  /* [M, ldr] */
+    const void* aux; int64_t ldaux;     /* [M, ldaux] */
+    void* aux_out; int64_t ldauxo;      /* [M, ldauxo] */
+    float* colsum_acc;                  /* optional [N] fp32: += column sums of the values written to C
+                                           (bias gradient of the linear whose output gradient C is) */
+    /* TP_EPI_QKV_SCATTER: row m of C is (t, b) = (m / batch, m % batch); column n is
+       head n / (3*head_dim), then [q | k | v] inside the head. */
+    void* q; void* k_cache; void* v_cache;
+    int32_t batch, heads, head_dim, cache_len;
+    int64_t cache_rows;                 /* L_max: rows per (b,h) in the caches */
+    float q_scale;
+    int32_t reserved;
+} tp_gemm_desc;
+
+size_t tp_gemm_workspace_bytes(const tp_gemm_desc* d);
+int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Prefix-cached causal attention (attn_helper, transformer_models.py:235-245, with the mask of :220
+ * and :229 applied as an index comparison, and the gradient contract of _AssignCache.backward
+ * :186-190).  Query row t of the slice attends to cache rows [0, cache_len + t].
+ */
+typedef struct tp_attn_desc {
+    int32_t dtype;
+    int32_t batch, heads, head_dim;     /* head_dim must be 64 or 128 */
+    int32_t T;                          /* slice length */
+    int32_t cache_len;                  /* P: rows of the caches filled by earlier slices */
+    int64_t cache_rows;                 /* L_max */
+    const void* q;                      /* [B*H, T, Dh], already multiplied by Dh^-0.5 */
+    const void* k_cache;                /* [B*H, L_max, Dh]; rows [0, P+T) valid */
+    const void* v_cache;
+    void* o;                            /* [T, B, H*Dh]  (heads concatenated, transformer_models.py:244) */
+    float* lse;                         /* [B*H, T] log-sum-exp of the scaled, masked scores */
+    /* backward only */
+    const void* d_o;                    /* [T, B, H*Dh] */
+    float* delta;                       /* [B*H, T] scratch: rowsum(dO * O) */
+    void* dqkv;                         /* [T*B, 3*H*Dh] gradient of the in_proj output (per-head
+                                           [q|k|v] order); the q part includes the Dh^-0.5 factor */
+    void* dk_cache; void* dv_cache;     /* [B*H, L_max, Dh] gradient caches */
+    int32_t grad_cache_dtype;           /* tp_dtype of dk_cache/dv_cache: `dtype` or TP_F32 */
+    int32_t accumulate_prefix;          /* 1: rows [0,P) += dK, dV;  0: rows [0,P) = dK, dV */
+    int32_t has_incoming;               /* 1: rows [P,P+T) hold the gradient handed back by later
+                                           slices and are added to this slice's dK, dV */
+    int32_t zero_slice_rows;            /* 1: rows [P,P+T) are set to zero after being consumed
+                                           (grad_cache.data[index] = 0, transformer_models.py:189) */
+    float q_scale;
+    float* colsum_dqkv_acc;             /* optional [3*H*Dh] fp32: += column sums of dqkv (in_proj bias grad) */
+} tp_attn_desc;
+
+size_t tp_attn_fwd_workspace_bytes(const tp_attn_desc* d);
+int tp_attn_prefix_fwd(const tp_attn_desc* d, void* workspace, size_t workspace_bytes, void* stream);
+size_t tp_attn_bwd_workspace_bytes(const tp_attn_desc* d);
+int tp_attn_prefix_bwd(const tp_attn_desc* d, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Small helpers around the kernels above.
+ */
+/* dst[n] (dtype) = (accumulate ? dst[n] : 0) + src[n] (fp32): folds the fp32 accumulators of the
+ * LayerNorm / bias gradients into parameter .grad tensors (autograd's sum over slices). */
+int tp_accum_cast(void* dst, const float* src, int64_t n, int accumulate, int dtype, void* stream);
+/* acc[N] += column sums of x[M, N] (fp32 accumulators). */
+int tp_colsum_acc(const void* x, int64_t ldx, float* acc, int M, int N, int dtype, void* stream);
+/* fills n 32-bit words with zero (a kernel, so it can be recorded into a HIP graph) */
+int tp_zero_words(void* dst, int64_t n_words, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TERAPIPE_HIP_H_ */

@@ -1,0 +1,160 @@
+"""Functional core of one GPT layer over one sequence slice: the kernel sequence for forward and
+backward, shared by the autograd wrappers in transformer_models.py and by the sliced runner in
+terapipe.py.  Follows TransformerLayer.forward (transformer_models.py:273-285 of the reference) and
+MultiheadLMAttentionWithCache.forward (:214-255); every arithmetic step is a call into
+libterapipe_hip.so through terapipe_amd.ops.
+"""
+import torch
+
+from . import ops
+from ._lib import (TP_EPI_ACCUMULATE, TP_EPI_BIAS_GELU, TP_EPI_BIAS_RELU, TP_EPI_BIAS_RESIDUAL, TP_EPI_GELU_GRAD,
+                   TP_EPI_QKV_SCATTER, TP_EPI_RELU_GRAD, TP_EPI_STORE, TP_GEMM_NN, TP_GEMM_NT, TP_GEMM_TN)
+
+# order of the small (vector) parameters inside one layer's fp32 gradient accumulator
+SMALL_PARAMS = ("attn_ln.weight", "attn_ln.bias", "attn.in_proj.bias", "attn.out_proj.bias",
+                "fc_ln.weight", "fc_ln.bias", "fc1.bias", "fc2.bias")
+BIG_PARAMS = ("attn.in_proj.weight", "attn.out_proj.weight", "fc1.weight", "fc2.weight")
+PARAM_NAMES = ("attn_ln.weight", "attn_ln.bias", "attn.in_proj.weight", "attn.in_proj.bias",
+               "attn.out_proj.weight", "attn.out_proj.bias", "fc_ln.weight", "fc_ln.bias",
+               "fc1.weight", "fc1.bias", "fc2.weight", "fc2.bias")
+
+
+def small_param_sizes(E, F):
+    return {"attn_ln.weight": E, "attn_ln.bias": E, "attn.in_proj.bias": 3 * E, "attn.out_proj.bias": E,
+            "fc_ln.weight": E, "fc_ln.bias": E, "fc1.bias": F, "fc2.bias": E}
+
+
+def small_acc_views(buf, E, F):
+    """Splits a flat fp32 buffer of small_acc_numel(E, F) elements into per-parameter views."""
+    views, off = {}, 0
+    for name in SMALL_PARAMS:
+        n = small_param_sizes(E, F)[name]
+        views[name] = buf[off:off + n]
+        off += n
+    return views
+
+
+def small_acc_numel(E, F):
+    return sum(small_param_sizes(E, F).values())
+
+
+class SliceState:
+    """What one layer keeps from the forward of one slice for its backward."""
+    __slots__ = ("x", "mean1", "rstd1", "xn", "q", "o", "lse", "h", "mean2", "rstd2", "hn", "a", "z",
+                 "k_cache", "v_cache", "cache_len", "T", "B")
+
+
+def attention_fwd(w, xn2d, T, B, heads, k_cache, v_cache, cache_len):
+    """in_proj GEMM with the q/k/v split, q scaling and cache assignment fused into its epilogue, then
+    the prefix-cached attention kernel.  Returns q [B*H, T, Dh], o [T, B, E], lse."""
+    E = xn2d.shape[1]
+    Dh = E // heads
+    M = T * B
+    q = torch.empty(B * heads, T, Dh, dtype=xn2d.dtype, device=xn2d.device)
+    scale = float(Dh) ** -0.5
+    ops.gemm(TP_GEMM_NT, xn2d, w["attn.in_proj.weight"], M, 3 * E, E, epilogue=TP_EPI_QKV_SCATTER,
+             bias=w["attn.in_proj.bias"],
+             qkv=dict(q=q, k_cache=k_cache, v_cache=v_cache, batch=B, heads=heads, head_dim=Dh,
+                      cache_len=cache_len, cache_rows=k_cache.shape[1], q_scale=scale))
+    o, lse = ops.attn_prefix_fwd(q, k_cache, v_cache, B, heads, Dh, T, cache_len, scale)
+    return q, o, lse
+
+
+def layer_fwd(w, x, heads, k_cache, v_cache, cache_len, activation="relu", need_state=True):
+    """x [T, B, E] contiguous.  Writes rows [cache_len, cache_len+T) of the caches.  Returns (out, state)."""
+    T, B, E = x.shape
+    M = T * B
+    F = w["fc1.weight"].shape[0]
+    x2d = x.view(M, E)
+    xn, mean1, rstd1 = ops.layernorm_fwd(x2d, w["attn_ln.weight"], w["attn_ln.bias"])
+    q, o, lse = attention_fwd(w, xn, T, B, heads, k_cache, v_cache, cache_len)
+    o2d = o.view(M, E)
+    h = torch.empty_like(x2d)
+    ops.gemm(TP_GEMM_NT, o2d, w["attn.out_proj.weight"], M, E, E, C=h, epilogue=TP_EPI_BIAS_RESIDUAL,
+             bias=w["attn.out_proj.bias"], residual=x2d)
+    hn, mean2, rstd2 = ops.layernorm_fwd(h, w["fc_ln.weight"], w["fc_ln.bias"])
+    a = torch.empty(M, F, dtype=x.dtype, device=x.device)
+    z = None
+    if activation == "relu":
+        ops.gemm(TP_GEMM_NT, hn, w["fc1.weight"], M, F, E, C=a, epilogue=TP_EPI_BIAS_RELU, bias=w["fc1.bias"])
+    elif activation == "gelu":
+        z = torch.empty_like(a)
+        ops.gemm(TP_GEMM_NT, hn, w["fc1.weight"], M, F, E, C=a, epilogue=TP_EPI_BIAS_GELU, bias=w["fc1.bias"],
+                 aux_out=z)
+    else:
+        raise ValueError("activation must be 'relu' or 'gelu'")
+    out = torch.empty_like(x2d)
+    ops.gemm(TP_GEMM_NT, a, w["fc2.weight"], M, E, F, C=out, epilogue=TP_EPI_BIAS_RESIDUAL,
+             bias=w["fc2.bias"], residual=h)
+    st = None
+    if need_state:
+        st = SliceState()
+        st.x, st.mean1, st.rstd1, st.xn = x2d, mean1, rstd1, xn
+        st.q, st.o, st.lse = q, o2d, lse
+        st.h, st.mean2, st.rstd2, st.hn = h, mean2, rstd2, hn
+        st.a, st.z = a, z
+        st.k_cache, st.v_cache, st.cache_len, st.T, st.B = k_cache, v_cache, cache_len, T, B
+    return out.view(T, B, E), st
+
+
+def _wgrad(target, accumulate, A, Bm, M_, N_, K_):
+    """target[M_, N_] (+)= A[K_, M_]^T . Bm[K_, N_]"""
+    ops.gemm(TP_GEMM_TN, A, Bm, M_, N_, K_, C=target, epilogue=TP_EPI_ACCUMULATE if accumulate else TP_EPI_STORE)
+
+
+def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, accumulate_prefix, has_incoming,
+              zero_slice_rows, activation="relu", defer=None):
+    """Backward of layer_fwd for one slice.
+
+    dout [T, B, E]; gk / gv gradient caches (see tp_attn_desc); wgrad maps the four weight names to
+    gradient tensors that are overwritten (accumulate_wgrad False) or added to; small_acc maps the
+    vector parameter names to fp32 accumulators that are added to.  If `defer` is a dict, the four
+    weight-gradient GEMMs are not run; their operand pairs (dY, X) are stored in it instead so the
+    caller can run one GEMM over all slices.  Returns dx [T, B, E].
+    """
+    T, B = st.T, st.B
+    M = T * B
+    E = st.x.shape[1]
+    F = st.a.shape[1]
+    Dh = E // heads
+    dout2d = dout.reshape(M, E)
+    # MLP
+    dz1 = torch.empty(M, F, dtype=dout.dtype, device=dout.device)
+    if activation == "relu":
+        ops.gemm(TP_GEMM_NN, dout2d, w["fc2.weight"], M, F, E, C=dz1, epilogue=TP_EPI_RELU_GRAD, aux=st.a,
+                 colsum_acc=small_acc["fc1.bias"])
+    else:
+        ops.gemm(TP_GEMM_NN, dout2d, w["fc2.weight"], M, F, E, C=dz1, epilogue=TP_EPI_GELU_GRAD, aux=st.z,
+                 colsum_acc=small_acc["fc1.bias"])
+    if defer is None:
+        _wgrad(wgrad["fc2.weight"], accumulate_wgrad, dout2d, st.a, E, F, M)
+    else:
+        defer["fc2.weight"] = (dout2d, st.a)
+    dhn = torch.empty(M, E, dtype=dout.dtype, device=dout.device)
+    ops.gemm(TP_GEMM_NN, dz1, w["fc1.weight"], M, E, F, C=dhn)
+    if defer is None:
+        _wgrad(wgrad["fc1.weight"], accumulate_wgrad, dz1, st.hn, F, E, M)
+    else:
+        defer["fc1.weight"] = (dz1, st.hn)
+    dh = ops.layernorm_bwd(dhn, st.h, st.mean2, st.rstd2, w["fc_ln.weight"], dout2d, small_acc["fc_ln.weight"],
+                           small_acc["fc_ln.bias"], small_acc["fc2.bias"], small_acc["attn.out_proj.bias"])
+    # attention
+    d_o = torch.empty(M, E, dtype=dout.dtype, device=dout.device)
+    ops.gemm(TP_GEMM_NN, dh, w["attn.out_proj.weight"], M, E, E, C=d_o)
+    if defer is None:
+        _wgrad(wgrad["attn.out_proj.weight"], accumulate_wgrad, dh, st.o, E, E, M)
+    else:
+        defer["attn.out_proj.weight"] = (dh, st.o)
+    dqkv = torch.empty(M, 3 * E, dtype=dout.dtype, device=dout.device)
+    ops.attn_prefix_bwd(st.q, st.k_cache, st.v_cache, st.o, st.lse, d_o, dqkv, gk, gv, B, heads, Dh, T,
+                        st.cache_len, float(Dh) ** -0.5, accumulate_prefix, has_incoming, zero_slice_rows,
+                        colsum_dqkv_acc=small_acc["attn.in_proj.bias"])
+    dxn = torch.empty(M, E, dtype=dout.dtype, device=dout.device)
+    ops.gemm(TP_GEMM_NN, dqkv, w["attn.in_proj.weight"], M, E, 3 * E, C=dxn)
+    if defer is None:
+        _wgrad(wgrad["attn.in_proj.weight"], accumulate_wgrad, dqkv, st.xn, 3 * E, E, M)
+    else:
+        defer["attn.in_proj.weight"] = (dqkv, st.xn)
+    dx = ops.layernorm_bwd(dxn, st.x, st.mean1, st.rstd1, w["attn_ln.weight"], dh, small_acc["attn_ln.weight"],
+                           small_acc["attn_ln.bias"], None, None)
+    return dx.view(T, B, E)

@@ -1,0 +1,641 @@
+// Prefix-cached causal attention for one sequence slice: forward (online softmax, optional split over
+// the key range) and backward (recompute from Q, K, LSE; dK/dV accumulated into the gradient caches).
+//
+// Register layouts.  All products are 32x32 MFMA blocks.  The forward and the dQ kernel compute the
+// TRANSPOSED score block S^T = K Q^T, so a lane owns one query (column lane & 31) and 16 keys: the
+// softmax row reductions are in-lane plus one exchange with lane ^ 32, and eight accumulator registers
+// are, unshuffled, the operand of the following product (P^T or dS^T) once V^T / K^T are fetched from
+// LDS in the interleaved row order (fetch_tr<..., true>).  The dK/dV kernel computes S = Q K^T so that a
+// lane owns one key and 16 queries, which makes P and dS the operands of dV^T = dO^T P and
+// dK^T = Q^T dS in the same way.
+#include "common.h"
+
+namespace tp {
+
+struct AttnArgs {
+    const void* q; const void* kc; const void* vc; void* o; float* lse;
+    const void* d_o; float* delta; void* dqkv; void* gk; void* gv;
+    int B, H, T, P;
+    long cache_rows;
+    int nsplit;
+    float* part_o; float* part_lse;
+    int accumulate_prefix, has_incoming, zero_slice_rows;
+    float qscale;
+};
+
+static constexpr float kLog2e = 1.4426950408889634f;
+
+template <typename T, int DH>
+__device__ __forceinline__ void load_row_operands(typename Elem<T>::opnd_t* reg, const T* rowptr, bool valid, int g) {
+    typedef Elem<T> E;
+    constexpr int NKS = DH / E::KSTEP;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+        if constexpr (sizeof(T) == 2) {
+            reg[ks] = valid ? *reinterpret_cast<const uint4*>(rowptr + ks * 16 + 8 * g) : make_uint4(0, 0, 0, 0);
+        } else {
+            reg[ks] = valid ? rowptr[ks * 2 + g] : 0.f;
+        }
+    }
+}
+
+// acc[db] += X^T-block (rows db*32.. of the tile's columns, k over tile rows krow_base..+31) times the
+// 32x32 accumulator `p` used as the k x n operand.
+template <typename T, int DH>
+__device__ __forceinline__ void mfma_acc_as_b(float16v* acc, const T* tile, int krow_base, const float16v& p, int lane) {
+    typedef Elem<T> E;
+    typedef TileLayout<T, DH> L;
+    constexpr int NDB = DH / 32;
+    const int g = lane >> 5, li = lane & 31;
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            float tmp[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) tmp[e] = p[8 * s + e];
+            uint4 bop = pack8<T>(tmp);
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) {
+                uint4 aop = fetch_tr<T, DH, true>(tile, krow_base + 16 * s, db * 32, lane);
+                acc[db] = E::mfma(aop, bop, acc[db]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            float bop = p[j];
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) {
+                float aop = tile[L::off(krow_base + acc_row(j, g), db * 32 + li)];
+                acc[db] = E::mfma(aop, bop, acc[db]);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// forward
+// ------------------------------------------------------------------------------------------------
+template <typename T, int DH, int NW, int BN>
+__global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs a) {
+    typedef Elem<T> E;
+    typedef TileLayout<T, DH> L;
+    constexpr int NT = NW * 64, NKB = BN / 32, NDB = DH / 32, NKS = DH / E::KSTEP;
+    __shared__ __attribute__((aligned(16))) T sK[L::size(BN)];
+    __shared__ __attribute__((aligned(16))) T sV[L::size(BN)];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, li = lane & 31;
+    const int bh = blockIdx.y, b = bh / a.H, h = bh - b * a.H;
+    const int T_ = a.T, P = a.P, S = a.P + a.T;
+    const int q0w = (blockIdx.x * NW + wave) * 32;
+    const int tq = q0w + li;
+    const int q_wg_end = min(T_, (int)(blockIdx.x + 1) * NW * 32);
+    const int kv_end = P + q_wg_end;
+    const int ntiles = (kv_end + BN - 1) / BN;
+    const int tps = (ntiles + a.nsplit - 1) / a.nsplit;
+    const int t_beg = blockIdx.z * tps, t_end = min(ntiles, t_beg + tps);
+
+    typename E::opnd_t qreg[NKS];
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * T_ + tq) * DH, tq < T_, g);
+
+    float16v oacc[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+    float m = -INFINITY, lsum = 0.f;
+
+    const T* Kb = reinterpret_cast<const T*>(a.kc) + (long)bh * a.cache_rows * DH;
+    const T* Vb = reinterpret_cast<const T*>(a.vc) + (long)bh * a.cache_rows * DH;
+    TileCopy<T, BN, DH, NT> ck, cv;
+    if (t_beg < t_end) {
+        ck.load(Kb, DH, t_beg * BN, 0, S, DH, tid);
+        cv.load(Vb, DH, t_beg * BN, 0, S, DH, tid);
+        ck.store(sK, tid);
+        cv.store(sV, tid);
+    }
+    __syncthreads();
+    for (int t = t_beg; t < t_end; ++t) {
+        if (t + 1 < t_end) {
+            ck.load(Kb, DH, (t + 1) * BN, 0, S, DH, tid);
+            cv.load(Vb, DH, (t + 1) * BN, 0, S, DH, tid);
+        }
+        const int key0 = t * BN;
+        if (q0w < T_ && key0 <= P + q0w + 31) {
+            float16v sacc[NKB];
+#pragma unroll
+            for (int kb = 0; kb < NKB; ++kb) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < NKS; ++ks) {
+                    typename E::opnd_t kop = fetch_km<T, DH>(sK, kb * 32 + li, ks * E::KSTEP, lane);
+                    sacc[kb] = E::mfma(kop, qreg[ks], sacc[kb]);
+                }
+            }
+            float mt = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    int key = key0 + kb * 32 + acc_row(j, g);
+                    float s = key > P + tq ? -INFINITY : sacc[kb][j];
+                    sacc[kb][j] = s;
+                    mt = fmaxf(mt, s);
+                }
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float m_new = fmaxf(m, mt);
+            const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = exp2f((m - m_safe) * kLog2e);
+            float psum = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    float p = exp2f((sacc[kb][j] - m_safe) * kLog2e);
+                    sacc[kb][j] = p;
+                    psum += p;
+                }
+            lsum = lsum * alpha + psum;
+            m = m_new;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+#pragma unroll
+            for (int kb = 0; kb < NKB; ++kb) mfma_acc_as_b<T, DH>(oacc, sV, kb * 32, sacc[kb], lane);
+        }
+        __syncthreads();
+        if (t + 1 < t_end) {
+            ck.store(sK, tid);
+            cv.store(sV, tid);
+        }
+        __syncthreads();
+    }
+
+    const float ltot = lsum + __shfl_xor(lsum, 32, 64);
+    if (tq < T_) {
+        const float inv = ltot > 0.f ? 1.0f / ltot : 0.f;
+        const float lse = ltot > 0.f ? m + logf(ltot) : -INFINITY;
+        if (a.nsplit == 1) {
+            T* O = reinterpret_cast<T*>(a.o) + ((long)tq * a.B + b) * ((long)a.H * DH) + (long)h * DH;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int jq = 0; jq < 4; ++jq) {
+                    int dh = db * 32 + 8 * jq + 4 * g;
+                    store4<T>(O + dh, oacc[db][4 * jq] * inv, oacc[db][4 * jq + 1] * inv,
+                              oacc[db][4 * jq + 2] * inv, oacc[db][4 * jq + 3] * inv);
+                }
+            if (g == 0) a.lse[(long)bh * T_ + tq] = lse;
+        } else {
+            const long BH = (long)a.B * a.H;
+            float* PO = a.part_o + (((long)blockIdx.z * BH + bh) * T_ + tq) * DH;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int jq = 0; jq < 4; ++jq) {
+                    int dh = db * 32 + 8 * jq + 4 * g;
+                    *reinterpret_cast<float4*>(PO + dh) =
+                        make_float4(oacc[db][4 * jq] * inv, oacc[db][4 * jq + 1] * inv,
+                                    oacc[db][4 * jq + 2] * inv, oacc[db][4 * jq + 3] * inv);
+                }
+            if (g == 0) a.part_lse[((long)blockIdx.z * BH + bh) * T_ + tq] = lse;
+        }
+    }
+}
+
+// merges the per-split partial outputs: one wave per (bh, t) row
+template <typename T, int DH>
+__global__ __launch_bounds__(256) void attn_fwd_merge_kernel(AttnArgs a) {
+    const long BH = (long)a.B * a.H;
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= BH * a.T) return;
+    const int bh = (int)(row / a.T), t = (int)(row - (long)bh * a.T);
+    const int b = bh / a.H, h = bh - b * a.H;
+    float mx = -INFINITY;
+    for (int z = 0; z < a.nsplit; ++z) mx = fmaxf(mx, a.part_lse[(long)z * BH * a.T + row]);
+    float wsum = 0.f;
+    float acc[DH / 64];
+#pragma unroll
+    for (int i = 0; i < DH / 64; ++i) acc[i] = 0.f;
+    for (int z = 0; z < a.nsplit; ++z) {
+        float l = a.part_lse[(long)z * BH * a.T + row];
+        float w = l == -INFINITY ? 0.f : exp2f((l - mx) * kLog2e);
+        wsum += w;
+        const float* PO = a.part_o + ((long)z * BH * a.T + row) * DH;
+#pragma unroll
+        for (int i = 0; i < DH / 64; ++i) acc[i] += w * PO[lane + 64 * i];
+    }
+    T* O = reinterpret_cast<T*>(a.o) + ((long)t * a.B + b) * ((long)a.H * DH) + (long)h * DH;
+    const float inv = 1.0f / wsum;
+#pragma unroll
+    for (int i = 0; i < DH / 64; ++i) O[lane + 64 * i] = Elem<T>::from_float(acc[i] * inv);
+    if (lane == 0) a.lse[row] = mx + logf(wsum);
+}
+
+// ------------------------------------------------------------------------------------------------
+// backward
+// ------------------------------------------------------------------------------------------------
+// delta[bh][t] = sum_d dO * O, one wave per (t, b, h)
+template <typename T, int DH>
+__global__ __launch_bounds__(256) void attn_bwd_delta_kernel(AttnArgs a) {
+    const long n = (long)a.T * a.B * a.H;
+    const long idx = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (idx >= n) return;
+    const int h = (int)(idx % a.H);
+    const long m = idx / a.H;  // row t*B + b
+    const int b = (int)(m % a.B), t = (int)(m / a.B);
+    const long off = m * ((long)a.H * DH) + (long)h * DH;
+    const T* O = reinterpret_cast<const T*>(a.o) + off;
+    const T* dO = reinterpret_cast<const T*>(a.d_o) + off;
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < DH / 64; ++i)
+        s += Elem<T>::to_float(O[lane + 64 * i]) * Elem<T>::to_float(dO[lane + 64 * i]);
+    s = wave_sum(s);
+    if (lane == 0) a.delta[((long)b * a.H + h) * a.T + t] = s;
+}
+
+// dK / dV: each wave owns 32 keys and walks over the query blocks that can see them.
+template <typename T, typename GT, int DH, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_kernel(AttnArgs a) {
+    typedef Elem<T> E;
+    typedef TileLayout<T, DH> L;
+    constexpr int NT = NW * 64, NDB = DH / 32, NKS = DH / E::KSTEP;
+    __shared__ __attribute__((aligned(16))) T sQ[L::size(32)];
+    __shared__ __attribute__((aligned(16))) T sdO[L::size(32)];
+    __shared__ __attribute__((aligned(16))) float sLse[32];
+    __shared__ __attribute__((aligned(16))) float sDelta[32];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, li = lane & 31;
+    const int bh = blockIdx.y, b = bh / a.H, h = bh - b * a.H;
+    const int T_ = a.T, P = a.P, S = a.P + a.T;
+    const long EE = (long)a.H * DH;
+    const int key0wg = blockIdx.x * NW * 32;
+    const int key0w = key0wg + wave * 32;
+    const int key = key0w + li;
+
+    typename E::opnd_t kreg[NKS], vreg[NKS];
+    load_row_operands<T, DH>(kreg, reinterpret_cast<const T*>(a.kc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
+    load_row_operands<T, DH>(vreg, reinterpret_cast<const T*>(a.vc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
+
+    float16v dk[NDB], dv[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
+
+    const T* Qb = reinterpret_cast<const T*>(a.q) + (long)bh * T_ * DH;
+    const T* dOb = reinterpret_cast<const T*>(a.d_o) + (long)b * EE + (long)h * DH;  // row t at stride B*E
+    const int nqb = (T_ + 31) / 32;
+    const int qb_start = key0wg > P ? (key0wg - P) / 32 : 0;
+    TileCopy<T, 32, DH, NT> cq, cdo;
+    for (int qb = qb_start; qb < nqb; ++qb) {
+        cq.load(Qb, DH, qb * 32, 0, T_, DH, tid);
+        cdo.load(dOb, (long)a.B * EE, qb * 32, 0, T_, DH, tid);
+        __syncthreads();  // previous iteration's readers are done
+        cq.store(sQ, tid);
+        cdo.store(sdO, tid);
+        if (tid < 32) {
+            int t = qb * 32 + tid;
+            sLse[tid] = t < T_ ? a.lse[(long)bh * T_ + t] : 0.f;
+            sDelta[tid] = t < T_ ? a.delta[(long)bh * T_ + t] : 0.f;
+        }
+        __syncthreads();
+        if (key0w < S && key0w <= P + qb * 32 + 31) {
+            float16v sacc, pacc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                typename E::opnd_t qop = fetch_km<T, DH>(sQ, li, ks * E::KSTEP, lane);
+                sacc = E::mfma(qop, kreg[ks], sacc);
+                typename E::opnd_t doop = fetch_km<T, DH>(sdO, li, ks * E::KSTEP, lane);
+                pacc = E::mfma(doop, vreg[ks], pacc);
+            }
+#pragma unroll
+            for (int jq = 0; jq < 4; ++jq) {
+                float4 l4 = *reinterpret_cast<const float4*>(sLse + 8 * jq + 4 * g);
+                float4 d4 = *reinterpret_cast<const float4*>(sDelta + 8 * jq + 4 * g);
+                const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+                const float dl[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    int j = 4 * jq + e;
+                    int t = qb * 32 + 8 * jq + 4 * g + e;
+                    bool vis = (t < T_) && (key <= P + t) && (key < S);
+                    float p = vis ? exp2f((sacc[j] - lv[e]) * kLog2e) : 0.f;
+                    float ds = p * (pacc[j] - dl[e]);
+                    sacc[j] = p;
+                    pacc[j] = ds;
+                }
+            }
+            mfma_acc_as_b<T, DH>(dv, sdO, 0, sacc, lane);
+            mfma_acc_as_b<T, DH>(dk, sQ, 0, pacc, lane);
+        }
+    }
+
+    if (key < S) {
+        GT* gK = reinterpret_cast<GT*>(a.gk) + ((long)bh * a.cache_rows + key) * DH;
+        GT* gV = reinterpret_cast<GT*>(a.gv) + ((long)bh * a.cache_rows + key) * DH;
+        if (key < P) {
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int jq = 0; jq < 4; ++jq) {
+                    int dh = db * 32 + 8 * jq + 4 * g;
+                    float ok[4] = {0.f, 0.f, 0.f, 0.f}, ov[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (a.accumulate_prefix) { load4<GT>(gK + dh, ok); load4<GT>(gV + dh, ov); }
+                    store4<GT>(gK + dh, ok[0] + dk[db][4 * jq], ok[1] + dk[db][4 * jq + 1],
+                               ok[2] + dk[db][4 * jq + 2], ok[3] + dk[db][4 * jq + 3]);
+                    store4<GT>(gV + dh, ov[0] + dv[db][4 * jq], ov[1] + dv[db][4 * jq + 1],
+                               ov[2] + dv[db][4 * jq + 2], ov[3] + dv[db][4 * jq + 3]);
+                }
+        } else {
+            const int t = key - P;
+            T* dst = reinterpret_cast<T*>(a.dqkv) + ((long)t * a.B + b) * (3 * EE) + (long)h * 3 * DH;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int jq = 0; jq < 4; ++jq) {
+                    int dh = db * 32 + 8 * jq + 4 * g;
+                    float ok[4] = {0.f, 0.f, 0.f, 0.f}, ov[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (a.has_incoming) { load4<GT>(gK + dh, ok); load4<GT>(gV + dh, ov); }
+                    store4<T>(dst + DH + dh, ok[0] + dk[db][4 * jq], ok[1] + dk[db][4 * jq + 1],
+                              ok[2] + dk[db][4 * jq + 2], ok[3] + dk[db][4 * jq + 3]);
+                    store4<T>(dst + 2 * DH + dh, ov[0] + dv[db][4 * jq], ov[1] + dv[db][4 * jq + 1],
+                              ov[2] + dv[db][4 * jq + 2], ov[3] + dv[db][4 * jq + 3]);
+                    if (a.zero_slice_rows) {
+                        store4<GT>(gK + dh, 0.f, 0.f, 0.f, 0.f);
+                        store4<GT>(gV + dh, 0.f, 0.f, 0.f, 0.f);
+                    }
+                }
+        }
+    }
+}
+
+// dQ: each wave owns 32 queries and walks over the key tiles they can see.
+template <typename T, int DH, int NW, int BN>
+__global__ __launch_bounds__(NW * 64) void attn_bwd_dq_kernel(AttnArgs a) {
+    typedef Elem<T> E;
+    typedef TileLayout<T, DH> L;
+    constexpr int NT = NW * 64, NKB = BN / 32, NDB = DH / 32, NKS = DH / E::KSTEP;
+    __shared__ __attribute__((aligned(16))) T sK[L::size(BN)];
+    __shared__ __attribute__((aligned(16))) T sV[L::size(BN)];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, li = lane & 31;
+    const int bh = blockIdx.y, b = bh / a.H, h = bh - b * a.H;
+    const int T_ = a.T, P = a.P, S = a.P + a.T;
+    const long EE = (long)a.H * DH;
+    const int q0w = (blockIdx.x * NW + wave) * 32;
+    const int tq = q0w + li;
+    const int q_wg_end = min(T_, (int)(blockIdx.x + 1) * NW * 32);
+    const int kv_end = P + q_wg_end;
+    const int ntiles = (kv_end + BN - 1) / BN;
+
+    typename E::opnd_t qreg[NKS], doreg[NKS];
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * T_ + tq) * DH, tq < T_, g);
+    load_row_operands<T, DH>(doreg, reinterpret_cast<const T*>(a.d_o) + ((long)tq * a.B + b) * EE + (long)h * DH, tq < T_, g);
+    const float lse_q = tq < T_ ? a.lse[(long)bh * T_ + tq] : 0.f;
+    const float delta_q = tq < T_ ? a.delta[(long)bh * T_ + tq] : 0.f;
+
+    float16v dq[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
+
+    const T* Kb = reinterpret_cast<const T*>(a.kc) + (long)bh * a.cache_rows * DH;
+    const T* Vb = reinterpret_cast<const T*>(a.vc) + (long)bh * a.cache_rows * DH;
+    TileCopy<T, BN, DH, NT> ck, cv;
+    if (ntiles > 0) {
+        ck.load(Kb, DH, 0, 0, S, DH, tid);
+        cv.load(Vb, DH, 0, 0, S, DH, tid);
+        ck.store(sK, tid);
+        cv.store(sV, tid);
+    }
+    __syncthreads();
+    for (int t = 0; t < ntiles; ++t) {
+        if (t + 1 < ntiles) {
+            ck.load(Kb, DH, (t + 1) * BN, 0, S, DH, tid);
+            cv.load(Vb, DH, (t + 1) * BN, 0, S, DH, tid);
+        }
+        const int key0 = t * BN;
+        if (q0w < T_ && key0 <= P + q0w + 31) {
+#pragma unroll
+            for (int kb = 0; kb < NKB; ++kb) {
+                float16v sacc, pacc;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+                for (int ks = 0; ks < NKS; ++ks) {
+                    typename E::opnd_t kop = fetch_km<T, DH>(sK, kb * 32 + li, ks * E::KSTEP, lane);
+                    sacc = E::mfma(kop, qreg[ks], sacc);
+                    typename E::opnd_t vop = fetch_km<T, DH>(sV, kb * 32 + li, ks * E::KSTEP, lane);
+                    pacc = E::mfma(vop, doreg[ks], pacc);
+                }
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    int key = key0 + kb * 32 + acc_row(j, g);
+                    float p = key > P + tq ? 0.f : exp2f((sacc[j] - lse_q) * kLog2e);
+                    pacc[j] = p * (pacc[j] - delta_q);
+                }
+                mfma_acc_as_b<T, DH>(dq, sK, kb * 32, pacc, lane);
+            }
+        }
+        __syncthreads();
+        if (t + 1 < ntiles) {
+            ck.store(sK, tid);
+            cv.store(sV, tid);
+        }
+        __syncthreads();
+    }
+    if (tq < T_) {
+        T* dst = reinterpret_cast<T*>(a.dqkv) + ((long)tq * a.B + b) * (3 * EE) + (long)h * 3 * DH;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int jq = 0; jq < 4; ++jq) {
+                int dh = db * 32 + 8 * jq + 4 * g;
+                store4<T>(dst + dh, dq[db][4 * jq] * a.qscale, dq[db][4 * jq + 1] * a.qscale,
+                          dq[db][4 * jq + 2] * a.qscale, dq[db][4 * jq + 3] * a.qscale);
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+static constexpr int kNumCU = 256;
+
+static int validate_attn(const tp_attn_desc* d, bool bwd) {
+    const char* who = bwd ? "tp_attn_prefix_bwd" : "tp_attn_prefix_fwd";
+    if (!d) { set_error("%s: null descriptor", who); return TP_ERR_ARG; }
+    if (d->dtype < TP_F32 || d->dtype > TP_BF16) { set_error("%s: bad dtype %d", who, d->dtype); return TP_ERR_ARG; }
+    if (d->head_dim != 64 && d->head_dim != 128) { set_error("%s: head_dim %d not supported (64 or 128)", who, d->head_dim); return TP_ERR_UNSUPPORTED; }
+    if (d->batch <= 0 || d->heads <= 0 || d->T <= 0 || d->cache_len < 0) { set_error("%s: bad geometry B=%d H=%d T=%d P=%d", who, d->batch, d->heads, d->T, d->cache_len); return TP_ERR_ARG; }
+    if ((long)d->cache_len + d->T > d->cache_rows) { set_error("%s: slice [%d, %d) does not fit a cache of %ld rows", who, d->cache_len, d->cache_len + d->T, (long)d->cache_rows); return TP_ERR_ARG; }
+    if (!d->q || !d->k_cache || !d->v_cache || !d->o || !d->lse) { set_error("%s: null tensor", who); return TP_ERR_ARG; }
+    if (((uintptr_t)d->q | (uintptr_t)d->k_cache | (uintptr_t)d->v_cache | (uintptr_t)d->o) & 15) { set_error("%s: tensors must be 16-byte aligned", who); return TP_ERR_ARG; }
+    if (bwd) {
+        if (!d->d_o || !d->delta || !d->dqkv) { set_error("%s: null gradient tensor", who); return TP_ERR_ARG; }
+        if (((uintptr_t)d->d_o | (uintptr_t)d->dqkv | (uintptr_t)d->dk_cache | (uintptr_t)d->dv_cache) & 15) { set_error("%s: tensors must be 16-byte aligned", who); return TP_ERR_ARG; }
+        if ((d->cache_len > 0 || d->has_incoming || d->zero_slice_rows) && (!d->dk_cache || !d->dv_cache)) { set_error("%s: gradient caches required", who); return TP_ERR_ARG; }
+        if (d->grad_cache_dtype != d->dtype && d->grad_cache_dtype != TP_F32) { set_error("%s: grad_cache_dtype must be dtype or fp32", who); return TP_ERR_ARG; }
+    }
+    return TP_OK;
+}
+
+struct FwdPlan { int nw, bn, nsplit, qblocks; };
+
+static FwdPlan plan_fwd(const tp_attn_desc* d) {
+    FwdPlan p;
+    p.nw = d->T > 64 ? 4 : (d->T > 32 ? 2 : 1);
+    p.bn = p.nw == 1 ? 32 : 64;
+    p.qblocks = (d->T + 32 * p.nw - 1) / (32 * p.nw);
+    long waves = (long)p.qblocks * d->batch * d->heads * p.nw;
+    int ntiles_min = (d->cache_len + (d->T < 32 * p.nw ? d->T : 32 * p.nw) + p.bn - 1) / p.bn;  // first q block
+    int ns = 1;
+    if (waves < 4L * kNumCU) {
+        ns = (int)((4L * kNumCU + waves - 1) / waves);
+        int cap = ntiles_min / 2;  // at least two tiles per split
+        if (ns > cap) ns = cap;
+        if (ns > 32) ns = 32;
+        if (ns < 1) ns = 1;
+    }
+    p.nsplit = ns;
+    return p;
+}
+
+static AttnArgs make_args(const tp_attn_desc* d) {
+    AttnArgs a;
+    a.q = d->q; a.kc = d->k_cache; a.vc = d->v_cache; a.o = d->o; a.lse = d->lse;
+    a.d_o = d->d_o; a.delta = d->delta; a.dqkv = d->dqkv; a.gk = d->dk_cache; a.gv = d->dv_cache;
+    a.B = d->batch; a.H = d->heads; a.T = d->T; a.P = d->cache_len; a.cache_rows = d->cache_rows;
+    a.nsplit = 1; a.part_o = nullptr; a.part_lse = nullptr;
+    a.accumulate_prefix = d->accumulate_prefix; a.has_incoming = d->has_incoming;
+    a.zero_slice_rows = d->zero_slice_rows; a.qscale = d->q_scale;
+    return a;
+}
+
+template <typename T, int DH>
+static void launch_fwd(const FwdPlan& p, const AttnArgs& a, hipStream_t s) {
+    dim3 grid(p.qblocks, a.B * a.H, p.nsplit);
+    if (p.nw == 4) attn_fwd_kernel<T, DH, 4, 64><<<grid, 256, 0, s>>>(a);
+    else if (p.nw == 2) attn_fwd_kernel<T, DH, 2, 64><<<grid, 128, 0, s>>>(a);
+    else attn_fwd_kernel<T, DH, 1, 32><<<grid, 64, 0, s>>>(a);
+    if (p.nsplit > 1) {
+        long rows = (long)a.B * a.H * a.T;
+        attn_fwd_merge_kernel<T, DH><<<(unsigned)((rows + 3) / 4), 256, 0, s>>>(a);
+    }
+}
+
+template <typename T, typename GT, int DH>
+static void launch_bwd(const AttnArgs& a, hipStream_t s) {
+    const int S = a.P + a.T;
+    long rows = (long)a.T * a.B * a.H;
+    attn_bwd_delta_kernel<T, DH><<<(unsigned)((rows + 3) / 4), 256, 0, s>>>(a);
+    {
+        // dK/dV: 4 waves x 32 keys per workgroup when that still fills the chip, else 2 or 1
+        long bh = (long)a.B * a.H;
+        int nw = 4;
+        if (((S + 127) / 128) * bh < 2L * kNumCU) nw = 2;
+        if (((S + 63) / 64) * bh < 2L * kNumCU) nw = 1;
+        dim3 grid((S + 32 * nw - 1) / (32 * nw), (unsigned)bh);
+        if (nw == 4) attn_bwd_dkdv_kernel<T, GT, DH, 4><<<grid, 256, 0, s>>>(a);
+        else if (nw == 2) attn_bwd_dkdv_kernel<T, GT, DH, 2><<<grid, 128, 0, s>>>(a);
+        else attn_bwd_dkdv_kernel<T, GT, DH, 1><<<grid, 64, 0, s>>>(a);
+    }
+    {
+        int nw = a.T > 64 ? 4 : (a.T > 32 ? 2 : 1);
+        dim3 grid((a.T + 32 * nw - 1) / (32 * nw), a.B * a.H);
+        if (nw == 4) attn_bwd_dq_kernel<T, DH, 4, 64><<<grid, 256, 0, s>>>(a);
+        else if (nw == 2) attn_bwd_dq_kernel<T, DH, 2, 64><<<grid, 128, 0, s>>>(a);
+        else attn_bwd_dq_kernel<T, DH, 1, 32><<<grid, 64, 0, s>>>(a);
+    }
+}
+
+template <typename T>
+static void dispatch_fwd(int hd, const FwdPlan& p, const AttnArgs& a, hipStream_t s) {
+    if (hd == 64) launch_fwd<T, 64>(p, a, s);
+    else launch_fwd<T, 128>(p, a, s);
+}
+
+template <typename T>
+static void dispatch_bwd(int hd, bool f32grad, const AttnArgs& a, hipStream_t s) {
+    if constexpr (sizeof(T) == 4) {
+        if (hd == 64) launch_bwd<T, float, 64>(a, s);
+        else launch_bwd<T, float, 128>(a, s);
+    } else {
+        if (f32grad) {
+            if (hd == 64) launch_bwd<T, float, 64>(a, s);
+            else launch_bwd<T, float, 128>(a, s);
+        } else {
+            if (hd == 64) launch_bwd<T, T, 64>(a, s);
+            else launch_bwd<T, T, 128>(a, s);
+        }
+    }
+}
+
+}  // namespace tp
+
+extern "C" size_t tp_attn_fwd_workspace_bytes(const tp_attn_desc* d) {
+    if (!d || d->T <= 0 || d->batch <= 0 || d->heads <= 0) return 0;
+    tp::FwdPlan p = tp::plan_fwd(d);
+    if (p.nsplit <= 1) return 0;
+    size_t rows = (size_t)p.nsplit * d->batch * d->heads * d->T;
+    return rows * d->head_dim * sizeof(float) + rows * sizeof(float);
+}
+
+extern "C" int tp_attn_prefix_fwd(const tp_attn_desc* d, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace tp;
+    int rc = validate_attn(d, false);
+    if (rc != TP_OK) return rc;
+    FwdPlan p = plan_fwd(d);
+    AttnArgs a = make_args(d);
+    if (p.nsplit > 1) {
+        size_t need = tp_attn_fwd_workspace_bytes(d);
+        if (!workspace || workspace_bytes < need) { set_error("tp_attn_prefix_fwd: workspace of %zu bytes needed, %zu given", need, workspace_bytes); return TP_ERR_WORKSPACE; }
+        if ((uintptr_t)workspace & 15) { set_error("tp_attn_prefix_fwd: workspace must be 16-byte aligned"); return TP_ERR_ARG; }
+        size_t rows = (size_t)p.nsplit * d->batch * d->heads * d->T;
+        a.nsplit = p.nsplit;
+        a.part_o = reinterpret_cast<float*>(workspace);
+        a.part_lse = a.part_o + rows * d->head_dim;
+    }
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    switch (d->dtype) {
+    case TP_F32: dispatch_fwd<float>(d->head_dim, p, a, s); break;
+    case TP_F16: dispatch_fwd<f16>(d->head_dim, p, a, s); break;
+    default: dispatch_fwd<bf16>(d->head_dim, p, a, s); break;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("tp_attn_prefix_fwd: launch failed: %s", hipGetErrorString(e)); return TP_ERR_LAUNCH; }
+    return TP_OK;
+}
+
+extern "C" size_t tp_attn_bwd_workspace_bytes(const tp_attn_desc* d) { (void)d; return 0; }
+
+extern "C" int tp_attn_prefix_bwd(const tp_attn_desc* d, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace tp;
+    (void)workspace; (void)workspace_bytes;
+    int rc = validate_attn(d, true);
+    if (rc != TP_OK) return rc;
+    AttnArgs a = make_args(d);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const bool f32grad = d->grad_cache_dtype == TP_F32;
+    switch (d->dtype) {
+    case TP_F32: dispatch_bwd<float>(d->head_dim, true, a, s); break;
+    case TP_F16: dispatch_bwd<f16>(d->head_dim, f32grad, a, s); break;
+    default: dispatch_bwd<bf16>(d->head_dim, f32grad, a, s); break;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("tp_attn_prefix_bwd: launch failed: %s", hipGetErrorString(e)); return TP_ERR_LAUNCH; }
+    if (d->colsum_dqkv_acc) {
+        return tp_colsum_acc(d->dqkv, 3L * d->heads * d->head_dim, d->colsum_dqkv_acc, d->T * d->batch,
+                             3 * d->heads * d->head_dim, d->dtype, stream);
+    }
+    return TP_OK;
+}

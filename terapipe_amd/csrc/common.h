@@ -1,0 +1,214 @@
+// Shared device helpers for the gfx950 (CDNA4, wave64) kernels of the sliced GPT-layer path.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/terapipe_hip.h"
+
+namespace tp {
+
+typedef _Float16 f16;
+typedef __bf16 bf16;
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+#define TP_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+// ---------------------------------------------------------------------------------------------
+// Element traits.  KP = k-values one lane feeds to one 32x32 MFMA; KSTEP = k covered by one MFMA.
+// 16-bit types use v_mfma_f32_32x32x16_{f16,bf16}: lane l holds row/col (l & 31) and the 8
+// consecutive k values 8 * (l >> 5) ... + 7.  fp32 uses v_mfma_f32_32x32x2_f32: lane l holds
+// row/col (l & 31) and k = (l >> 5).  The 32x32 fp32 accumulator is 16 registers per lane:
+// acc[j] is row 8 * (j / 4) + 4 * (l >> 5) + (j % 4), column (l & 31).
+// ---------------------------------------------------------------------------------------------
+template <typename T> struct Elem;
+
+template <> struct Elem<f16> {
+    static constexpr int KP = 8, KSTEP = 16, CH = 8;
+    typedef uint4 opnd_t;
+    static __device__ __forceinline__ float16v mfma(opnd_t a, opnd_t b, float16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a),
+                                                     __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_float(f16 x) { return (float)x; }
+    static __device__ __forceinline__ f16 from_float(float x) { return (f16)x; }
+};
+
+template <> struct Elem<bf16> {
+    static constexpr int KP = 8, KSTEP = 16, CH = 8;
+    typedef uint4 opnd_t;
+    static __device__ __forceinline__ float16v mfma(opnd_t a, opnd_t b, float16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                      __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_float(bf16 x) { return (float)x; }
+    static __device__ __forceinline__ bf16 from_float(float x) { return (bf16)x; }
+};
+
+template <> struct Elem<float> {
+    static constexpr int KP = 1, KSTEP = 2, CH = 4;
+    typedef float opnd_t;
+    static __device__ __forceinline__ float16v mfma(opnd_t a, opnd_t b, float16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_float(float x) { return x; }
+    static __device__ __forceinline__ float from_float(float x) { return x; }
+};
+
+// Row of accumulator register j for the lane's k-group g = lane >> 5.
+__device__ __forceinline__ int acc_row(int j, int g) { return 8 * (j >> 2) + 4 * g + (j & 3); }
+
+// ---------------------------------------------------------------------------------------------
+// LDS tiles.  A tile is ROWS x COLS elements, COLS contiguous, exactly as it lies in global memory.
+// 16-bit tiles are XOR-swizzled at 16-byte chunk granularity so that both access patterns used by
+// the MFMA operand fetches are free of avoidable bank conflicts:
+//   (a) "k-major" fetch: 16 consecutive rows, the same 16-byte chunk (ds_read_b128), and
+//   (b) "transposed" fetch: ds_read_b64_tr_b16 over 4 consecutive rows x 64 bytes.
+// fp32 tiles are padded by 4 floats per row instead.
+// ---------------------------------------------------------------------------------------------
+template <int COLS> __device__ __forceinline__ int swz16(int row) {
+    // returns the chunk XOR mask for a 16-bit tile with COLS elements per row
+    if constexpr (COLS >= 128) {
+        return ((row & 3) << 2) | ((row >> 2) & 3);
+    } else if constexpr (COLS == 64) {
+        return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+    } else if constexpr (COLS == 32) {
+        return (row >> 2) & 3;
+    } else {
+        return 0;
+    }
+}
+
+template <typename T, int COLS> struct TileLayout {
+    static constexpr bool kSwz = (sizeof(T) == 2);
+    static constexpr int LD = kSwz ? COLS : COLS + 4;   // row pitch in elements
+    // element offset of (row, col); for swizzled tiles col's 8-element chunk index is permuted
+    static __device__ __forceinline__ int off(int row, int col) {
+        if constexpr (kSwz) {
+            return row * LD + ((((col >> 3) ^ swz16<COLS>(row)) << 3) | (col & 7));
+        } else {
+            return row * LD + col;
+        }
+    }
+    static constexpr int size(int rows) { return rows * LD; }
+};
+
+// Cooperative global -> register -> LDS copy of a ROWS x COLS tile by NT threads, 16 bytes a chunk.
+// Chunks wholly outside [0, rmax) x [0, cmax) are zero-filled (cmax and the leading dimension must be
+// multiples of the chunk length, which the host checks).
+template <typename T, int ROWS, int COLS, int NT> struct TileCopy {
+    static constexpr int CH = 16 / sizeof(T);
+    static constexpr int CPR = COLS / CH;
+    static constexpr int TOTAL = ROWS * CPR;
+    static constexpr int N = (TOTAL + NT - 1) / NT;
+    uint4 r[N];
+
+    __device__ __forceinline__ void load(const T* __restrict__ base, long ld, int r0, int c0, int rmax,
+                                         int cmax, int tid) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            int c = tid + i * NT;
+            int row = c / CPR, cc = c % CPR;
+            int gr = r0 + row, gc = c0 + cc * CH;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if ((TOTAL % NT == 0 || c < TOTAL) && gr < rmax && gc < cmax)
+                v = *reinterpret_cast<const uint4*>(base + (long)gr * ld + gc);
+            r[i] = v;
+        }
+    }
+    __device__ __forceinline__ void store(T* lds, int tid) const {
+        typedef TileLayout<T, COLS> L;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            int c = tid + i * NT;
+            int row = c / CPR, cc = c % CPR;
+            if (TOTAL % NT == 0 || c < TOTAL)
+                *reinterpret_cast<uint4*>(lds + L::off(row, cc * CH)) = r[i];
+        }
+    }
+};
+
+// MFMA operand fetches from an LDS tile.
+//   fetch_km: operand whose k runs along the tile's columns.  `row` is the lane's own row
+//             (tile-relative, already including lane & 31); k0 the first column of this k-step.
+//   fetch_tr: operand whose k runs along the tile's rows (two ds_read_b64_tr_b16 per operand).
+//             `col0` is the first of the 32 columns of the MFMA block.  Natural order: k-slot e of lane
+//             group g is row krow0 + 8 * g + e, the same k the k-major fetch gives that slot.
+//             Interleaved order: slot e of group g is row krow0 + 8 * (e / 4) + 4 * g + (e % 4), the
+//             order in which a 32x32 accumulator lays rows over registers, so that eight accumulator
+//             registers of another MFMA can be fed back as the matching operand without a shuffle.
+//             For fp32 (natural only) the single k-slot of group g is row krow0 + g.
+template <typename T, int COLS>
+__device__ __forceinline__ typename Elem<T>::opnd_t fetch_km(const T* tile, int row, int k0, int lane) {
+    typedef TileLayout<T, COLS> L;
+    int g = lane >> 5;
+    if constexpr (sizeof(T) == 2) {
+        return *reinterpret_cast<const uint4*>(tile + L::off(row, k0 + 8 * g));
+    } else {
+        return tile[L::off(row, k0 + g)];
+    }
+}
+
+template <typename T, int COLS, bool INTERLEAVED>
+__device__ __forceinline__ typename Elem<T>::opnd_t fetch_tr(const T* tile, int krow0, int col0, int lane) {
+    typedef TileLayout<T, COLS> L;
+    int g = lane >> 5;
+    if constexpr (sizeof(T) == 2) {
+        int p = lane & 15;
+        int col = col0 + 16 * ((lane & 31) >> 4) + 4 * (p & 3);
+        int r0 = krow0 + (INTERLEAVED ? 4 * g : 8 * g) + (p >> 2);
+        int r1 = r0 + (INTERLEAVED ? 8 : 4);
+        short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TP_LDS_PTR(short4v, tile + L::off(r0, col)));
+        short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TP_LDS_PTR(short4v, tile + L::off(r1, col)));
+        uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+        return make_uint4(l2.x, l2.y, h2.x, h2.y);
+    } else {
+        static_assert(!INTERLEAVED || sizeof(T) == 2, "fp32 interleaved fetches address rows directly");
+        return tile[L::off(krow0 + g, col0 + (lane & 31))];
+    }
+}
+
+// Pack 8 fp32 accumulator values (registers j0 .. j0+7 of a 32x32 block) into one 16-bit MFMA operand.
+template <typename T>
+__device__ __forceinline__ uint4 pack8(const float* v) {
+    T h[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) h[e] = Elem<T>::from_float(v[e]);
+    return *reinterpret_cast<uint4*>(h);
+}
+
+template <typename T> __device__ __forceinline__ void store4(T* dst, float a, float b, float c, float d) {
+    if constexpr (sizeof(T) == 2) {
+        T h[4] = {Elem<T>::from_float(a), Elem<T>::from_float(b), Elem<T>::from_float(c), Elem<T>::from_float(d)};
+        *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<uint2*>(h);
+    } else {
+        *reinterpret_cast<float4*>(dst) = make_float4(a, b, c, d);
+    }
+}
+
+template <typename T> __device__ __forceinline__ void load4(const T* src, float* out) {
+    if constexpr (sizeof(T) == 2) {
+        uint2 raw = *reinterpret_cast<const uint2*>(src);
+        const T* h = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[e] = Elem<T>::to_float(h[e]);
+    } else {
+        float4 v = *reinterpret_cast<const float4*>(src);
+        out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+    }
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// error plumbing shared by the host-side entry points
+void set_error(const char* fmt, ...);
+
+}  // namespace tp

@@ -1,0 +1,261 @@
+// Fused LayerNorm forward / backward: one workgroup per row, the row cached in registers, 16-byte
+// coalesced accesses, fp32 statistics, wave64 shuffle + LDS block reductions.
+#include "common.h"
+
+namespace tp {
+
+template <int NREDUCE>
+__device__ __forceinline__ void block_sum(float (&v)[NREDUCE], float* scratch /* [NREDUCE][16] */) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+#pragma unroll
+    for (int i = 0; i < NREDUCE; ++i) v[i] = wave_sum(v[i]);
+    __syncthreads();  // scratch may still be read by the previous reduction
+    if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < NREDUCE; ++i) scratch[i * 16 + wave] = v[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NREDUCE; ++i) {
+        float s = 0.f;
+        for (int w = 0; w < nw; ++w) s += scratch[i * 16 + w];
+        v[i] = s;
+    }
+}
+
+template <typename T> __device__ __forceinline__ void load_chunk(const T* p, float* out) {
+    constexpr int CH = 16 / sizeof(T);
+    uint4 raw = *reinterpret_cast<const uint4*>(p);
+    if constexpr (sizeof(T) == 2) {
+        const T* h = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+        for (int e = 0; e < CH; ++e) out[e] = Elem<T>::to_float(h[e]);
+    } else {
+        const float* f = reinterpret_cast<const float*>(&raw);
+#pragma unroll
+        for (int e = 0; e < CH; ++e) out[e] = f[e];
+    }
+}
+
+template <typename T> __device__ __forceinline__ void store_chunk(T* p, const float* v) {
+    constexpr int CH = 16 / sizeof(T);
+    uint4 raw;
+    if constexpr (sizeof(T) == 2) {
+        T* h = reinterpret_cast<T*>(&raw);
+#pragma unroll
+        for (int e = 0; e < CH; ++e) h[e] = Elem<T>::from_float(v[e]);
+    } else {
+        float* f = reinterpret_cast<float*>(&raw);
+#pragma unroll
+        for (int e = 0; e < CH; ++e) f[e] = v[e];
+    }
+    *reinterpret_cast<uint4*>(p) = raw;
+}
+
+template <typename T, int MAXC>
+__global__ __launch_bounds__(1024) void ln_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
+                                                      const T* __restrict__ beta, T* __restrict__ y,
+                                                      float* __restrict__ mean, float* __restrict__ rstd,
+                                                      int M, int E, float eps) {
+    constexpr int CH = 16 / sizeof(T);
+    __shared__ float scratch[16];
+    const int row = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
+    const int nch = E / CH;
+    const T* xr = x + (long)row * E;
+    float v[MAXC][CH];
+    float s[1] = {0.f};
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        int c = tid + i * nt;
+        if (c < nch) {
+            load_chunk<T>(xr + (long)c * CH, v[i]);
+#pragma unroll
+            for (int e = 0; e < CH; ++e) s[0] += v[i][e];
+        }
+    }
+    block_sum<1>(s, scratch);
+    const float mu = s[0] / (float)E;
+    float q[1] = {0.f};
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        int c = tid + i * nt;
+        if (c < nch) {
+#pragma unroll
+            for (int e = 0; e < CH; ++e) { float d = v[i][e] - mu; q[0] += d * d; }
+        }
+    }
+    block_sum<1>(q, scratch);
+    const float rs = 1.0f / sqrtf(q[0] / (float)E + eps);
+    if (tid == 0) { mean[row] = mu; rstd[row] = rs; }
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        int c = tid + i * nt;
+        if (c < nch) {
+            float gm[CH], bt[CH], o[CH];
+            load_chunk<T>(gamma + (long)c * CH, gm);
+            load_chunk<T>(beta + (long)c * CH, bt);
+#pragma unroll
+            for (int e = 0; e < CH; ++e) o[e] = (v[i][e] - mu) * rs * gm[e] + bt[e];
+            store_chunk<T>(y + (long)row * E + (long)c * CH, o);
+        }
+    }
+}
+
+template <typename T, int MAXC>
+__global__ __launch_bounds__(1024) void ln_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                                      const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                      const T* __restrict__ gamma, const T* __restrict__ dres,
+                                                      T* __restrict__ dx, float* dgamma, float* dbeta,
+                                                      float* cs_dres, float* cs_dx, int M, int E) {
+    constexpr int CH = 16 / sizeof(T);
+    __shared__ float scratch[32];
+    const int tid = threadIdx.x, nt = blockDim.x;
+    const int nch = E / CH;
+    float gm[MAXC][CH], a_dg[MAXC][CH], a_db[MAXC][CH], a_dr[MAXC][CH], a_dx[MAXC][CH];
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        int c = tid + i * nt;
+        if (c < nch) load_chunk<T>(gamma + (long)c * CH, gm[i]);
+#pragma unroll
+        for (int e = 0; e < CH; ++e) { a_dg[i][e] = 0.f; a_db[i][e] = 0.f; a_dr[i][e] = 0.f; a_dx[i][e] = 0.f; }
+    }
+    for (int row = blockIdx.x; row < M; row += gridDim.x) {
+        const float mu = mean[row], rs = rstd[row];
+        float g[MAXC][CH], xh[MAXC][CH];
+        float s[2] = {0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+            int c = tid + i * nt;
+            if (c < nch) {
+                float d[CH], xv[CH];
+                load_chunk<T>(dy + (long)row * E + (long)c * CH, d);
+                load_chunk<T>(x + (long)row * E + (long)c * CH, xv);
+#pragma unroll
+                for (int e = 0; e < CH; ++e) {
+                    xh[i][e] = (xv[e] - mu) * rs;
+                    g[i][e] = d[e] * gm[i][e];
+                    s[0] += g[i][e];
+                    s[1] += g[i][e] * xh[i][e];
+                    a_dg[i][e] += d[e] * xh[i][e];
+                    a_db[i][e] += d[e];
+                }
+            }
+        }
+        block_sum<2>(s, scratch);
+        const float m1 = s[0] / (float)E, m2 = s[1] / (float)E;
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+            int c = tid + i * nt;
+            if (c < nch) {
+                float o[CH];
+#pragma unroll
+                for (int e = 0; e < CH; ++e) o[e] = rs * (g[i][e] - m1 - xh[i][e] * m2);
+                if (dres) {
+                    float r[CH];
+                    load_chunk<T>(dres + (long)row * E + (long)c * CH, r);
+#pragma unroll
+                    for (int e = 0; e < CH; ++e) { o[e] += r[e]; a_dr[i][e] += r[e]; }
+                }
+#pragma unroll
+                for (int e = 0; e < CH; ++e) a_dx[i][e] += o[e];
+                store_chunk<T>(dx + (long)row * E + (long)c * CH, o);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        int c = tid + i * nt;
+        if (c < nch) {
+#pragma unroll
+            for (int e = 0; e < CH; ++e) {
+                long col = (long)c * CH + e;
+                atomicAdd(dgamma + col, a_dg[i][e]);
+                atomicAdd(dbeta + col, a_db[i][e]);
+                if (cs_dres && dres) atomicAdd(cs_dres + col, a_dr[i][e]);
+                if (cs_dx) atomicAdd(cs_dx + col, a_dx[i][e]);
+            }
+        }
+    }
+}
+
+static int ln_geometry(int E, int dtype, int* threads, int* maxc) {
+    const int ch = dtype == TP_F32 ? 4 : 8;
+    if (E <= 0 || E % ch) { set_error("layernorm: E=%d must be a positive multiple of %d", E, ch); return TP_ERR_UNSUPPORTED; }
+    const int nch = E / ch;
+    int nt = 64;
+    while (nt < nch && nt < 1024) nt *= 2;
+    int mc = (nch + nt - 1) / nt;
+    if (mc > 4) { set_error("layernorm: E=%d too large (max %d)", E, 1024 * 4 * ch); return TP_ERR_UNSUPPORTED; }
+    *threads = nt;
+    *maxc = mc <= 1 ? 1 : (mc <= 2 ? 2 : 4);
+    return TP_OK;
+}
+
+template <typename T>
+static void launch_ln_fwd(int maxc, int nt, const void* x, const void* gamma, const void* beta, void* y,
+                          float* mean, float* rstd, int M, int E, float eps, hipStream_t s) {
+    const T* xp = (const T*)x; const T* gp = (const T*)gamma; const T* bp = (const T*)beta; T* yp = (T*)y;
+    if (maxc == 1) ln_fwd_kernel<T, 1><<<M, nt, 0, s>>>(xp, gp, bp, yp, mean, rstd, M, E, eps);
+    else if (maxc == 2) ln_fwd_kernel<T, 2><<<M, nt, 0, s>>>(xp, gp, bp, yp, mean, rstd, M, E, eps);
+    else ln_fwd_kernel<T, 4><<<M, nt, 0, s>>>(xp, gp, bp, yp, mean, rstd, M, E, eps);
+}
+
+template <typename T>
+static void launch_ln_bwd(int maxc, int nt, int grid, const void* dy, const void* x, const float* mean,
+                          const float* rstd, const void* gamma, const void* dres, void* dx, float* dg,
+                          float* db, float* cr, float* cx, int M, int E, hipStream_t s) {
+    const T* dyp = (const T*)dy; const T* xp = (const T*)x; const T* gp = (const T*)gamma;
+    const T* rp = (const T*)dres; T* dxp = (T*)dx;
+    if (maxc == 1) ln_bwd_kernel<T, 1><<<grid, nt, 0, s>>>(dyp, xp, mean, rstd, gp, rp, dxp, dg, db, cr, cx, M, E);
+    else if (maxc == 2) ln_bwd_kernel<T, 2><<<grid, nt, 0, s>>>(dyp, xp, mean, rstd, gp, rp, dxp, dg, db, cr, cx, M, E);
+    else ln_bwd_kernel<T, 4><<<grid, nt, 0, s>>>(dyp, xp, mean, rstd, gp, rp, dxp, dg, db, cr, cx, M, E);
+}
+
+static int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("%s: launch failed: %s", what, hipGetErrorString(e)); return TP_ERR_LAUNCH; }
+    return TP_OK;
+}
+
+}  // namespace tp
+
+extern "C" int tp_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
+                                float* rstd, int M, int E, float eps, int dtype, void* stream) {
+    using namespace tp;
+    if (!x || !gamma || !beta || !y || !mean || !rstd) { set_error("tp_layernorm_fwd: null pointer"); return TP_ERR_ARG; }
+    if (M <= 0) { set_error("tp_layernorm_fwd: M=%d", M); return TP_ERR_ARG; }
+    if (dtype < TP_F32 || dtype > TP_BF16) { set_error("tp_layernorm_fwd: bad dtype %d", dtype); return TP_ERR_ARG; }
+    if (((uintptr_t)x | (uintptr_t)gamma | (uintptr_t)beta | (uintptr_t)y) & 15) { set_error("tp_layernorm_fwd: pointers must be 16-byte aligned"); return TP_ERR_ARG; }
+    int nt, maxc;
+    int rc = ln_geometry(E, dtype, &nt, &maxc);
+    if (rc != TP_OK) return rc;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    switch (dtype) {
+    case TP_F32: launch_ln_fwd<float>(maxc, nt, x, gamma, beta, y, mean, rstd, M, E, eps, s); break;
+    case TP_F16: launch_ln_fwd<f16>(maxc, nt, x, gamma, beta, y, mean, rstd, M, E, eps, s); break;
+    default: launch_ln_fwd<bf16>(maxc, nt, x, gamma, beta, y, mean, rstd, M, E, eps, s); break;
+    }
+    return check_launch("tp_layernorm_fwd");
+}
+
+extern "C" int tp_layernorm_bwd(const void* dy, const void* x, const float* mean, const float* rstd,
+                                const void* gamma, const void* dres, void* dx, float* dgamma_acc,
+                                float* dbeta_acc, float* colsum_dres_acc, float* colsum_dx_acc, int M, int E,
+                                int dtype, void* stream) {
+    using namespace tp;
+    if (!dy || !x || !mean || !rstd || !gamma || !dx || !dgamma_acc || !dbeta_acc) { set_error("tp_layernorm_bwd: null pointer"); return TP_ERR_ARG; }
+    if (M <= 0) { set_error("tp_layernorm_bwd: M=%d", M); return TP_ERR_ARG; }
+    if (dtype < TP_F32 || dtype > TP_BF16) { set_error("tp_layernorm_bwd: bad dtype %d", dtype); return TP_ERR_ARG; }
+    if (((uintptr_t)dy | (uintptr_t)x | (uintptr_t)gamma | (uintptr_t)dres | (uintptr_t)dx) & 15) { set_error("tp_layernorm_bwd: pointers must be 16-byte aligned"); return TP_ERR_ARG; }
+    int nt, maxc;
+    int rc = ln_geometry(E, dtype, &nt, &maxc);
+    if (rc != TP_OK) return rc;
+    int grid = M < 128 ? M : 128;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    switch (dtype) {
+    case TP_F32: launch_ln_bwd<float>(maxc, nt, grid, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc, M, E, s); break;
+    case TP_F16: launch_ln_bwd<f16>(maxc, nt, grid, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc, M, E, s); break;
+    default: launch_ln_bwd<bf16>(maxc, nt, grid, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc, M, E, s); break;
+    }
+    return check_launch("tp_layernorm_bwd");
+}

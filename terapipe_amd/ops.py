@@ -1,0 +1,173 @@
+"""Thin torch-tensor wrappers over the C ABI (include/terapipe_hip.h).
+
+PyTorch owns all device memory and the stream; these functions only pass ``data_ptr()``s, shapes and
+``torch.cuda.current_stream()`` to the library.  Nothing here computes on the host and nothing falls
+back to PyTorch kernels: a missing library or a non-zero status raises.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import (AttnDesc, GemmDesc, TP_BF16, TP_F16, TP_F32, TP_GEMM_NN, TP_GEMM_NT, TP_GEMM_TN,
+                   TP_EPI_ACCUMULATE, TP_EPI_BIAS, TP_EPI_BIAS_GELU, TP_EPI_BIAS_RELU, TP_EPI_BIAS_RESIDUAL,
+                   TP_EPI_GELU_GRAD, TP_EPI_QKV_SCATTER, TP_EPI_RELU_GRAD, TP_EPI_STORE)
+
+_DTYPES = {torch.float32: TP_F32, torch.float16: TP_F16, torch.bfloat16: TP_BF16}
+
+
+def tp_dtype(dtype):
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise TypeError("unsupported dtype %s (float32, float16, bfloat16)" % dtype)
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def _require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise _lib.TeraPipeHipError("terapipe_amd kernels need CUDA/HIP tensors; there is no CPU path")
+
+
+class Workspace:
+    """A grow-only scratch tensor per device (torch-owned), handed to calls that need workspace."""
+    _bufs = {}
+
+    @classmethod
+    def get(cls, nbytes, device):
+        key = (device.type, device.index)
+        buf = cls._bufs.get(key)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+            cls._bufs[key] = buf
+        return buf
+
+
+def layernorm_fwd(x2d, gamma, beta, eps=1e-5):
+    _require_cuda(x2d, gamma, beta)
+    M, E = x2d.shape
+    y = torch.empty_like(x2d)
+    mean = torch.empty(M, dtype=torch.float32, device=x2d.device)
+    rstd = torch.empty(M, dtype=torch.float32, device=x2d.device)
+    lib = _lib.load()
+    _lib.check(lib.tp_layernorm_fwd(_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps,
+                                    tp_dtype(x2d.dtype), _stream()), "tp_layernorm_fwd")
+    return y, mean, rstd
+
+
+def layernorm_bwd(dy, x2d, mean, rstd, gamma, dres, dgamma_acc, dbeta_acc, colsum_dres_acc=None,
+                  colsum_dx_acc=None):
+    _require_cuda(dy, x2d, gamma)
+    M, E = x2d.shape
+    dx = torch.empty_like(x2d)
+    lib = _lib.load()
+    _lib.check(lib.tp_layernorm_bwd(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx),
+                                    _p(dgamma_acc), _p(dbeta_acc), _p(colsum_dres_acc), _p(colsum_dx_acc),
+                                    M, E, tp_dtype(x2d.dtype), _stream()), "tp_layernorm_bwd")
+    return dx
+
+
+def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=None, aux=None, aux_out=None,
+         colsum_acc=None, qkv=None):
+    """Runs one GEMM.  A, B, C, residual, aux are 2-D row-major tensors (stride(1) == 1).
+    qkv = dict(q, k_cache, v_cache, batch, heads, head_dim, cache_len, cache_rows, q_scale)."""
+    _require_cuda(A, B, C)
+    d = GemmDesc()
+    d.op, d.dtype, d.epilogue = op, tp_dtype(A.dtype), epilogue
+    d.M, d.N, d.K = M, N, K
+    d.A, d.lda = A.data_ptr(), A.stride(0)
+    d.B, d.ldb = B.data_ptr(), B.stride(0)
+    if C is not None:
+        d.C, d.ldc = C.data_ptr(), C.stride(0)
+    d.bias = _p(bias)
+    if residual is not None:
+        d.residual, d.ldr = residual.data_ptr(), residual.stride(0)
+    if aux is not None:
+        d.aux, d.ldaux = aux.data_ptr(), aux.stride(0)
+    if aux_out is not None:
+        d.aux_out, d.ldauxo = aux_out.data_ptr(), aux_out.stride(0)
+    d.colsum_acc = _p(colsum_acc)
+    if qkv is not None:
+        d.q, d.k_cache, d.v_cache = qkv["q"].data_ptr(), qkv["k_cache"].data_ptr(), qkv["v_cache"].data_ptr()
+        d.batch, d.heads, d.head_dim = qkv["batch"], qkv["heads"], qkv["head_dim"]
+        d.cache_len, d.cache_rows, d.q_scale = qkv["cache_len"], qkv["cache_rows"], qkv["q_scale"]
+    lib = _lib.load()
+    need = lib.tp_gemm_workspace_bytes(ctypes.byref(d))
+    ws = Workspace.get(need, A.device) if need else None
+    _lib.check(lib.tp_gemm(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()), "tp_gemm")
+    return C
+
+
+def _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale):
+    d = AttnDesc()
+    d.dtype = tp_dtype(q.dtype)
+    d.batch, d.heads, d.head_dim, d.T, d.cache_len = batch, heads, head_dim, T, cache_len
+    d.cache_rows = k_cache.shape[1]
+    d.q, d.k_cache, d.v_cache, d.o, d.lse = q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), o.data_ptr(), lse.data_ptr()
+    d.q_scale = q_scale
+    return d
+
+
+def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q_scale):
+    """q [B*H, T, Dh] (pre-scaled); caches [B*H, L, Dh] with rows [0, cache_len+T) valid.
+    Returns o [T, B, H*Dh] and lse [B*H, T]."""
+    _require_cuda(q, k_cache, v_cache)
+    o = torch.empty(T, batch, heads * head_dim, dtype=q.dtype, device=q.device)
+    lse = torch.empty(batch * heads, T, dtype=torch.float32, device=q.device)
+    d = _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale)
+    lib = _lib.load()
+    need = lib.tp_attn_fwd_workspace_bytes(ctypes.byref(d))
+    ws = Workspace.get(need, q.device) if need else None
+    _lib.check(lib.tp_attn_prefix_fwd(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()),
+               "tp_attn_prefix_fwd")
+    return o, lse
+
+
+def attn_prefix_bwd(q, k_cache, v_cache, o, lse, d_o, dqkv, dk_cache, dv_cache, batch, heads, head_dim, T,
+                    cache_len, q_scale, accumulate_prefix, has_incoming, zero_slice_rows, colsum_dqkv_acc=None):
+    """Writes dqkv [T*B, 3*H*Dh]; updates rows [0, cache_len) of the gradient caches."""
+    _require_cuda(q, k_cache, v_cache, d_o, dqkv)
+    delta = torch.empty(batch * heads, T, dtype=torch.float32, device=q.device)
+    d = _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale)
+    d.d_o, d.delta, d.dqkv = d_o.data_ptr(), delta.data_ptr(), dqkv.data_ptr()
+    d.dk_cache, d.dv_cache = _p(dk_cache), _p(dv_cache)
+    d.grad_cache_dtype = tp_dtype(dk_cache.dtype) if dk_cache is not None else d.dtype
+    d.accumulate_prefix, d.has_incoming, d.zero_slice_rows = int(accumulate_prefix), int(has_incoming), int(zero_slice_rows)
+    d.colsum_dqkv_acc = _p(colsum_dqkv_acc)
+    lib = _lib.load()
+    _lib.check(lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()), "tp_attn_prefix_bwd")
+    return dqkv
+
+
+def accum_cast(dst, src_f32, accumulate):
+    _require_cuda(dst, src_f32)
+    lib = _lib.load()
+    _lib.check(lib.tp_accum_cast(_p(dst), _p(src_f32), dst.numel(), int(accumulate), tp_dtype(dst.dtype), _stream()),
+               "tp_accum_cast")
+    return dst
+
+
+def colsum_acc(x2d, acc_f32):
+    _require_cuda(x2d, acc_f32)
+    lib = _lib.load()
+    _lib.check(lib.tp_colsum_acc(_p(x2d), x2d.stride(0), _p(acc_f32), x2d.shape[0], x2d.shape[1],
+                                 tp_dtype(x2d.dtype), _stream()), "tp_colsum_acc")
+    return acc_f32
+
+
+def zero_(t):
+    """Zero-fills a contiguous tensor whose byte size is a multiple of 4 with the library's fill kernel."""
+    _require_cuda(t)
+    nbytes = t.numel() * t.element_size()
+    assert t.is_contiguous() and nbytes % 4 == 0
+    lib = _lib.load()
+    _lib.check(lib.tp_zero_words(_p(t), nbytes // 4, _stream()), "tp_zero_words")
+    return t

@@ -1,0 +1,259 @@
+"""Kernel-level parity: each C-ABI entry point against a plain fp32/fp64 PyTorch statement of the
+same op on the same seeded inputs.  Tolerances: max rel err (relative to max|ref| of the tensor)
+<= 1e-5 for fp32, <= 2e-2 for fp16/bf16 (inputs are pre-rounded to the kernel dtype so the tolerance
+measures kernel error only)."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from tests.util import TOL, assert_close, rel_err
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+DEV = "cuda:0"
+
+
+def _ops():
+    from terapipe_amd import ops
+    return ops
+
+
+def _rnd(shape, dtype, gen, scale=1.0):
+    return (torch.randn(*shape, generator=gen) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("M,E", [(32, 256), (7, 64), (256, 2048), (160, 5120), (33, 12288)])
+def test_layernorm_fwd_bwd(dtype, M, E):
+    ops = _ops()
+    if dtype == torch.float32 and E > 8192 * 2:
+        pytest.skip("fp32 rows above 16384 elements are outside the kernel's register cache")
+    g = torch.Generator().manual_seed(M * 131 + E)
+    x = _rnd((M, E), dtype, g) + 0.3
+    gamma = (1 + 0.2 * torch.randn(E, generator=g)).to(dtype)
+    beta = _rnd((E,), dtype, g, 0.1)
+    dy = _rnd((M, E), dtype, g)
+    dres = _rnd((M, E), dtype, g)
+    xd, gd, bd, dyd, dresd = [t.to(DEV) for t in (x, gamma, beta, dy, dres)]
+    y, mean, rstd = ops.layernorm_fwd(xd, gd, bd)
+    x64 = x.double().requires_grad_(True)
+    g64, b64 = gamma.double().requires_grad_(True), beta.double().requires_grad_(True)
+    yref = F.layer_norm(x64, (E,), g64, b64, 1e-5)
+    assert_close(y, yref, dtype, "ln y")
+    assert_close(mean, x64.mean(-1), torch.float32, "ln mean", 10)
+    yref.backward(dy.double())
+    acc = torch.zeros(4, E, dtype=torch.float32, device=DEV)
+    dx = ops.layernorm_bwd(dyd, xd, mean, rstd, gd, dresd, acc[0], acc[1], acc[2], acc[3])
+    dx_ref = x64.grad + dres.double()
+    assert_close(dx, dx_ref, dtype, "ln dx")
+    # accumulators are fp32 sums of products of dtype-rounded inputs
+    assert_close(acc[0], g64.grad, torch.float32, "ln dgamma", 20)
+    assert_close(acc[1], b64.grad, torch.float32, "ln dbeta", 20)
+    assert_close(acc[2], dres.double().sum(0), torch.float32, "colsum dres", 20)
+    assert_close(acc[3], dx_ref.sum(0), dtype, "colsum dx", 1)
+    # without the residual input
+    acc.zero_()
+    dx2 = ops.layernorm_bwd(dyd, xd, mean, rstd, gd, None, acc[0], acc[1], None, None)
+    assert_close(dx2, x64.grad, dtype, "ln dx (no dres)")
+
+
+GEMM_SHAPES = [
+    # M, N, K
+    (32, 256, 256),     # C1 out_proj
+    (32, 768, 256),     # C1 in_proj
+    (32, 256, 1024),    # C1 fc2
+    (256, 2048, 2048),  # C2 out_proj (split-K)
+    (160, 5120, 5120),  # C3 last slice
+    (512, 15360, 5120),  # C3 in_proj, large-tile config
+    (70, 136, 200),     # ragged everything
+    (1, 8, 8),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_nt_nn_tn(dtype, M, N, K):
+    ops = _ops()
+    from terapipe_amd._lib import TP_GEMM_NN, TP_GEMM_NT, TP_GEMM_TN, TP_EPI_ACCUMULATE
+    if dtype == torch.float32 and M * N * K > 256 * 2048 * 2048:
+        pytest.skip("large shapes are covered in 16-bit")
+    g = torch.Generator().manual_seed(M + 7 * N + 13 * K)
+    sc = 1.0 / math.sqrt(K)
+    # NT: C[M,N] = A[M,K] B[N,K]^T
+    A, B = _rnd((M, K), dtype, g), _rnd((N, K), dtype, g, sc)
+    C = torch.empty(M, N, dtype=dtype, device=DEV)
+    ops.gemm(TP_GEMM_NT, A.to(DEV), B.to(DEV), M, N, K, C=C)
+    assert_close(C, A.double() @ B.double().t(), dtype, "NT")
+    # NN: C[M,N] = A[M,K] B[K,N]
+    if N % 8 == 0:
+        B2 = _rnd((K, N), dtype, g, sc)
+        ops.gemm(TP_GEMM_NN, A.to(DEV), B2.to(DEV), M, N, K, C=C)
+        assert_close(C, A.double() @ B2.double(), dtype, "NN")
+    # TN: C[M2,N2] = A[K2,M2]^T B[K2,N2] with K2 = M (tokens), M2 = N, N2 = K: the weight-gradient shape
+    if K % 8 == 0 and N % 8 == 0:
+        dY, X = _rnd((M, N), dtype, g), _rnd((M, K), dtype, g, 1.0 / math.sqrt(M))
+        W = torch.empty(N, K, dtype=dtype, device=DEV)
+        ops.gemm(TP_GEMM_TN, dY.to(DEV), X.to(DEV), N, K, M, C=W)
+        ref = dY.double().t() @ X.double()
+        assert_close(W, ref, dtype, "TN")
+        ops.gemm(TP_GEMM_TN, dY.to(DEV), X.to(DEV), N, K, M, C=W, epilogue=TP_EPI_ACCUMULATE)
+        assert_close(W, 2 * ref, dtype, "TN accumulate")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("M,N,K", [(32, 1024, 256), (256, 8192, 2048), (48, 264, 136)])
+def test_gemm_epilogues(dtype, M, N, K):
+    ops = _ops()
+    from terapipe_amd import _lib as L
+    g = torch.Generator().manual_seed(5 * M + N + K)
+    sc = 1.0 / math.sqrt(K)
+    A, B = _rnd((M, K), dtype, g), _rnd((N, K), dtype, g, sc)
+    bias, R = _rnd((N,), dtype, g, 0.5), _rnd((M, N), dtype, g)
+    Ad, Bd, bd, Rd = A.to(DEV), B.to(DEV), bias.to(DEV), R.to(DEV)
+    base = A.double() @ B.double().t() + bias.double()
+    C = torch.empty(M, N, dtype=dtype, device=DEV)
+    ops.gemm(L.TP_GEMM_NT, Ad, Bd, M, N, K, C=C, epilogue=L.TP_EPI_BIAS, bias=bd)
+    assert_close(C, base, dtype, "bias")
+    ops.gemm(L.TP_GEMM_NT, Ad, Bd, M, N, K, C=C, epilogue=L.TP_EPI_BIAS_RELU, bias=bd)
+    assert_close(C, base.relu(), dtype, "bias+relu")
+    Z = torch.empty_like(C)
+    ops.gemm(L.TP_GEMM_NT, Ad, Bd, M, N, K, C=C, epilogue=L.TP_EPI_BIAS_GELU, bias=bd, aux_out=Z)
+    assert_close(C, oracle.gelu_erf(base), dtype, "bias+gelu")
+    assert_close(Z, base, dtype, "gelu pre-activation")
+    ops.gemm(L.TP_GEMM_NT, Ad, Bd, M, N, K, C=C, epilogue=L.TP_EPI_BIAS_RESIDUAL, bias=bd, residual=Rd)
+    assert_close(C, base + R.double(), dtype, "bias+residual")
+    # activation gradients fused into the data-gradient GEMM, with the bias-gradient column sums
+    plain = A.double() @ B.double().t()
+    acc = torch.zeros(N, dtype=torch.float32, device=DEV)
+    ops.gemm(L.TP_GEMM_NT, Ad, Bd, M, N, K, C=C, epilogue=L.TP_EPI_RELU_GRAD, aux=Rd, colsum_acc=acc)
+    ref = plain * (R.double() > 0)
+    assert_close(C, ref, dtype, "relu grad")
+    assert_close(acc, ref.sum(0), dtype, "relu grad colsum")
+    acc.zero_()
+    ops.gemm(L.TP_GEMM_NT, Ad, Bd, M, N, K, C=C, epilogue=L.TP_EPI_GELU_GRAD, aux=Rd, colsum_acc=acc)
+    z = R.double().requires_grad_(True)
+    oracle.gelu_erf(z).sum().backward()
+    ref = plain * z.grad
+    assert_close(C, ref, dtype, "gelu grad")
+    assert_close(acc, ref.sum(0), dtype, "gelu grad colsum")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("T,B,H,Dh,P,L", [(16, 2, 4, 64, 32, 128), (32, 1, 2, 128, 0, 64), (5, 3, 2, 64, 3, 16)])
+def test_gemm_qkv_scatter(dtype, T, B, H, Dh, P, L):
+    ops = _ops()
+    from terapipe_amd import _lib as Lb
+    E = H * Dh
+    g = torch.Generator().manual_seed(T + B + H)
+    x, W, b = _rnd((T, B, E), dtype, g), _rnd((3 * E, E), dtype, g, E ** -0.5), _rnd((3 * E,), dtype, g, 0.3)
+    q = torch.zeros(B * H, T, Dh, dtype=dtype, device=DEV)
+    kc = torch.full((B * H, L, Dh), 7.0, dtype=dtype, device=DEV)
+    vc = torch.full((B * H, L, Dh), 7.0, dtype=dtype, device=DEV)
+    ops.gemm(Lb.TP_GEMM_NT, x.view(T * B, E).to(DEV), W.to(DEV), T * B, 3 * E, E, epilogue=Lb.TP_EPI_QKV_SCATTER,
+             bias=b.to(DEV), qkv=dict(q=q, k_cache=kc, v_cache=vc, batch=B, heads=H, head_dim=Dh, cache_len=P,
+                                      cache_rows=L, q_scale=Dh ** -0.5))
+    qkv = oracle.linear_col(x.double(), W.double(), b.double())
+    qr, kr, vr = oracle.split_qkv(qkv, H)
+    assert_close(q, qr * Dh ** -0.5, dtype, "q")
+    assert_close(kc[:, P:P + T], kr, dtype, "k rows")
+    assert_close(vc[:, P:P + T], vr, dtype, "v rows")
+    # rows outside the slice are untouched
+    assert (kc[:, :P] == 7).all() and (kc[:, P + T:] == 7).all()
+    assert (vc[:, :P] == 7).all() and (vc[:, P + T:] == 7).all()
+
+
+def _attn_ref(q, kc, vc, B, H, T, P):
+    """fp64 restatement through the oracle's attention_core; q, kc, vc are leaf tensors."""
+    S = P + T
+    mask = oracle.causal_prefix_mask(T, P, torch.float64)
+    return oracle.attention_core(q, kc[:, :S], vc[:, :S], mask, T, B)
+
+
+ATTN_CASES = [
+    # T, B, H, Dh, P, L
+    (16, 2, 4, 64, 0, 128),
+    (16, 2, 4, 64, 112, 128),
+    (32, 2, 3, 128, 480, 512),     # single-wave workgroups + split over keys
+    (128, 1, 4, 128, 896, 1024),   # four waves, split
+    (256, 1, 2, 128, 256, 512),    # multiple query blocks
+    (160, 1, 2, 128, 100, 300),    # ragged against every tile size
+    (7, 1, 1, 64, 5, 12),
+    (1, 1, 1, 64, 0, 1),
+    (64, 1, 2, 128, 0, 64),        # two waves
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("T,B,H,Dh,P,L", ATTN_CASES)
+def test_attn_prefix_fwd_bwd(dtype, T, B, H, Dh, P, L):
+    ops = _ops()
+    S, E, BH = P + T, H * Dh, B * H
+    g = torch.Generator().manual_seed(T * 3 + P)
+    q = _rnd((BH, T, Dh), dtype, g, 1.0)          # already "scaled" q as far as the kernel is concerned
+    kc, vc = _rnd((BH, L, Dh), dtype, g, Dh ** -0.25), _rnd((BH, L, Dh), dtype, g)
+    d_o = _rnd((T, B, E), dtype, g)
+    inc_k, inc_v = _rnd((BH, L, Dh), dtype, g), _rnd((BH, L, Dh), dtype, g)
+    qd, kd, vd = q.to(DEV), kc.to(DEV), vc.to(DEV)
+    o, lse = ops.attn_prefix_fwd(qd, kd, vd, B, H, Dh, T, P, 1.0)
+    q64 = q.double().requires_grad_(True)
+    k64, v64 = kc.double().requires_grad_(True), vc.double().requires_grad_(True)
+    oref = _attn_ref(q64, k64, v64, B, H, T, P)
+    assert_close(o, oref, dtype, "attn o")
+    s = torch.bmm(q64, k64[:, :S].transpose(1, 2)) + oracle.causal_prefix_mask(T, P, torch.float64)
+    assert_close(lse, torch.logsumexp(s, -1), torch.float32, "attn lse", 1e3 if dtype != torch.float32 else 10)
+    oref.backward(d_o.double())
+    # library-routine pin for the no-prefix case
+    if P == 0:
+        sd = F.scaled_dot_product_attention(q.double(), kc[:, :S].double(), vc[:, :S].double(), is_causal=True, scale=1.0)
+        assert_close(o, sd.transpose(0, 1).reshape(T, B, E), dtype, "attn o vs SDPA")
+
+    for gdt in ([dtype] if dtype == torch.float32 else [dtype, torch.float32]):
+        for incoming in (False, True):
+            gk = inc_k.to(gdt).to(DEV) if incoming else torch.full((BH, L, Dh), 3.0, dtype=gdt, device=DEV)
+            gv = inc_v.to(gdt).to(DEV) if incoming else torch.full((BH, L, Dh), 3.0, dtype=gdt, device=DEV)
+            dqkv = torch.empty(T * B, 3 * E, dtype=dtype, device=DEV)
+            acc = torch.zeros(3 * E, dtype=torch.float32, device=DEV)
+            ops.attn_prefix_bwd(qd, kd, vd, o, lse, d_o.to(DEV), dqkv, gk, gv, B, H, Dh, T, P, 0.5,
+                                accumulate_prefix=incoming, has_incoming=incoming, zero_slice_rows=incoming,
+                                colsum_dqkv_acc=acc)
+            dq, dk, dv = oracle.split_qkv(dqkv.view(T, B, 3 * E).double().cpu(), H)
+            tag = "[gdt=%s incoming=%s]" % (gdt, incoming)
+            assert_close(dq, q64.grad * 0.5, dtype, "dq" + tag)
+            ik = inc_k.double() if incoming else torch.zeros(BH, L, Dh, dtype=torch.float64)
+            iv = inc_v.double() if incoming else torch.zeros(BH, L, Dh, dtype=torch.float64)
+            assert_close(dk, k64.grad[:, P:S] + ik[:, P:S], dtype, "dk slice" + tag)
+            assert_close(dv, v64.grad[:, P:S] + iv[:, P:S], dtype, "dv slice" + tag)
+            if P > 0:
+                assert_close(gk[:, :P], k64.grad[:, :P] + ik[:, :P], dtype, "gk prefix" + tag)
+                assert_close(gv[:, :P], v64.grad[:, :P] + iv[:, :P], dtype, "gv prefix" + tag)
+            if incoming:
+                assert (gk[:, P:S] == 0).all() and (gv[:, P:S] == 0).all(), "slice rows zeroed" + tag
+                assert torch.equal(gk[:, S:].cpu(), inc_k.to(gdt)[:, S:]), "rows beyond the slice untouched" + tag
+            else:
+                assert (gk[:, P:] == 3).all() and (gv[:, P:] == 3).all(), "rows beyond the prefix untouched" + tag
+            assert_close(acc, dqkv.double().sum(0), dtype, "dqkv colsum" + tag)
+
+
+def test_error_paths():
+    """Bad arguments come back as status codes with a message; nothing is launched."""
+    import ctypes
+    from terapipe_amd import _lib as L
+    lib = L.load()
+    d = L.GemmDesc()
+    assert lib.tp_gemm(ctypes.byref(d), None, 0, None) != 0
+    assert b"tp_gemm" in lib.tp_last_error()
+    ops = _ops()
+    x = torch.zeros(4, 20, dtype=torch.float16, device=DEV)   # E not a multiple of 8
+    w = torch.zeros(20, dtype=torch.float16, device=DEV)
+    with pytest.raises(L.TeraPipeHipError):
+        ops.layernorm_fwd(x, w, w)
+    q = torch.zeros(2, 4, 96, dtype=torch.float16, device=DEV)  # head_dim 96 unsupported
+    kc = torch.zeros(2, 8, 96, dtype=torch.float16, device=DEV)
+    with pytest.raises(L.TeraPipeHipError):
+        ops.attn_prefix_fwd(q, kc, kc, 1, 2, 96, 4, 0, 1.0)
+    with pytest.raises(L.TeraPipeHipError):
+        ops.layernorm_fwd(torch.zeros(4, 64), torch.zeros(64), torch.zeros(64))  # CPU tensors

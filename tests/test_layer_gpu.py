@@ -1,0 +1,335 @@
+"""Layer / stack / sliced-runner parity on the GPU against the CPU oracle (same seeded inputs).
+
+Tolerance (per tensor, max |got - ref| / max |ref|): 1e-5 fp32, 2e-2 fp16/bf16.  For 16-bit runs the
+oracle consumes the weights and inputs already rounded to the kernel dtype and computes in fp32.
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from tests.util import TOL, assert_close, load_params_into, make_params, oracle_run, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+
+
+def _mods():
+    import terapipe_amd
+    return terapipe_amd
+
+
+def _build_layers(ta, n_layers, E, Fd, H, dtype, ps, activation="relu"):
+    layers = ta.TransformerLayers(n_layers, E, Fd, H, mixed_precision=(dtype != torch.float32), dtype=dtype,
+                                  device=DEV, activation=activation)
+    load_params_into(layers, ps, dtype)
+    return layers
+
+
+def _param_grads(layers):
+    return [{n: t.grad for n, t in layer.param_dict().items()} for layer in layers.layers]
+
+
+def _check_param_grads(got, ref, dtype, tag):
+    worst = 0.0
+    for l, (g, r) in enumerate(zip(got, ref)):
+        for n in r:
+            assert g[n] is not None, "%s layer %d %s has no grad" % (tag, l, n)
+            worst = max(worst, assert_close(g[n], r[n], dtype, "%s layer %d d(%s)" % (tag, l, n)))
+    return worst
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("activation", ["relu", "gelu"])
+def test_single_layer_with_prefix(dtype, activation):
+    """One layer, one slice, a pre-filled prefix: outputs, the cache rows it writes, and every gradient
+    including the cache-input gradients and their zeroed slice rows (transformer_models.py:186-190)."""
+    ta = _mods()
+    T, B, H, Dh, P, L = 16, 2, 4, 64, 24, 64
+    E, Fd = H * Dh, 4 * H * Dh
+    ps = make_params(1, E, Fd, dtype, seed=3)
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(T, B, E, generator=g).to(dtype)
+    kc0, vc0 = torch.randn(B * H, L, Dh, generator=g).to(dtype), torch.randn(B * H, L, Dh, generator=g).to(dtype)
+    dy = torch.randn(T, B, E, generator=g).to(dtype)
+    dkc, dvc = torch.randn(B * H, L, Dh, generator=g).to(dtype), torch.randn(B * H, L, Dh, generator=g).to(dtype)
+
+    # oracle in fp32
+    p32 = {k: v.clone().requires_grad_(True) for k, v in ps[0].items()}
+    xo = x.float().requires_grad_(True)
+    ko, vo = kc0.float().clone().requires_grad_(True), vc0.float().clone().requires_grad_(True)
+    yo, (ko_out, vo_out) = oracle.layer_forward(p32, xo, H, (ko, vo), P, activation=activation)
+    torch.autograd.backward([yo, ko_out, vo_out], [dy.float(), dkc.float(), dvc.float()])
+
+    layers = _build_layers(ta, 1, E, Fd, H, dtype, ps, activation)
+    layer = layers.layers[0]
+    xd = x.to(DEV).requires_grad_(True)
+    kd, vd = kc0.to(DEV).clone().requires_grad_(True), vc0.to(DEV).clone().requires_grad_(True)
+    y, (k_out, v_out) = layer(xd, (kd, vd), P)
+    assert k_out.data_ptr() == kd.data_ptr() and v_out.data_ptr() == vd.data_ptr(), "caches are updated in place"
+    assert_close(y, yo, dtype, "y")
+    assert_close(k_out, ko_out, dtype, "k cache")
+    assert_close(v_out, vo_out, dtype, "v cache")
+    torch.autograd.backward([y, k_out, v_out], [dy.to(DEV), dkc.to(DEV), dvc.to(DEV)])
+    assert_close(xd.grad, xo.grad, dtype, "dx")
+    assert_close(kd.grad, ko.grad, dtype, "d k_cache")
+    assert_close(vd.grad, vo.grad, dtype, "d v_cache")
+    assert (kd.grad[:, P:P + T] == 0).all() and (vd.grad[:, P:P + T] == 0).all()
+    _check_param_grads(_param_grads(layers), [{k: v.grad for k, v in p32.items()}], dtype, "single layer")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_layer_without_cache_is_plain_causal_attention(dtype):
+    """full_cache=None path (transformer_models.py:230-234)."""
+    ta = _mods()
+    T, B, H, Dh = 48, 2, 2, 64
+    E, Fd = H * Dh, 2 * H * Dh
+    ps = make_params(1, E, Fd, dtype, seed=5)
+    g = torch.Generator().manual_seed(2)
+    x, dy = torch.randn(T, B, E, generator=g).to(dtype), torch.randn(T, B, E, generator=g).to(dtype)
+    p32 = {k: v.clone().requires_grad_(True) for k, v in ps[0].items()}
+    xo = x.float().requires_grad_(True)
+    yo, none = oracle.layer_forward(p32, xo, H, None, 0)
+    assert none is None
+    yo.backward(dy.float())
+    layers = _build_layers(ta, 1, E, Fd, H, dtype, ps)
+    xd = x.to(DEV).requires_grad_(True)
+    y, cache = layers.layers[0](xd)
+    assert cache is None
+    y.backward(dy.to(DEV))
+    assert_close(y, yo, dtype, "y")
+    assert_close(xd.grad, xo.grad, dtype, "dx")
+    _check_param_grads(_param_grads(layers), [{k: v.grad for k, v in p32.items()}], dtype, "no-cache layer")
+    with pytest.raises(AssertionError):
+        layers.layers[0](xd, None, 4)      # cache_len must be 0 without a cache
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_attention_module_alone(dtype):
+    """MultiheadLMAttentionWithCache.forward(x, full_cache, cache_len) with autograd through the caches."""
+    ta = _mods()
+    T, B, H, Dh, P, L = 8, 1, 2, 128, 8, 24
+    E = H * Dh
+    ps = make_params(1, E, 4 * E, dtype, seed=9)
+    g = torch.Generator().manual_seed(4)
+    x, dy = torch.randn(T, B, E, generator=g).to(dtype), torch.randn(T, B, E, generator=g).to(dtype)
+    kc0, vc0 = torch.randn(B * H, L, Dh, generator=g).to(dtype), torch.randn(B * H, L, Dh, generator=g).to(dtype)
+    p32 = {k: v.clone().requires_grad_(True) for k, v in ps[0].items()}
+    xo = x.float().requires_grad_(True)
+    ko, vo = kc0.float().clone().requires_grad_(True), vc0.float().clone().requires_grad_(True)
+    yo, (ko_out, vo_out) = oracle.attention_forward(p32, "attn.", xo, H, (ko, vo), P)
+    yo.backward(dy.float())
+    layers = _build_layers(ta, 1, E, 4 * E, H, dtype, ps)
+    attn = layers.layers[0].attn
+    xd = x.to(DEV).requires_grad_(True)
+    kd, vd = kc0.to(DEV).clone().requires_grad_(True), vc0.to(DEV).clone().requires_grad_(True)
+    y, (k_out, v_out) = attn(xd, (kd, vd), P)
+    y.backward(dy.to(DEV))
+    assert_close(y, yo, dtype, "attn y")
+    assert_close(xd.grad, xo.grad, dtype, "attn dx")
+    assert_close(kd.grad, ko.grad, dtype, "attn d k_cache")
+    assert_close(vd.grad, vo.grad, dtype, "attn d v_cache")
+    for n in ("attn.in_proj.weight", "attn.in_proj.bias", "attn.out_proj.weight", "attn.out_proj.bias"):
+        assert_close(layers.layers[0].param_dict()[n].grad, p32[n].grad, dtype, n)
+
+
+def _reference_style_loop(layers, x, dy, batch_slices, seq_slices):
+    """The slice loop of the reference's TeraPipe.forward + TeraPipeBackwardPassHook.backward
+    (terapipe.py:249-264, :182-191) driven through the layer-level autograd surface."""
+    ta = _mods()
+    xs = ta.grid_slice_batch_and_sequence(x, batch_slices, seq_slices, requires_grad=True)
+    dys = ta.grid_slice_batch_and_sequence(dy, batch_slices, seq_slices)
+    nb, ns = len(batch_slices), len(seq_slices)
+    cache_inputs = np.empty((nb, ns), dtype="O")
+    cache_outputs = np.empty((nb, ns), dtype="O")
+    outputs = np.empty((nb, ns), dtype="O")
+    finals = []
+    for b in range(nb):
+        cache = layers.create_cache(batch_slices[b], x.size(0))
+        cache_len = 0
+        for i in range(ns):
+            cache = [c.detach().requires_grad_() for c in cache]
+            y, cache_out = layers(xs[b, i], cache, cache_len)
+            cache_inputs[b, i], cache_outputs[b, i], outputs[b, i] = cache, cache_out, y
+            cache = cache_out
+            cache_len += seq_slices[i]
+        finals.append([c.detach() for c in cache])
+    for b in reversed(range(nb)):
+        da = []
+        for i in reversed(range(ns)):
+            a = list(cache_outputs[b, i]) if i < ns - 1 else []
+            torch.autograd.backward([outputs[b, i]] + a, [dys[b, i]] + da)
+            da = [t.grad for t in cache_inputs[b, i]]
+    y = torch.cat([torch.cat(list(outputs[b]), 0) for b in range(nb)], 1).detach()
+    dx = torch.cat([torch.cat([xs[b, i].grad for i in range(ns)], 0) for b in range(nb)], 1)
+    cg = [[[t.grad for t in cache_inputs[b, i]] for i in range(ns)] for b in range(nb)]
+    return y, dx, finals, cg
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_reference_style_slice_loop(dtype):
+    """Layer-level autograd contract: detach()/requires_grad_() caches per slice, backward with the
+    cache-output gradients of the next slice, cache-input .grad as hand-off."""
+    ta = _mods()
+    n_layers, E, H, L, B = 2, 256, 4, 64, 2
+    Fd = 4 * E
+    bs, ss = [1, 1], [16, 24, 8, 16]
+    ps = make_params(n_layers, E, Fd, dtype, seed=1)
+    g = torch.Generator().manual_seed(7)
+    x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
+    leaf = [{k: v.clone().requires_grad_(True) for k, v in p.items()} for p in ps]
+    yo, dxo, fco, cgo = oracle.terapipe_forward_backward(leaf, x.float(), dy.float(), H, bs, ss, return_cache_grads=True)
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    y, dx, finals, cg = _reference_style_loop(layers, x.to(DEV), dy.to(DEV), bs, ss)
+    assert_close(y, yo, dtype, "y")
+    assert_close(dx, dxo, dtype, "dx")
+    for b in range(len(bs)):
+        for j in range(2 * n_layers):
+            assert_close(finals[b][j], fco[b][j], dtype, "final cache %d/%d" % (b, j))
+            for i in range(1, len(ss)):
+                P = sum(ss[:i])
+                assert_close(cg[b][i][j], cgo[b][i][j], dtype, "cache grad b%d slice %d tensor %d" % (b, i, j))
+                assert (cg[b][i][j][:, P:] == 0).all(), "rows >= P of the cache gradient are zero"
+    _check_param_grads(_param_grads(layers), [{k: v.grad for k, v in p.items()} for p in leaf], dtype, "ref loop")
+
+
+def _run_terapipe(ta, layers, x, dy, B, L, bs, ss, **kw):
+    for p in layers.parameters():
+        p.grad = None
+    runner = ta.TeraPipe(layers, B, L, bs, ss, **kw)
+    xd = x.to(DEV).requires_grad_(True)
+    y = runner(xd)
+    (y * dy.to(DEV)).sum().backward()
+    return runner, y.detach(), xd.grad
+
+
+@pytest.mark.parametrize("defer,fp32gc", [(True, True), (False, True), (False, False), (True, False)])
+def test_terapipe_c1_tiny_fp32(defer, fp32gc):
+    """BASELINE config 1 (layer stack part): 4 layers, hidden 256, 4 heads, FFN 1024, seq 128, batch 2,
+    fp32, 8 slices of 16, reverse-slice backward, tolerance 1e-5."""
+    ta = _mods()
+    n_layers, E, H, Fd, L, B = 4, 256, 4, 1024, 128, 2
+    ss = oracle.uniform_slice(L, 8)
+    ps = make_params(n_layers, E, Fd, torch.float32, seed=0)
+    g = torch.Generator().manual_seed(0)
+    x, dy = torch.randn(L, B, E, generator=g), torch.randn(L, B, E, generator=g)
+    yo, dxo, fco, go = oracle_run(ps, x, dy, H, [B], ss)
+    layers = _build_layers(ta, n_layers, E, Fd, H, torch.float32, ps)
+    runner, y, dx = _run_terapipe(ta, layers, x, dy, B, L, [B], ss, defer_weight_grads=defer, fp32_grad_cache=fp32gc)
+    assert_close(y, yo, torch.float32, "y")
+    assert_close(dx, dxo, torch.float32, "dx")
+    for j in range(2 * n_layers):
+        assert_close(runner.last_caches[0][j], fco[0][j], torch.float32, "final cache %d" % j)
+    _check_param_grads(_param_grads(layers), go, torch.float32, "C1")
+
+
+def test_terapipe_c1_tokens_and_cross_entropy():
+    """BASELINE config 1 end to end: token ids -> embedding -> sliced stack -> LM head -> mean cross
+    entropy on random next-token targets.  The embedding / LM head / loss are harness-owned torch ops on
+    both sides; the stack between them is the HIP path vs the oracle."""
+    ta = _mods()
+    n_layers, E, H, Fd, L, B, V = 4, 256, 4, 1024, 128, 2, 50257
+    ss = oracle.uniform_slice(L, 8)
+    ps = make_params(n_layers, E, Fd, torch.float32, seed=0, rand_small=False)
+    g = torch.Generator().manual_seed(123)
+    emb = torch.randn(V, E, generator=g) * 0.02
+    ids = torch.randint(0, V, (L, B), generator=g)
+    tgt = torch.randint(0, V, (L, B), generator=g)
+
+    def head_loss(y, emb_w):
+        return F.cross_entropy((y @ emb_w.t()).view(L * B, V), tgt.to(y.device).view(-1))
+
+    # oracle side
+    emb_o = emb.clone().requires_grad_(True)
+    x_o = F.embedding(ids, emb_o)
+    x_leaf = x_o.detach().clone()
+    y_tmp = x_leaf.clone().requires_grad_(True)
+    leaf = [{k: v.clone().requires_grad_(True) for k, v in p.items()} for p in ps]
+    # forward once without grad to get y, then the loss gradient dy, then the sliced backward
+    with torch.no_grad():
+        h = x_leaf
+        cache = oracle.create_cache(n_layers, B, H, L, E // H)
+        outs, cl = [], 0
+        for s in ss:
+            yi, cache = oracle.stack_forward(leaf, h[cl:cl + s], H, cache, cl)
+            outs.append(yi)
+            cl += s
+        y_full = torch.cat(outs, 0)
+    y_req = y_full.clone().requires_grad_(True)
+    loss_o = head_loss(y_req, emb_o)
+    loss_o.backward()
+    yo, dxo, _ = oracle.terapipe_forward_backward(leaf, x_leaf, y_req.grad, H, [B], ss)
+    x_o.backward(dxo)
+
+    layers = _build_layers(ta, n_layers, E, Fd, H, torch.float32, ps)
+    emb_d = emb.to(DEV).requires_grad_(True)
+    runner = ta.TeraPipe(layers, B, L, [B], ss)
+    y = runner(F.embedding(ids.to(DEV), emb_d))
+    loss = head_loss(y, emb_d)
+    loss.backward()
+    assert abs(loss.item() - loss_o.item()) <= 1e-5 * abs(loss_o.item())
+    assert_close(y, yo, torch.float32, "y")
+    assert_close(emb_d.grad, emb_o.grad, torch.float32, "d embedding", 2)
+    _check_param_grads(_param_grads(layers), [{k: v.grad for k, v in p.items()} for p in leaf], torch.float32, "C1 CE")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("case", ["uniform", "nonuniform", "fine", "batch_sliced"])
+def test_terapipe_16bit_reduced_shapes(dtype, case):
+    """Reduced-size versions of BASELINE configs 2-5 (head dim 128, N(0,1) inputs, random-projection
+    loss): uniform 256-token slices, the non-uniform DP-style slice list, 32-token slices, and a batch
+    of 2 cut into two batch slices."""
+    ta = _mods()
+    H, Dh = 4, 128
+    E, Fd = H * Dh, 4 * H * Dh
+    n_layers, L, B, bs = 2, 1024, 1, [1]
+    if case == "uniform":
+        ss = [256] * 4
+    elif case == "nonuniform":
+        ss = [256, 192, 160, 128, 112, 96, 80]
+    elif case == "fine":
+        L, B, bs = 512, 2, [2]
+        ss = [32] * 16
+    else:
+        L, B, bs = 512, 2, [1, 1]
+        ss = [128] * 4
+    ps = make_params(n_layers, E, Fd, dtype, seed=2, rand_small=True)
+    g = torch.Generator().manual_seed(17)
+    x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
+    yo, dxo, fco, go = oracle_run(ps, x, dy, H, bs, ss)
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    for defer, fp32gc in [(True, True), (False, False)]:
+        runner, y, dx = _run_terapipe(ta, layers, x, dy, B, L, bs, ss, defer_weight_grads=defer, fp32_grad_cache=fp32gc)
+        tag = "%s defer=%s fp32gc=%s" % (case, defer, fp32gc)
+        assert_close(y, yo, dtype, tag + " y")
+        assert_close(dx, dxo, dtype, tag + " dx")
+        for b in range(len(bs)):
+            for j in range(2 * n_layers):
+                assert_close(runner.last_caches[b][j], fco[b][j], dtype, tag + " final cache")
+        _check_param_grads(_param_grads(layers), go, dtype, tag)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_slicing_invariance_full_width(dtype):
+    """Size-independent property at a BASELINE width (hidden 2048, 16 heads, seq 2048): gradients with 8
+    slices equal gradients with one slice (the invariant of test_transformer_terapipe.py:333-352),
+    computed entirely by the HIP path."""
+    ta = _mods()
+    n_layers, E, H, L, B = 2, 2048, 16, 2048, 1
+    Fd = 4 * E
+    layers = ta.TransformerLayers(n_layers, E, Fd, H, dtype=dtype, device=DEV)
+    g = torch.Generator().manual_seed(5)
+    with torch.no_grad():
+        for p in layers.parameters():
+            if p.dim() == 2:
+                p.copy_((torch.randn(p.shape, generator=g) * 0.02).to(dtype))
+    x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
+    _, y8, dx8 = _run_terapipe(ta, layers, x, dy, B, L, [B], [256] * 8)
+    g8 = [{n: t.grad.clone() for n, t in layer.param_dict().items()} for layer in layers.layers]
+    _, y1, dx1 = _run_terapipe(ta, layers, x, dy, B, L, [B], [L])
+    g1 = _param_grads(layers)
+    assert_close(y8, y1, dtype, "y")
+    assert_close(dx8, dx1, dtype, "dx")
+    _check_param_grads(g8, g1, dtype, "sliced vs unsliced")
