@@ -88,12 +88,12 @@ def split_qkv(qkv: torch.Tensor, num_heads: int):
     return q, k, v
 
 
-def causal_prefix_mask(T: int, P: int, dtype=torch.float32):
+def causal_prefix_mask(T: int, P: int, dtype=torch.float32, device=None):
     """transformer_models.py:220,229 -- additive mask [T, P+T]: zeros over the prefix columns,
     NEG_INF strictly above the diagonal of the slice block."""
-    tri = torch.full((T, T), NEG_INF, dtype=dtype).triu_(1)
+    tri = torch.full((T, T), NEG_INF, dtype=dtype, device=device).triu_(1)
     if P > 0:
-        return torch.cat([torch.zeros(T, P, dtype=dtype), tri], dim=1)
+        return torch.cat([torch.zeros(T, P, dtype=dtype, device=device), tri], dim=1)
     return tri
 
 
@@ -148,11 +148,11 @@ def attention_forward(p: Dict[str, torch.Tensor], prefix: str, x, num_heads: int
         cache_v = assign_cache(cache_v, new_v, cache_len, S)        # :226
         k = cache_k[:, :S, :]                                       # :227
         v = cache_v[:, :S, :]                                       # :228
-        mask = causal_prefix_mask(T, cache_len, x.dtype)            # :229
+        mask = causal_prefix_mask(T, cache_len, x.dtype, x.device)  # :229
     else:
         assert cache_len == 0                                       # :231
         k, v = new_k, new_v
-        mask = causal_prefix_mask(T, 0, x.dtype)
+        mask = causal_prefix_mask(T, 0, x.dtype, x.device)
     a = attention_core(q, k, v, mask, T, B)
     out = linear_row(a, p[prefix + "out_proj.weight"], p[prefix + "out_proj.bias"])  # :251
     if full_cache is not None:
@@ -161,8 +161,13 @@ def attention_forward(p: Dict[str, torch.Tensor], prefix: str, x, num_heads: int
 
 
 def layer_forward(p: Dict[str, torch.Tensor], x, num_heads: int, full_cache=None,
-                  cache_len: int = 0, prefix: str = "", activation: str = "relu"):
-    """TransformerLayer.forward, transformer_models.py:273-285 (pre-LN block, ReLU MLP)."""
+                  cache_len: int = 0, prefix: str = "", activation: str = "relu", relu_mask=None):
+    """TransformerLayer.forward, transformer_models.py:273-285 (pre-LN block, ReLU MLP).
+
+    relu_mask (optional bool tensor shaped like the fc1 output) replaces ``z > 0`` as the ReLU's
+    active set: a 16-bit run decides the sign of near-zero pre-activations by its own rounding, and a
+    parity test that wants to measure arithmetic error rather than those sign flips hands the mask of
+    the run under test to the oracle.  The reference path is relu_mask=None."""
     y = x
     h = layer_norm(x, p[prefix + "attn_ln.weight"], p[prefix + "attn_ln.bias"])       # :275
     h, new_cache = attention_forward(p, prefix + "attn.", h, num_heads, full_cache, cache_len)
@@ -170,28 +175,35 @@ def layer_forward(p: Dict[str, torch.Tensor], x, num_heads: int, full_cache=None
     y = h
     z = layer_norm(h, p[prefix + "fc_ln.weight"], p[prefix + "fc_ln.bias"])           # :280
     z = linear_col(z, p[prefix + "fc1.weight"], p[prefix + "fc1.bias"])
-    z = torch.relu(z) if activation == "relu" else gelu_erf(z)                       # :282
+    if activation == "relu":
+        z = torch.relu(z) if relu_mask is None else z * relu_mask.to(z.dtype)        # :282
+    else:
+        z = gelu_erf(z)
     z = linear_row(z, p[prefix + "fc2.weight"], p[prefix + "fc2.bias"])               # :283
     return z + y, new_cache                                                          # :284-285
 
 
-def stack_forward(params: List[Dict[str, torch.Tensor]], x, num_heads: int, cache, cache_len: int):
-    """TransformerLayers.forward, terapipe.py:79-86; cache is the flat list [k0, v0, k1, v1, ...]."""
+def stack_forward(params: List[Dict[str, torch.Tensor]], x, num_heads: int, cache, cache_len: int,
+                  activation: str = "relu", relu_masks=None):
+    """TransformerLayers.forward, terapipe.py:79-86; cache is the flat list [k0, v0, k1, v1, ...].
+    relu_masks: optional list (one per layer) passed to layer_forward."""
     cache_outputs = []
     for i, p in enumerate(params):
-        x, (ko, vo) = layer_forward(p, x, num_heads, (cache[2 * i], cache[2 * i + 1]), cache_len)
+        x, (ko, vo) = layer_forward(p, x, num_heads, (cache[2 * i], cache[2 * i + 1]), cache_len,
+                                    activation=activation,
+                                    relu_mask=None if relu_masks is None else relu_masks[i])
         cache_outputs += [ko, vo]
     return x, cache_outputs
 
 
 def create_cache(n_layers: int, batch_size: int, num_heads: int, seq_len: int, head_dim: int,
-                 dtype=torch.float32):
+                 dtype=torch.float32, device=None):
     """TransformerLayers.create_cache (terapipe.py:70-77) over create_attn_cache
     (transformer_models.py:257-261): zeros [B*H, L, Dh] for K and V of every layer."""
     cache = []
     for _ in range(n_layers):
-        cache += [torch.zeros(batch_size * num_heads, seq_len, head_dim, dtype=dtype),
-                  torch.zeros(batch_size * num_heads, seq_len, head_dim, dtype=dtype)]
+        cache += [torch.zeros(batch_size * num_heads, seq_len, head_dim, dtype=dtype, device=device),
+                  torch.zeros(batch_size * num_heads, seq_len, head_dim, dtype=dtype, device=device)]
     return cache
 
 
@@ -241,14 +253,15 @@ def grid_slice_batch_and_sequence(x, batch_slices, seq_slices, requires_grad=Fal
 
 def terapipe_forward_backward(params: List[Dict[str, torch.Tensor]], x, dy, num_heads: int,
                               batch_slices: Sequence[int], seq_slices: Sequence[int],
-                              return_cache_grads: bool = False):
+                              return_cache_grads: bool = False, activation: str = "relu", relu_masks=None):
     """TeraPipe.forward (terapipe.py:238-271) followed by TeraPipeBackwardPassHook.backward
     (terapipe.py:167-201) on a single pipeline stage.
 
     ``params`` must be leaf tensors with requires_grad=True; their .grad accumulates over slices
     exactly as in the reference (autograd sum).  Returns (y, dx, final_caches[, cache_grads]) where
     final_caches[b] is the flat K/V list after the last slice of batch slice b and cache_grads[b][i]
-    is the list of .grad tensors of the cache inputs of slice i.
+    is the list of .grad tensors of the cache inputs of slice i.  relu_masks, if given, maps
+    (batch slice, sequence slice) to the per-layer list of ReLU active sets (see layer_forward).
     """
     L = x.size(0)
     E = x.size(2)
@@ -261,12 +274,13 @@ def terapipe_forward_backward(params: List[Dict[str, torch.Tensor]], x, dy, num_
     outputs = np.empty((nb, ns), dtype="O")
     final_caches = []
     for b in range(nb):
-        cache = create_cache(n_layers, inputs[b, 0].size(1), num_heads, L, Dh, x.dtype)   # :251
+        cache = create_cache(n_layers, inputs[b, 0].size(1), num_heads, L, Dh, x.dtype, x.device)  # :251
         cache_len = 0
         for i in range(ns):
             xi = inputs[b, i]
             cache = [c.detach().requires_grad_() for c in cache]                          # :257
-            y, cache_out = stack_forward(params, xi, num_heads, cache, cache_len)          # :258
+            y, cache_out = stack_forward(params, xi, num_heads, cache, cache_len, activation,      # :258
+                                         None if relu_masks is None else relu_masks[(b, i)])
             cache_inputs[b, i] = cache
             cache_outputs[b, i] = cache_out
             cache = cache_out

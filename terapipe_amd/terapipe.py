@@ -103,6 +103,8 @@ class _TeraPipeFunction(torch.autograd.Function):
                 cache_len += runner.seq_slices[i]                                    # terapipe.py:264
             caches.append(cache)
         runner.last_caches = caches
+        if runner.keep_states:
+            runner.last_states = states.copy()
         y = torch.cat([torch.cat(list(outs[b]), dim=runner.sequence_dim) for b in range(nb)], dim=runner.batch_dim)
         ctx.runner, ctx.ws, ctx.act, ctx.states = runner, ws, act, states
         ctx.in_shape = inputs.shape
@@ -194,6 +196,8 @@ class TeraPipe(nn.Module):
         self.defer_weight_grads = defer_weight_grads
         self.fp32_grad_cache = fp32_grad_cache
         self.last_caches = None
+        self.keep_states = False   # debugging / tests: keep the per-slice saved activations of the last forward
+        self.last_states = None
 
     @property
     def n_batch_slices(self):

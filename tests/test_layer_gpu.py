@@ -2,6 +2,15 @@
 
 Tolerance (per tensor, max |got - ref| / max |ref|): 1e-5 fp32, 2e-2 fp16/bf16.  For 16-bit runs the
 oracle consumes the weights and inputs already rounded to the kernel dtype and computes in fp32.
+
+ReLU in 16 bit: the derivative of relu_ (reference transformer_models.py:282) is discontinuous, and a
+16-bit run decides the sign of near-zero pre-activations by its own rounding.  A few in a thousand
+elements flip, and each flip moves a gradient entry by its full magnitude: plain PyTorch fp16/bf16 (the
+reference's own numerics) is 2e-2 ... 1e-1 away from the fp32 oracle on the gradients behind the ReLU
+for exactly this reason (measured; test_relu_flip_error_is_not_worse_than_plain_torch_16bit keeps that
+comparison alive).  The 16-bit gradient checks therefore give the oracle the HIP run's ReLU active set
+(oracle.layer_forward(relu_mask=...)), which makes the 2e-2 bound measure arithmetic error only; the
+fp32 runs (1e-5) and the GeLU runs (2e-2) need no such alignment and cover the same kernels.
 """
 import numpy as np
 import pytest
@@ -26,6 +35,15 @@ def _build_layers(ta, n_layers, E, Fd, H, dtype, ps, activation="relu"):
                                   device=DEV, activation=activation)
     load_params_into(layers, ps, dtype)
     return layers
+
+
+def _relu_masks_from_states(states):
+    """{(b, i): [mask per layer]} with mask = (saved fc1 activation > 0) reshaped [T, B, F], on the CPU."""
+    out = {}
+    for b in range(states.shape[0]):
+        for i in range(states.shape[1]):
+            out[(b, i)] = [(st.a > 0).view(st.T, st.B, -1).cpu() for st in states[b, i]]
+    return out
 
 
 def _param_grads(layers):
@@ -56,18 +74,21 @@ def test_single_layer_with_prefix(dtype, activation):
     dy = torch.randn(T, B, E, generator=g).to(dtype)
     dkc, dvc = torch.randn(B * H, L, Dh, generator=g).to(dtype), torch.randn(B * H, L, Dh, generator=g).to(dtype)
 
-    # oracle in fp32
-    p32 = {k: v.clone().requires_grad_(True) for k, v in ps[0].items()}
-    xo = x.float().requires_grad_(True)
-    ko, vo = kc0.float().clone().requires_grad_(True), vc0.float().clone().requires_grad_(True)
-    yo, (ko_out, vo_out) = oracle.layer_forward(p32, xo, H, (ko, vo), P, activation=activation)
-    torch.autograd.backward([yo, ko_out, vo_out], [dy.float(), dkc.float(), dvc.float()])
-
     layers = _build_layers(ta, 1, E, Fd, H, dtype, ps, activation)
     layer = layers.layers[0]
     xd = x.to(DEV).requires_grad_(True)
     kd, vd = kc0.to(DEV).clone().requires_grad_(True), vc0.to(DEV).clone().requires_grad_(True)
     y, (k_out, v_out) = layer(xd, (kd, vd), P)
+    mask = None
+    if dtype != torch.float32 and activation == "relu":
+        mask = (y.grad_fn.st.a > 0).view(T, B, Fd).cpu()
+
+    # oracle in fp32
+    p32 = {k: v.clone().requires_grad_(True) for k, v in ps[0].items()}
+    xo = x.float().clone().requires_grad_(True)
+    ko, vo = kc0.float().clone().requires_grad_(True), vc0.float().clone().requires_grad_(True)
+    yo, (ko_out, vo_out) = oracle.layer_forward(p32, xo, H, (ko, vo), P, activation=activation, relu_mask=mask)
+    torch.autograd.backward([yo, ko_out, vo_out], [dy.float(), dkc.float(), dvc.float()])
     assert k_out.data_ptr() == kd.data_ptr() and v_out.data_ptr() == vd.data_ptr(), "caches are updated in place"
     assert_close(y, yo, dtype, "y")
     assert_close(k_out, ko_out, dtype, "k cache")
@@ -89,15 +110,16 @@ def test_layer_without_cache_is_plain_causal_attention(dtype):
     ps = make_params(1, E, Fd, dtype, seed=5)
     g = torch.Generator().manual_seed(2)
     x, dy = torch.randn(T, B, E, generator=g).to(dtype), torch.randn(T, B, E, generator=g).to(dtype)
-    p32 = {k: v.clone().requires_grad_(True) for k, v in ps[0].items()}
-    xo = x.float().requires_grad_(True)
-    yo, none = oracle.layer_forward(p32, xo, H, None, 0)
-    assert none is None
-    yo.backward(dy.float())
     layers = _build_layers(ta, 1, E, Fd, H, dtype, ps)
     xd = x.to(DEV).requires_grad_(True)
     y, cache = layers.layers[0](xd)
     assert cache is None
+    mask = None if dtype == torch.float32 else (y.grad_fn.st.a > 0).view(T, B, Fd).cpu()
+    p32 = {k: v.clone().requires_grad_(True) for k, v in ps[0].items()}
+    xo = x.float().clone().requires_grad_(True)
+    yo, none = oracle.layer_forward(p32, xo, H, None, 0, relu_mask=mask)
+    assert none is None
+    yo.backward(dy.float())
     y.backward(dy.to(DEV))
     assert_close(y, yo, dtype, "y")
     assert_close(xd.grad, xo.grad, dtype, "dx")
@@ -117,7 +139,7 @@ def test_attention_module_alone(dtype):
     x, dy = torch.randn(T, B, E, generator=g).to(dtype), torch.randn(T, B, E, generator=g).to(dtype)
     kc0, vc0 = torch.randn(B * H, L, Dh, generator=g).to(dtype), torch.randn(B * H, L, Dh, generator=g).to(dtype)
     p32 = {k: v.clone().requires_grad_(True) for k, v in ps[0].items()}
-    xo = x.float().requires_grad_(True)
+    xo = x.float().clone().requires_grad_(True)
     ko, vo = kc0.float().clone().requires_grad_(True), vc0.float().clone().requires_grad_(True)
     yo, (ko_out, vo_out) = oracle.attention_forward(p32, "attn.", xo, H, (ko, vo), P)
     yo.backward(dy.float())
@@ -176,12 +198,16 @@ def test_reference_style_slice_loop(dtype):
     n_layers, E, H, L, B = 2, 256, 4, 64, 2
     Fd = 4 * E
     bs, ss = [1, 1], [16, 24, 8, 16]
+    # fp32 runs the reference's ReLU; the 16-bit runs use the smooth activation so that the bound is not
+    # dominated by ReLU sign flips (see the module docstring)
+    act = "relu" if dtype == torch.float32 else "gelu"
     ps = make_params(n_layers, E, Fd, dtype, seed=1)
     g = torch.Generator().manual_seed(7)
     x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
     leaf = [{k: v.clone().requires_grad_(True) for k, v in p.items()} for p in ps]
-    yo, dxo, fco, cgo = oracle.terapipe_forward_backward(leaf, x.float(), dy.float(), H, bs, ss, return_cache_grads=True)
-    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    yo, dxo, fco, cgo = oracle.terapipe_forward_backward(leaf, x.float(), dy.float(), H, bs, ss,
+                                                         return_cache_grads=True, activation=act)
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps, act)
     y, dx, finals, cg = _reference_style_loop(layers, x.to(DEV), dy.to(DEV), bs, ss)
     assert_close(y, yo, dtype, "y")
     assert_close(dx, dxo, dtype, "dx")
@@ -195,10 +221,11 @@ def test_reference_style_slice_loop(dtype):
     _check_param_grads(_param_grads(layers), [{k: v.grad for k, v in p.items()} for p in leaf], dtype, "ref loop")
 
 
-def _run_terapipe(ta, layers, x, dy, B, L, bs, ss, **kw):
+def _run_terapipe(ta, layers, x, dy, B, L, bs, ss, keep_states=False, **kw):
     for p in layers.parameters():
         p.grad = None
     runner = ta.TeraPipe(layers, B, L, bs, ss, **kw)
+    runner.keep_states = keep_states
     xd = x.to(DEV).requires_grad_(True)
     y = runner(xd)
     (y * dy.to(DEV)).sum().backward()
@@ -298,10 +325,15 @@ def test_terapipe_16bit_reduced_shapes(dtype, case):
     ps = make_params(n_layers, E, Fd, dtype, seed=2, rand_small=True)
     g = torch.Generator().manual_seed(17)
     x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
-    yo, dxo, fco, go = oracle_run(ps, x, dy, H, bs, ss)
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
     for defer, fp32gc in [(True, True), (False, False)]:
-        runner, y, dx = _run_terapipe(ta, layers, x, dy, B, L, bs, ss, defer_weight_grads=defer, fp32_grad_cache=fp32gc)
+        runner, y, dx = _run_terapipe(ta, layers, x, dy, B, L, bs, ss, keep_states=True,
+                                      defer_weight_grads=defer, fp32_grad_cache=fp32gc)
+        # oracle with the ReLU active set of this run (module docstring)
+        leaf = [{k: v.clone().requires_grad_(True) for k, v in p.items()} for p in ps]
+        yo, dxo, fco = oracle.terapipe_forward_backward(leaf, x.float(), dy.float(), H, bs, ss,
+                                                        relu_masks=_relu_masks_from_states(runner.last_states))
+        go = [{k: v.grad for k, v in p.items()} for p in leaf]
         tag = "%s defer=%s fp32gc=%s" % (case, defer, fp32gc)
         assert_close(y, yo, dtype, tag + " y")
         assert_close(dx, dxo, dtype, tag + " dx")
@@ -319,7 +351,8 @@ def test_slicing_invariance_full_width(dtype):
     ta = _mods()
     n_layers, E, H, L, B = 2, 2048, 16, 2048, 1
     Fd = 4 * E
-    layers = ta.TransformerLayers(n_layers, E, Fd, H, dtype=dtype, device=DEV)
+    # smooth activation: the two runs round differently, and ReLU sign flips would dominate the bound
+    layers = ta.TransformerLayers(n_layers, E, Fd, H, dtype=dtype, device=DEV, activation="gelu")
     g = torch.Generator().manual_seed(5)
     with torch.no_grad():
         for p in layers.parameters():
@@ -333,3 +366,32 @@ def test_slicing_invariance_full_width(dtype):
     assert_close(y8, y1, dtype, "y")
     assert_close(dx8, dx1, dtype, "dx")
     _check_param_grads(g8, g1, dtype, "sliced vs unsliced")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_relu_flip_error_is_not_worse_than_plain_torch_16bit(dtype):
+    """Against the UNALIGNED fp32 oracle (ReLU decided by the oracle's own fp32 pre-activations) the HIP
+    path is no further away than the reference's own numerics: the same op sequence run by plain PyTorch
+    kernels in the same 16-bit dtype on the same inputs (with a 1.5x + 5e-3 margin)."""
+    ta = _mods()
+    n_layers, E, H, L, B = 2, 512, 4, 512, 1
+    Fd, ss = 4 * E, [128] * 4
+    ps = make_params(n_layers, E, Fd, dtype, seed=2)
+    g = torch.Generator().manual_seed(17)
+    x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
+    yo, dxo, _, go = oracle_run(ps, x, dy, H, [B], ss)
+    leaf16 = [{k: v.to(dtype).to(DEV).requires_grad_(True) for k, v in p.items()} for p in ps]
+    y16, dx16, _ = oracle.terapipe_forward_backward(leaf16, x.to(DEV), dy.to(DEV), H, [B], ss)
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    _, y, dx = _run_terapipe(ta, layers, x, dy, B, L, [B], ss)
+    got = _param_grads(layers)
+    assert_close(y, yo, dtype, "y")
+
+    def bound(t16, ref):
+        return 1.5 * rel_err(t16, ref) + 5e-3
+
+    assert rel_err(dx, dxo) <= bound(dx16, dxo), "dx"
+    for l in range(n_layers):
+        for n in go[l]:
+            e_hip, b = rel_err(got[l][n], go[l][n]), bound(leaf16[l][n].grad, go[l][n])
+            assert e_hip <= b, "layer %d d(%s): hip %.3e, plain torch bound %.3e" % (l, n, e_hip, b)
