@@ -1,0 +1,197 @@
+#!/usr/bin/env python3
+"""Headline benchmark: sliced GPT-layer-stack forward + reverse-slice backward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3|C4|C5|C1]
+
+One step = every sequence slice of one synthetic batch through the whole layer stack forward (K/V
+caches growing slice by slice), then the reverse-order slice backward, with the loss
+``sum(y * R)`` for a fixed random R (inputs N(0,1), weights N(0,0.02), all resident in HBM before the
+timed region).  Prints ONE JSON line: tokens/s, the MFMA roofline of the GEMM kernels (algorithmic
+flops / HIP-event kernel time, measured live in an extra instrumented step), the HBM figure of the
+prefix-attention kernels, and the CPU oracle timed on this host's cores on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+PEAK_MFMA_16BIT = 2.5e15     # dense fp16/bf16 MFMA flop/s
+PEAK_MFMA_FP32 = 157.3e12
+PEAK_HBM = 8.0e12            # bytes/s
+
+WORKLOADS = {
+    # name: layers, hidden, heads, ffn, seq, batch, dtype, slices, weight std
+    "C1": dict(desc="tiny GPT stack fp32: 4 layers, hidden 256, 4 heads, FFN 1024, seq 128, batch 2, 8x16 slices",
+               n_layers=4, E=256, H=4, F=1024, L=128, B=2, dtype="f32", slices=[16] * 8, std=0.02),
+    "C2": dict(desc="GPT-3 1.3B shape: 24 layers, hidden 2048, 16 heads, FFN 8192, seq 2048, batch 1, fp16, 8x256 slices",
+               n_layers=24, E=2048, H=16, F=8192, L=2048, B=1, dtype="f16", slices=[256] * 8, std=0.02),
+    "C3": dict(desc="GPT-3 13B stage share: 5 layers, hidden 5120, 40 heads, FFN 20480, seq 2048, batch 1, fp16, "
+                    "slices [512,384,320,256,224,192,160]",
+               n_layers=5, E=5120, H=40, F=20480, L=2048, B=1, dtype="f16",
+               slices=[512, 384, 320, 256, 224, 192, 160], std=0.02),
+    "C4": dict(desc="GPT-3 175B stage share: 2 layers, hidden 12288, 96 heads, FFN 49152, seq 2048, batch 1, bf16, 16x128 slices",
+               n_layers=2, E=12288, H=96, F=49152, L=2048, B=1, dtype="bf16", slices=[128] * 16, std=0.006),
+    "C5": dict(desc="GPT-3 44B stage share: 4 layers, hidden 6144, 48 heads, FFN 24576, seq 2048, batch 2, bf16, 64x32 slices",
+               n_layers=4, E=6144, H=48, F=24576, L=2048, B=2, dtype="bf16", slices=[32] * 64, std=0.02),
+}
+TORCH_DTYPE = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+
+
+def gemm_flops_per_step(w):
+    """72 * E^2 flops per token per layer fwd+bwd for F = 4E; stated generally as
+    3 passes (fwd, dX, dW) x 2 * (3E*E + E*E + 2*E*F) per token."""
+    per_token_fwd = 2 * (3 * w["E"] * w["E"] + w["E"] * w["E"] + 2 * w["E"] * w["F"])
+    return 3 * per_token_fwd * w["L"] * w["B"] * w["n_layers"]
+
+
+def attn_bytes_per_call(w, T, P, bwd):
+    """Algorithmic HBM bytes of one prefix-attention call (one layer, one slice): elements x dtype size
+    plus the fp32 LSE / delta vectors.  fwd (2T + 2S) B E; bwd (6T + 2S + 4P) B E."""
+    es = 4 if w["dtype"] == "f32" else 2
+    S, BE, BH = P + T, w["B"] * w["E"], w["B"] * w["H"]
+    if not bwd:
+        return (2 * T + 2 * S) * BE * es + 4 * BH * T
+    return (6 * T + 2 * S + 4 * P) * BE * es + 8 * BH * T
+
+
+def build_model(w, device):
+    import terapipe_amd as ta
+    dt = TORCH_DTYPE[w["dtype"]]
+    layers = ta.TransformerLayers(w["n_layers"], w["E"], w["F"], w["H"], dtype=dt, device=device)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    with torch.no_grad():
+        for p in layers.parameters():
+            if p.dim() == 2:   # weights N(0, std); biases stay 0, LayerNorm gamma 1 / beta 0
+                p.copy_((torch.randn(p.shape, generator=g) * w["std"]).to(dt))
+    runner = ta.TeraPipe(layers, w["B"], w["L"], [w["B"]], w["slices"])
+    x = torch.randn(w["L"], w["B"], w["E"], generator=g).to(dt).to(device)
+    R = torch.randn(w["L"], w["B"], w["E"], generator=g).to(dt).to(device)
+    return layers, runner, x, R
+
+
+def one_step(layers, runner, x, R):
+    for p in layers.parameters():
+        p.grad = None
+    y = runner(x)
+    loss = (y * R).sum()
+    loss.backward()
+    return loss
+
+
+def cpu_baseline(w, budget_layers=None):
+    """The CPU oracle (fp32 restatement of the reference path) on this host's cores, on a bounded
+    sample: the full sequence and slice list through `sample_layers` layers of the stack; the
+    whole-stack rate is that rate divided by n_layers / sample_layers."""
+    import oracle
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    flops_layer = gemm_flops_per_step(w) / w["n_layers"]
+    sample_layers = budget_layers or max(1, min(w["n_layers"], int(4e12 // flops_layer)))
+    ps = oracle.init_stack_params(sample_layers, w["E"], w["F"], w["std"], torch.float32, seed=0)
+    for p in ps:
+        for v in p.values():
+            v.requires_grad_(True)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(w["L"], w["B"], w["E"], generator=g)
+    R = torch.randn(w["L"], w["B"], w["E"], generator=g)
+    t0 = time.time()
+    oracle.terapipe_forward_backward(ps, x, R, w["H"], [w["B"]], w["slices"])
+    dt = time.time() - t0
+    tokens = w["L"] * w["B"]
+    value = tokens / (dt * w["n_layers"] / sample_layers)
+    return {"value": value, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": "fp32 torch-CPU oracle, full sequence and slice list through %d of %d layers, one step "
+                      "(%.1f s), scaled by the layer count" % (sample_layers, w["n_layers"], dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-roofline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
+              "(no collectives or sharding are part of this build)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    w = WORKLOADS[args.workload]
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    from terapipe_amd import ops
+
+    layers, runner, x, R = build_model(w, device)
+    for _ in range(args.warmup):
+        one_step(layers, runner, x, R)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        one_step(layers, runner, x, R)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    tokens = w["L"] * w["B"]
+    value = tokens * args.steps / elapsed
+
+    out = {
+        "metric": "sliced-layer fwd+bwd tokens/s on 1 MI355X; % MFMA peak (GEMM), % HBM BW (attn)",
+        "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": w["dtype"], "data": "synthetic",
+        "config": {"workload": "%s: %s" % (args.workload, w["desc"]),
+                   "loss": "sum(y * R), R ~ N(0,1) fixed", "optimizer_step": "not part of the path"},
+    }
+
+    if not args.no_roofline:
+        # one instrumented step: every library call bracketed by HIP events on the launch stream
+        with ops.KernelTimer() as kt:
+            one_step(layers, runner, x, R)
+            torch.cuda.synchronize()
+        summ = kt.summary()
+        g_calls, g_ms, _ = summ.get("gemm", (0, 0.0, []))
+        flops = gemm_flops_per_step(w)
+        peak = PEAK_MFMA_FP32 if w["dtype"] == "f32" else PEAK_MFMA_16BIT
+        achieved = flops / (g_ms * 1e-3) if g_ms > 0 else 0.0
+        out["roofline"] = {
+            "kernel": "tp::gemm_kernel (all NT/NN/TN launches of one step, split-K reduce included)",
+            "bound": "mfma", "achieved": achieved / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
+            "frac": achieved / peak, "traffic": None,
+            "launches": g_calls, "avg_launch_us": g_ms * 1e3 / max(g_calls, 1),
+            "algorithmic_flops_per_step": flops, "kernel_ms_per_step": g_ms,
+        }
+        # prefix attention: algorithmic bytes / kernel time, over all calls of the step
+        a_bytes = {"attn_fwd": 0.0, "attn_bwd": 0.0}
+        for tag in a_bytes:
+            for (_b, _h, _d, T, P) in summ.get(tag, (0, 0.0, []))[2]:
+                a_bytes[tag] += attn_bytes_per_call(w, T, P, tag == "attn_bwd")
+        attn = {}
+        for tag in a_bytes:
+            c, ms, _ = summ.get(tag, (0, 0.0, []))
+            gbs = a_bytes[tag] / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+            attn[tag] = {"calls": c, "kernel_ms_per_step": ms, "algorithmic_GB_per_step": a_bytes[tag] / 1e9,
+                         "achieved_GBps": gbs, "frac_of_hbm_peak": gbs * 1e9 / PEAK_HBM}
+        out["roofline_attention"] = {"bound": "hbm", "peak": PEAK_HBM / 1e9, "unit": "GB/s", **attn}
+        out["kernel_time_ms_per_step"] = {k: round(v[1], 3) for k, v in summ.items()}
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w)
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -37,6 +37,50 @@ def _require_cuda(*tensors):
             raise _lib.TeraPipeHipError("terapipe_amd kernels need CUDA/HIP tensors; there is no CPU path")
 
 
+class KernelTimer:
+    """Optional per-call HIP-event timing of the library calls (used by bench.py for the roofline
+    figures).  While active, every wrapped call is bracketed by two events on the current stream."""
+    active = None
+
+    def __init__(self):
+        self.records = []   # (tag, meta, start_event, end_event)
+
+    def __enter__(self):
+        KernelTimer.active = self
+        return self
+
+    def __exit__(self, *exc):
+        KernelTimer.active = None
+
+    def summary(self):
+        """{tag: (calls, total_ms, [meta...])} -- call after torch.cuda.synchronize()."""
+        out = {}
+        for tag, meta, e0, e1 in self.records:
+            c, ms, metas = out.get(tag, (0, 0.0, []))
+            metas.append(meta)
+            out[tag] = (c + 1, ms + e0.elapsed_time(e1), metas)
+        return out
+
+
+class _timed:
+    __slots__ = ("tag", "meta", "e0")
+
+    def __init__(self, tag, meta=None):
+        self.tag, self.meta = tag, meta
+
+    def __enter__(self):
+        if KernelTimer.active is not None:
+            self.e0 = torch.cuda.Event(enable_timing=True)
+            self.e0.record()
+        return self
+
+    def __exit__(self, *exc):
+        if KernelTimer.active is not None:
+            e1 = torch.cuda.Event(enable_timing=True)
+            e1.record()
+            KernelTimer.active.records.append((self.tag, self.meta, self.e0, e1))
+
+
 class Workspace:
     """A grow-only scratch tensor per device (torch-owned), handed to calls that need workspace."""
     _bufs = {}
@@ -58,8 +102,9 @@ def layernorm_fwd(x2d, gamma, beta, eps=1e-5):
     mean = torch.empty(M, dtype=torch.float32, device=x2d.device)
     rstd = torch.empty(M, dtype=torch.float32, device=x2d.device)
     lib = _lib.load()
-    _lib.check(lib.tp_layernorm_fwd(_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps,
-                                    tp_dtype(x2d.dtype), _stream()), "tp_layernorm_fwd")
+    with _timed("layernorm_fwd", (M, E)):
+        _lib.check(lib.tp_layernorm_fwd(_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps,
+                                        tp_dtype(x2d.dtype), _stream()), "tp_layernorm_fwd")
     return y, mean, rstd
 
 
@@ -69,9 +114,10 @@ def layernorm_bwd(dy, x2d, mean, rstd, gamma, dres, dgamma_acc, dbeta_acc, colsu
     M, E = x2d.shape
     dx = torch.empty_like(x2d)
     lib = _lib.load()
-    _lib.check(lib.tp_layernorm_bwd(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx),
-                                    _p(dgamma_acc), _p(dbeta_acc), _p(colsum_dres_acc), _p(colsum_dx_acc),
-                                    M, E, tp_dtype(x2d.dtype), _stream()), "tp_layernorm_bwd")
+    with _timed("layernorm_bwd", (M, E)):
+        _lib.check(lib.tp_layernorm_bwd(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx),
+                                        _p(dgamma_acc), _p(dbeta_acc), _p(colsum_dres_acc), _p(colsum_dx_acc),
+                                        M, E, tp_dtype(x2d.dtype), _stream()), "tp_layernorm_bwd")
     return dx
 
 
@@ -102,7 +148,8 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
     lib = _lib.load()
     need = lib.tp_gemm_workspace_bytes(ctypes.byref(d))
     ws = Workspace.get(need, A.device) if need else None
-    _lib.check(lib.tp_gemm(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()), "tp_gemm")
+    with _timed("gemm", (op, M, N, K)):
+        _lib.check(lib.tp_gemm(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()), "tp_gemm")
     return C
 
 
@@ -126,8 +173,9 @@ def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q
     lib = _lib.load()
     need = lib.tp_attn_fwd_workspace_bytes(ctypes.byref(d))
     ws = Workspace.get(need, q.device) if need else None
-    _lib.check(lib.tp_attn_prefix_fwd(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()),
-               "tp_attn_prefix_fwd")
+    with _timed("attn_fwd", (batch, heads, head_dim, T, cache_len)):
+        _lib.check(lib.tp_attn_prefix_fwd(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()),
+                   "tp_attn_prefix_fwd")
     return o, lse
 
 
@@ -143,7 +191,8 @@ def attn_prefix_bwd(q, k_cache, v_cache, o, lse, d_o, dqkv, dk_cache, dv_cache, 
     d.accumulate_prefix, d.has_incoming, d.zero_slice_rows = int(accumulate_prefix), int(has_incoming), int(zero_slice_rows)
     d.colsum_dqkv_acc = _p(colsum_dqkv_acc)
     lib = _lib.load()
-    _lib.check(lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()), "tp_attn_prefix_bwd")
+    with _timed("attn_bwd", (batch, heads, head_dim, T, cache_len)):
+        _lib.check(lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()), "tp_attn_prefix_bwd")
     return dqkv
 
 
