@@ -1,0 +1,121 @@
+"""CPU-side checks of the boundary: the shared library loads and exports every symbol that
+include/terapipe_hip.h declares, the ctypes mirrors match the C struct sizes, and argument errors are
+reported without touching a GPU.  No compute calls."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+import tempfile
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "terapipe_hip.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound(lib):
+    from terapipe_amd import _lib
+    names = _declared_symbols()
+    assert len(names) >= 13
+    for n in names:
+        assert hasattr(lib, n), "library does not export %s" % n
+        assert n in _lib.SYMBOLS, "ctypes binding misses %s" % n
+    assert sorted(_lib.SYMBOLS) == names
+
+
+def test_struct_sizes_match_c_compiler(lib):
+    """Compiles a 10-line C program against the header with gcc and compares sizeof/offsetof."""
+    from terapipe_amd import _lib
+    src = r'''
+#include <stdio.h>
+#include <stddef.h>
+#include "terapipe_hip.h"
+int main(void) {
+  printf("%zu %zu %zu %zu %zu %zu\n", sizeof(tp_gemm_desc), offsetof(tp_gemm_desc, colsum_acc),
+         offsetof(tp_gemm_desc, q_scale), sizeof(tp_attn_desc), offsetof(tp_attn_desc, q_scale),
+         offsetof(tp_attn_desc, colsum_dqkv_acc));
+  return 0;
+}'''
+    with tempfile.TemporaryDirectory() as d:
+        c = os.path.join(d, "t.c")
+        open(c, "w").write(src)
+        exe = os.path.join(d, "t")
+        subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), c, "-o", exe])
+        got = [int(v) for v in subprocess.check_output([exe]).split()]
+    G, A = _lib.GemmDesc, _lib.AttnDesc
+    assert got == [ctypes.sizeof(G), G.colsum_acc.offset, G.q_scale.offset, ctypes.sizeof(A), A.q_scale.offset,
+                   A.colsum_dqkv_acc.offset]
+
+
+def test_argument_errors_without_gpu(lib):
+    from terapipe_amd import _lib
+    assert lib.tp_version() >= 100
+    d = _lib.GemmDesc()
+    assert lib.tp_gemm(ctypes.byref(d), None, 0, None) == 1          # TP_ERR_ARG
+    assert b"shape" in lib.tp_last_error()
+    d.M, d.N, d.K, d.dtype = 8, 8, 12, _lib.TP_F16                   # K not a multiple of 8
+    d.A = d.B = d.C = 256
+    d.lda = d.ldb = 12
+    d.ldc = 8
+    assert lib.tp_gemm(ctypes.byref(d), None, 0, None) == 2          # TP_ERR_UNSUPPORTED
+    assert lib.tp_gemm_workspace_bytes(ctypes.byref(d)) == 0
+    a = _lib.AttnDesc()
+    a.head_dim = 96
+    assert lib.tp_attn_prefix_fwd(ctypes.byref(a), None, 0, None) != 0
+    assert b"head_dim" in lib.tp_last_error()
+    assert lib.tp_layernorm_fwd(None, None, None, None, None, None, 4, 64, 1e-5, 0, None) == 1
+    assert lib.tp_zero_words(None, 4, None) == 1
+
+
+def test_ops_refuse_cpu_tensors():
+    """There is no CPU fallback: host tensors raise instead of computing."""
+    from terapipe_amd import _lib, ops
+    with pytest.raises(_lib.TeraPipeHipError):
+        ops.layernorm_fwd(torch.zeros(4, 64), torch.ones(64), torch.zeros(64))
+    with pytest.raises(_lib.TeraPipeHipError):
+        ops.gemm(_lib.TP_GEMM_NT, torch.zeros(8, 8), torch.zeros(8, 8), 8, 8, 8, C=torch.zeros(8, 8))
+
+
+def test_package_does_not_import_the_oracle():
+    """The shipped package must not reach into oracle/ (test infrastructure only)."""
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "terapipe_amd")):
+        for f in files:
+            if f.endswith(".py"):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(import|from)\s+oracle\b", text, flags=re.M), f
+    code = "import sys; sys.path.insert(0, %r); import terapipe_amd; assert 'oracle' not in sys.modules" % ROOT
+    subprocess.check_call([sys.executable, "-c", code])
+
+
+def test_host_side_surface_mirrors_reference_names():
+    import terapipe_amd as ta
+    from terapipe_amd import transformer_models as tm
+    layer = ta.ModelParallelTransformerLayer(64, 256, 1, device="cpu")
+    keys = set(layer.state_dict().keys())
+    assert keys == {"attn_ln.weight", "attn_ln.bias", "attn.in_proj.weight", "attn.in_proj.bias",
+                    "attn.out_proj.weight", "attn.out_proj.bias", "fc_ln.weight", "fc_ln.bias",
+                    "fc1.weight", "fc1.bias", "fc2.weight", "fc2.bias"}
+    assert layer.attn.in_proj.weight.shape == (192, 64) and layer.fc1.weight.shape == (256, 64)
+    assert not layer.fc1.bias.abs().any() and not layer.attn.out_proj.bias.abs().any()   # zero-init biases
+    k, v = layer.attn.create_attn_cache(2, 16, device="cpu", dtype=torch.float16)
+    assert k.shape == (2, 16, 64) and k.dtype == torch.float16 and not k.abs().any()
+    with pytest.raises(AssertionError):
+        tm.MultiheadLMAttentionWithCache(100, 3)              # embed_dim not divisible by heads
+    with pytest.raises(AssertionError):
+        layer(torch.zeros(4, 1, 32))                          # wrong embedding dim
+    with pytest.raises(AssertionError):
+        layer(torch.zeros(4, 1, 64), None, 3)                 # cache_len without a cache
+    assert ta.uniform_slice(10, 4) == [3, 3, 2, 2]
+    assert tm.MODEL_CONFIGS["gpt3-13b"] == (40, 5120, 2048, 40) and tm.BATCH_CONFIGS["gpt3-175b"] == 2
+    cfg = tm.TransformerConfig.from_predefined_model("gpt3-1b")
+    assert (cfg.n_layers, cfg.embedding_dim, cfg.ffn_embedding_dim, cfg.attention_heads_dim) == (24, 2048, 8192, 128)
+    with pytest.raises(AssertionError):
+        ta.TeraPipe(None, 2, 16, [2], [8, 4])                 # slices must sum to the sequence length
