@@ -45,7 +45,8 @@ int tp_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y
 
 /* Backward of the above fused with the residual-path add that follows it in the layer
  * (transformer_models.py:277, :284 are `x += y`, so the gradient of the LayerNorm input is
- * LN'(dy) + dres).  dres may be NULL.  The parameter gradients are ADDED into fp32 accumulators:
+ * LN'(dy) + dres).  dres may be NULL.  The parameter gradients are ADDED into fp32 accumulators
+ * (dgamma_acc and dbeta_acc may both be NULL to skip them, see tp_ln_param_grads):
  *   dgamma_acc[E] += sum_m dy * xhat,   dbeta_acc[E] += sum_m dy,
  *   colsum_dres_acc[E] += sum_m dres    (NULL to skip; this is the bias gradient of the
  *                                        row-parallel linear whose output fed the residual add),
@@ -56,6 +57,13 @@ int tp_layernorm_bwd(const void* dy, const void* x, const float* mean, const flo
                      const void* gamma, const void* dres, void* dx, float* dgamma_acc,
                      float* dbeta_acc, float* colsum_dres_acc, float* colsum_dx_acc, int M, int E,
                      int dtype, void* stream);
+
+/* LayerNorm parameter gradients over a block of rows (used once per layer over ALL tokens of a step
+ * when the per-slice tp_layernorm_bwd calls pass NULL accumulators):
+ *   dgamma_acc[E] += sum_m dy[m] * (x[m] - mean[m]) * rstd[m],   dbeta_acc[E] += sum_m dy[m].
+ * Same sums autograd accumulates into nn.LayerNorm's weight.grad / bias.grad across slices. */
+int tp_ln_param_grads(const void* dy, const void* x, const float* mean, const float* rstd,
+                      float* dgamma_acc, float* dbeta_acc, int M, int E, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * GEMMs that mpu.ColumnParallelLinear / RowParallelLinear reduce to at tensor-parallel size 1
@@ -103,7 +111,7 @@ typedef struct tp_gemm_desc {
     int32_t batch, heads, head_dim, cache_len;
     int64_t cache_rows;                 /* L_max: rows per (b,h) in the caches */
     float q_scale;
-    int32_t reserved;
+    int32_t reserved;                   /* 0 = automatic; bits 0-7: tile configuration + 1, bits 8-15: k splits (tuning, tests) */
 } tp_gemm_desc;
 
 size_t tp_gemm_workspace_bytes(const tp_gemm_desc* d);

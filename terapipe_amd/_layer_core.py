@@ -44,46 +44,67 @@ class SliceState:
                  "k_cache", "v_cache", "cache_len", "T", "B")
 
 
-def attention_fwd(w, xn2d, T, B, heads, k_cache, v_cache, cache_len):
+class Bufs:
+    """Optional preallocated outputs for one layer-slice call (views into the runner's per-layer
+    buffers).  Any attribute left at None is allocated by the call."""
+    __slots__ = ("xn", "mean1", "rstd1", "q", "o", "lse", "h", "mean2", "rstd2", "hn", "a", "z", "out",
+                 "dz1", "dhn", "dh", "d_o", "dqkv", "dxn", "dx", "delta")
+
+    def __init__(self, **kw):
+        for n in self.__slots__:
+            setattr(self, n, kw.get(n))
+
+
+_NOBUF = Bufs()
+
+
+def _buf(t, shape, dtype, device):
+    return torch.empty(shape, dtype=dtype, device=device) if t is None else t
+
+
+def attention_fwd(w, xn2d, T, B, heads, k_cache, v_cache, cache_len, buf=_NOBUF):
     """in_proj GEMM with the q/k/v split, q scaling and cache assignment fused into its epilogue, then
     the prefix-cached attention kernel.  Returns q [B*H, T, Dh], o [T, B, E], lse."""
     E = xn2d.shape[1]
     Dh = E // heads
     M = T * B
-    q = torch.empty(B * heads, T, Dh, dtype=xn2d.dtype, device=xn2d.device)
+    q = _buf(buf.q, (B * heads, T, Dh), xn2d.dtype, xn2d.device)
     scale = float(Dh) ** -0.5
     ops.gemm(TP_GEMM_NT, xn2d, w["attn.in_proj.weight"], M, 3 * E, E, epilogue=TP_EPI_QKV_SCATTER,
              bias=w["attn.in_proj.bias"],
              qkv=dict(q=q, k_cache=k_cache, v_cache=v_cache, batch=B, heads=heads, head_dim=Dh,
                       cache_len=cache_len, cache_rows=k_cache.shape[1], q_scale=scale))
-    o, lse = ops.attn_prefix_fwd(q, k_cache, v_cache, B, heads, Dh, T, cache_len, scale)
+    o, lse = ops.attn_prefix_fwd(q, k_cache, v_cache, B, heads, Dh, T, cache_len, scale, out=buf.o, lse=buf.lse)
     return q, o, lse
 
 
-def layer_fwd(w, x, heads, k_cache, v_cache, cache_len, activation="relu", need_state=True):
+def layer_fwd(w, x, heads, k_cache, v_cache, cache_len, activation="relu", need_state=True, buf=_NOBUF):
     """x [T, B, E] contiguous.  Writes rows [cache_len, cache_len+T) of the caches.  Returns (out, state)."""
     T, B, E = x.shape
     M = T * B
     F = w["fc1.weight"].shape[0]
+    dt, dev = x.dtype, x.device
     x2d = x.view(M, E)
-    xn, mean1, rstd1 = ops.layernorm_fwd(x2d, w["attn_ln.weight"], w["attn_ln.bias"])
-    q, o, lse = attention_fwd(w, xn, T, B, heads, k_cache, v_cache, cache_len)
+    xn, mean1, rstd1 = ops.layernorm_fwd(x2d, w["attn_ln.weight"], w["attn_ln.bias"], out=buf.xn, mean=buf.mean1,
+                                         rstd=buf.rstd1)
+    q, o, lse = attention_fwd(w, xn, T, B, heads, k_cache, v_cache, cache_len, buf)
     o2d = o.view(M, E)
-    h = torch.empty_like(x2d)
+    h = _buf(buf.h, (M, E), dt, dev)
     ops.gemm(TP_GEMM_NT, o2d, w["attn.out_proj.weight"], M, E, E, C=h, epilogue=TP_EPI_BIAS_RESIDUAL,
              bias=w["attn.out_proj.bias"], residual=x2d)
-    hn, mean2, rstd2 = ops.layernorm_fwd(h, w["fc_ln.weight"], w["fc_ln.bias"])
-    a = torch.empty(M, F, dtype=x.dtype, device=x.device)
+    hn, mean2, rstd2 = ops.layernorm_fwd(h, w["fc_ln.weight"], w["fc_ln.bias"], out=buf.hn, mean=buf.mean2,
+                                         rstd=buf.rstd2)
+    a = _buf(buf.a, (M, F), dt, dev)
     z = None
     if activation == "relu":
         ops.gemm(TP_GEMM_NT, hn, w["fc1.weight"], M, F, E, C=a, epilogue=TP_EPI_BIAS_RELU, bias=w["fc1.bias"])
     elif activation == "gelu":
-        z = torch.empty_like(a)
+        z = _buf(buf.z, (M, F), dt, dev)
         ops.gemm(TP_GEMM_NT, hn, w["fc1.weight"], M, F, E, C=a, epilogue=TP_EPI_BIAS_GELU, bias=w["fc1.bias"],
                  aux_out=z)
     else:
         raise ValueError("activation must be 'relu' or 'gelu'")
-    out = torch.empty_like(x2d)
+    out = _buf(buf.out, (M, E), dt, dev)
     ops.gemm(TP_GEMM_NT, a, w["fc2.weight"], M, E, F, C=out, epilogue=TP_EPI_BIAS_RESIDUAL,
              bias=w["fc2.bias"], residual=h)
     st = None
@@ -103,58 +124,53 @@ def _wgrad(target, accumulate, A, Bm, M_, N_, K_):
 
 
 def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, accumulate_prefix, has_incoming,
-              zero_slice_rows, activation="relu", defer=None):
+              zero_slice_rows, activation="relu", buf=_NOBUF):
     """Backward of layer_fwd for one slice.
 
-    dout [T, B, E]; gk / gv gradient caches (see tp_attn_desc); wgrad maps the four weight names to
-    gradient tensors that are overwritten (accumulate_wgrad False) or added to; small_acc maps the
-    vector parameter names to fp32 accumulators that are added to.  If `defer` is a dict, the four
-    weight-gradient GEMMs are not run; their operand pairs (dY, X) are stored in it instead so the
-    caller can run one GEMM over all slices.  Returns dx [T, B, E].
+    dout [T, B, E]; gk / gv gradient caches (see tp_attn_desc).  wgrad maps the four weight names to
+    gradient tensors that are overwritten (accumulate_wgrad False) or added to; small_acc maps the vector
+    parameter names to fp32 accumulators that are added to.  With wgrad None / small_acc None the weight
+    / vector-parameter gradients of this slice are NOT computed: the caller keeps the intermediate
+    gradients this call leaves in `buf` (dz1, dhn, dh, dqkv, dxn) and reduces over all slices at once.
+    Returns dx [T, B, E].
     """
     T, B = st.T, st.B
     M = T * B
     E = st.x.shape[1]
     F = st.a.shape[1]
     Dh = E // heads
+    dt, dev = dout.dtype, dout.device
     dout2d = dout.reshape(M, E)
+    sa = small_acc if small_acc is not None else {}
     # MLP
-    dz1 = torch.empty(M, F, dtype=dout.dtype, device=dout.device)
+    dz1 = _buf(buf.dz1, (M, F), dt, dev)
     if activation == "relu":
         ops.gemm(TP_GEMM_NN, dout2d, w["fc2.weight"], M, F, E, C=dz1, epilogue=TP_EPI_RELU_GRAD, aux=st.a,
-                 colsum_acc=small_acc["fc1.bias"])
+                 colsum_acc=sa.get("fc1.bias"))
     else:
         ops.gemm(TP_GEMM_NN, dout2d, w["fc2.weight"], M, F, E, C=dz1, epilogue=TP_EPI_GELU_GRAD, aux=st.z,
-                 colsum_acc=small_acc["fc1.bias"])
-    if defer is None:
+                 colsum_acc=sa.get("fc1.bias"))
+    if wgrad is not None:
         _wgrad(wgrad["fc2.weight"], accumulate_wgrad, dout2d, st.a, E, F, M)
-    else:
-        defer["fc2.weight"] = (dout2d, st.a)
-    dhn = torch.empty(M, E, dtype=dout.dtype, device=dout.device)
+    dhn = _buf(buf.dhn, (M, E), dt, dev)
     ops.gemm(TP_GEMM_NN, dz1, w["fc1.weight"], M, E, F, C=dhn)
-    if defer is None:
+    if wgrad is not None:
         _wgrad(wgrad["fc1.weight"], accumulate_wgrad, dz1, st.hn, F, E, M)
-    else:
-        defer["fc1.weight"] = (dz1, st.hn)
-    dh = ops.layernorm_bwd(dhn, st.h, st.mean2, st.rstd2, w["fc_ln.weight"], dout2d, small_acc["fc_ln.weight"],
-                           small_acc["fc_ln.bias"], small_acc["fc2.bias"], small_acc["attn.out_proj.bias"])
+    dh = ops.layernorm_bwd(dhn, st.h, st.mean2, st.rstd2, w["fc_ln.weight"], dout2d, sa.get("fc_ln.weight"),
+                           sa.get("fc_ln.bias"), sa.get("fc2.bias"), sa.get("attn.out_proj.bias"), out=buf.dh)
     # attention
-    d_o = torch.empty(M, E, dtype=dout.dtype, device=dout.device)
+    d_o = _buf(buf.d_o, (M, E), dt, dev)
     ops.gemm(TP_GEMM_NN, dh, w["attn.out_proj.weight"], M, E, E, C=d_o)
-    if defer is None:
+    if wgrad is not None:
         _wgrad(wgrad["attn.out_proj.weight"], accumulate_wgrad, dh, st.o, E, E, M)
-    else:
-        defer["attn.out_proj.weight"] = (dh, st.o)
-    dqkv = torch.empty(M, 3 * E, dtype=dout.dtype, device=dout.device)
+    dqkv = _buf(buf.dqkv, (M, 3 * E), dt, dev)
     ops.attn_prefix_bwd(st.q, st.k_cache, st.v_cache, st.o, st.lse, d_o, dqkv, gk, gv, B, heads, Dh, T,
                         st.cache_len, float(Dh) ** -0.5, accumulate_prefix, has_incoming, zero_slice_rows,
-                        colsum_dqkv_acc=small_acc["attn.in_proj.bias"])
-    dxn = torch.empty(M, E, dtype=dout.dtype, device=dout.device)
+                        colsum_dqkv_acc=sa.get("attn.in_proj.bias"), delta=buf.delta)
+    dxn = _buf(buf.dxn, (M, E), dt, dev)
     ops.gemm(TP_GEMM_NN, dqkv, w["attn.in_proj.weight"], M, E, 3 * E, C=dxn)
-    if defer is None:
+    if wgrad is not None:
         _wgrad(wgrad["attn.in_proj.weight"], accumulate_wgrad, dqkv, st.xn, 3 * E, E, M)
-    else:
-        defer["attn.in_proj.weight"] = (dqkv, st.xn)
-    dx = ops.layernorm_bwd(dxn, st.x, st.mean1, st.rstd1, w["attn_ln.weight"], dh, small_acc["attn_ln.weight"],
-                           small_acc["attn_ln.bias"], None, None)
+    dx = ops.layernorm_bwd(dxn, st.x, st.mean1, st.rstd1, w["attn_ln.weight"], dh, sa.get("attn_ln.weight"),
+                           sa.get("attn_ln.bias"), None, None, out=buf.dx)
     return dx.view(T, B, E)

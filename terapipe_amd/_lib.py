@@ -61,6 +61,7 @@ SYMBOLS = {
     "tp_last_error": (ctypes.c_char_p, []),
     "tp_layernorm_fwd": (c_int, [c_void_p] * 6 + [c_int, c_int, c_float, c_int, c_void_p]),
     "tp_layernorm_bwd": (c_int, [c_void_p] * 11 + [c_int, c_int, c_int, c_void_p]),
+    "tp_ln_param_grads": (c_int, [c_void_p] * 6 + [c_int, c_int, c_int, c_void_p]),
     "tp_gemm_workspace_bytes": (c_size_t, [ctypes.POINTER(GemmDesc)]),
     "tp_gemm": (c_int, [ctypes.POINTER(GemmDesc), c_void_p, c_size_t, c_void_p]),
     "tp_attn_fwd_workspace_bytes": (c_size_t, [ctypes.POINTER(AttnDesc)]),

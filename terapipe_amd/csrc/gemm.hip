@@ -133,6 +133,207 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& a, int row, int co
     }
 }
 
+// Epilogue shared by the GEMM kernels.  Each wave transposes one 32x32 accumulator block at a time
+// through its own LDS staging block so that a lane ends up with 8 consecutive columns of a row: 16-byte
+// stores and a vector epilogue.  Lane -> (row = lane / 4 + 16 * pass, columns 8 * (lane % 4) .. + 7).
+// `stage_base` must hold 32 * 36 floats per wave and must no longer be read as tile data by any wave.
+template <typename T, int TM, int TN, int WM, int WN>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, float16v (&acc)[TM][TN], float* stage_base,
+                                              int m0, int n0) {
+    constexpr int SPITCH = 36;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WM, wn = wave / WM;
+    float* stage = stage_base + wave * 32 * SPITCH;
+    const int g = lane >> 5, li = lane & 31;
+    const int er = lane >> 2, ec = (lane & 3) * 8;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int col0 = n0 + (wn * TN + j) * 32 + ec;
+        float csum[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) csum[e] = 0.f;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) stage[acc_row(r, g) * SPITCH + li] = acc[i][j][r];
+            // the block is private to the wave: LDS operations of one wave complete in order
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int pass = 0; pass < 2; ++pass) {
+                const int rr = er + 16 * pass;
+                const int row = m0 + (wm * TM + i) * 32 + rr;
+                float v[8];
+                float4 v0 = *reinterpret_cast<const float4*>(stage + rr * SPITCH + ec);
+                float4 v1 = *reinterpret_cast<const float4*>(stage + rr * SPITCH + ec + 4);
+                v[0] = v0.x; v[1] = v0.y; v[2] = v0.z; v[3] = v0.w;
+                v[4] = v1.x; v[5] = v1.y; v[6] = v1.z; v[7] = v1.w;
+                if (row < a.M && col0 < a.N) {
+                    if (a.nsplit > 1) {
+                        float* dst = a.partial + ((long)blockIdx.z * a.M + row) * a.N + col0;
+                        *reinterpret_cast<float4*>(dst) = v0;
+                        *reinterpret_cast<float4*>(dst + 4) = v1;
+                    } else {
+                        epilogue_vec8<T>(a, row, col0, v);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) csum[e] += v[e];
+                    }
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (a.nsplit == 1 && a.colsum) {
+            // lanes with equal (lane & 3) hold the same columns
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float s = csum[e];
+                s += __shfl_xor(s, 4, 64);
+                s += __shfl_xor(s, 8, 64);
+                s += __shfl_xor(s, 16, 64);
+                s += __shfl_xor(s, 32, 64);
+                csum[e] = s;
+            }
+            if (lane < 4 && col0 < a.N) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) atomicAdd(a.colsum + col0 + e, csum[e]);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// 16-bit kernel with direct global->LDS loads (global_load_lds_dwordx4) and a STAGES-deep ring of
+// LDS tiles.  A wave instruction writes 64 consecutive 16-byte chunks of LDS, so the XOR swizzle of the
+// tile layout is applied on the global side: the lane that fills LDS chunk (row, pc) loads the global
+// chunk (row, pc ^ swz(row)).  Chunks outside the matrix are loaded from a zero buffer so that every
+// lane issues every load and the per-tile vmcnt accounting is exact.  The loads are inline asm: the
+// compiler does not see them as LDS writes (it would otherwise force vmcnt(0) before every ds_read),
+// and the kernel waits with explicit s_waitcnt vmcnt(n) + s_barrier once per k-tile.
+// ---------------------------------------------------------------------------------------------
+__device__ __attribute__((aligned(16))) unsigned int g_zero_chunk[4] = {0u, 0u, 0u, 0u};
+
+__device__ __forceinline__ void dma16(const void* gptr, const void* lds_wave_base) {
+    unsigned lds = (unsigned)(unsigned long)(__attribute__((address_space(3))) const void*)lds_wave_base;
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+                 :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory");
+}
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N <= 63, "vmcnt immediate is 6 bits");
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
+template <typename T, int ROWS, int COLS, int NT> struct TileDma {
+    static constexpr int CPR = COLS / 8;
+    static constexpr int TOTAL = ROWS * CPR;
+    static constexpr int N = TOTAL / NT;
+    static_assert(TOTAL % NT == 0 && NT % 64 == 0, "tile must split evenly over the waves");
+    // issues the N loads of this thread for the tile whose first element is (r0, c0)
+    static __device__ __forceinline__ void issue(T* lds, const T* __restrict__ base, long ld, int r0, int c0,
+                                                 int rmax, int cmax, int tid) {
+        const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int p0 = (i * (NT / 64) + wave) * 64;
+            const int p = p0 + lane;
+            const int row = p / CPR, pc = p % CPR;
+            const int lc = pc ^ swz16<COLS>(row);
+            const int gr = r0 + row, gc = c0 + lc * 8;
+            const void* src = (gr < rmax && gc < cmax) ? (const void*)(base + (long)gr * ld + gc)
+                                                       : (const void*)g_zero_chunk;
+            dma16(src, lds + p0 * 8);
+        }
+    }
+};
+
+template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN, int STAGES>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_dma_kernel(GemmArgs a) {
+    typedef Elem<T> E;
+    static_assert(sizeof(T) == 2, "the direct-to-LDS kernel is for fp16 / bf16");
+    constexpr int NT = WM * WN * 64;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int AR = AKM ? BM : BK, AC = AKM ? BK : BM;
+    constexpr int BR = BKM ? BN : BK, BC = BKM ? BK : BN;
+    constexpr int A_ELEMS = AR * AC, B_ELEMS = BR * BC;
+    constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
+    typedef TileDma<T, AR, AC, NT> DA;
+    typedef TileDma<T, BR, BC, NT> DB;
+    constexpr int NLOAD = DA::N + DB::N;                 // DMA instructions per thread per k-tile
+    static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
+    constexpr int TILE_BYTES = STAGES * STAGE_ELEMS * 2;
+    constexpr int EPI_BYTES = WM * WN * 32 * 36 * 4;
+    constexpr int SMEM_BYTES = TILE_BYTES > EPI_BYTES ? TILE_BYTES : EPI_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
+    T* tiles = reinterpret_cast<T*>(smem);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WM, wn = wave / WM;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int kbeg = blockIdx.z * a.kper;
+    const int kend = min(a.K, kbeg + a.kper);
+    const T* A = reinterpret_cast<const T*>(a.A);
+    const T* B = reinterpret_cast<const T*>(a.B);
+
+    auto issue = [&](int kt, int stage) {
+        T* sA = tiles + stage * STAGE_ELEMS;
+        T* sB = sA + A_ELEMS;
+        const int k0 = kbeg + kt * BK;
+        if constexpr (AKM) DA::issue(sA, A, a.lda, m0, k0, a.M, kend, tid);
+        else DA::issue(sA, A, a.lda, k0, m0, kend, a.M, tid);
+        if constexpr (BKM) DB::issue(sB, B, a.ldb, n0, k0, a.N, kend, tid);
+        else DB::issue(sB, B, a.ldb, k0, n0, kend, a.N, tid);
+    };
+
+    float16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int nk = (kend - kbeg + BK - 1) / BK;
+    // prologue: tiles 0 .. STAGES-2 in flight (tiles past the end load zeros; keeps the counts uniform)
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) issue(s, s);
+
+    for (int kt = 0; kt < nk; ++kt) {
+        // tile kt has landed once at most the loads of the STAGES-2 younger tiles are outstanding
+        wait_vmcnt<NLOAD * (STAGES - 2)>();
+        __builtin_amdgcn_s_barrier();   // every wave's part of tile kt is in LDS; tile kt-1 is no longer read
+        asm volatile("" ::: "memory");
+        issue(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);   // refills the buffer tile kt-1 used
+        const T* tA = tiles + (kt % STAGES) * STAGE_ELEMS;
+        const T* tB = tA + A_ELEMS;
+#pragma unroll
+        for (int ks = 0; ks < BK / E::KSTEP; ++ks) {
+            typename E::opnd_t fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                int mb = (wm * TM + i) * 32;
+                if constexpr (AKM) fa[i] = fetch_km<T, AC>(tA, mb + (lane & 31), ks * E::KSTEP, lane);
+                else fa[i] = fetch_tr<T, AC, false>(tA, ks * E::KSTEP, mb, lane);
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                int nb = (wn * TN + j) * 32;
+                if constexpr (BKM) fb[j] = fetch_km<T, BC>(tB, nb + (lane & 31), ks * E::KSTEP, lane);
+                else fb[j] = fetch_tr<T, BC, false>(tB, ks * E::KSTEP, nb, lane);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = E::mfma(fa[i], fb[j], acc[i][j]);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave's LDS reads of tile kt are done
+    }
+    // drain the zero-tile loads still in flight before LDS is reused for the epilogue
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
+}
+
 template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(GemmArgs a) {
     typedef Elem<T> E;
@@ -215,96 +416,54 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(GemmArgs a) {
         __syncthreads();
     }
 
-    // Epilogue.  Each wave transposes one 32x32 accumulator block at a time through its own LDS
-    // staging block so that a lane ends up with 8 consecutive columns of a row: 16-byte stores,
-    // and a vector epilogue.  Lane -> (row = lane / 4 + 16 * pass, columns 8 * (lane % 4) .. + 7).
-    float* stage = reinterpret_cast<float*>(smem) + wave * 32 * SPITCH;
-    const int g = lane >> 5, li = lane & 31;
-    const int er = lane >> 2, ec = (lane & 3) * 8;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int col0 = n0 + (wn * TN + j) * 32 + ec;
-        float csum[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) csum[e] = 0.f;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) stage[acc_row(r, g) * SPITCH + li] = acc[i][j][r];
-            // the block is private to the wave: LDS operations of one wave complete in order
-            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int pass = 0; pass < 2; ++pass) {
-                const int rr = er + 16 * pass;
-                const int row = m0 + (wm * TM + i) * 32 + rr;
-                float v[8];
-                float4 v0 = *reinterpret_cast<const float4*>(stage + rr * SPITCH + ec);
-                float4 v1 = *reinterpret_cast<const float4*>(stage + rr * SPITCH + ec + 4);
-                v[0] = v0.x; v[1] = v0.y; v[2] = v0.z; v[3] = v0.w;
-                v[4] = v1.x; v[5] = v1.y; v[6] = v1.z; v[7] = v1.w;
-                if (row < a.M && col0 < a.N) {
-                    if (a.nsplit > 1) {
-                        float* dst = a.partial + ((long)blockIdx.z * a.M + row) * a.N + col0;
-                        *reinterpret_cast<float4*>(dst) = v0;
-                        *reinterpret_cast<float4*>(dst + 4) = v1;
-                    } else {
-                        epilogue_vec8<T>(a, row, col0, v);
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) csum[e] += v[e];
-                    }
-                }
-            }
-            __builtin_amdgcn_wave_barrier();
-        }
-        if (a.nsplit == 1 && a.colsum) {
-            // lanes with equal (lane & 3) hold the same columns
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float s = csum[e];
-                s += __shfl_xor(s, 4, 64);
-                s += __shfl_xor(s, 8, 64);
-                s += __shfl_xor(s, 16, 64);
-                s += __shfl_xor(s, 32, 64);
-                csum[e] = s;
-            }
-            if (lane < 4 && col0 < a.N) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) atomicAdd(a.colsum + col0 + e, csum[e]);
-            }
-        }
-    }
+    gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
 }
 
-// Sums the split-K partials and applies the epilogue.  One thread per 8 columns and rows_per_block
-// rows per block, so the column sums cost 8 atomics per thread.
+// Sums the split-K partials and applies the epilogue.  A block of 256 threads covers 256 columns
+// (32 threads x 8 columns) by 32 rows (8 row lanes x 4 rows); column sums are combined across the
+// row lanes in LDS so that they cost one atomic per column per block.
 template <typename T>
-__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmArgs a, int rows_per_block) {
-    const int col0 = (blockIdx.x * 256 + threadIdx.x) * 8;
-    if (col0 >= a.N) return;
-    const int r0 = blockIdx.y * rows_per_block;
-    const int r1 = min(a.M, r0 + rows_per_block);
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmArgs a) {
+    __shared__ float cs[8][256];
+    const int cl = threadIdx.x & 31, rl = threadIdx.x >> 5;
+    const int col0 = (blockIdx.x * 32 + cl) * 8;
+    const int rbase = blockIdx.y * 32;
     float csum[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) csum[e] = 0.f;
-    for (int row = r0; row < r1; ++row) {
-        float v[8];
+    if (col0 < a.N) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = 0.f;
-        for (int z = 0; z < a.nsplit; ++z) {
-            const float* src = a.partial + ((long)z * a.M + row) * a.N + col0;
-            float4 p0 = *reinterpret_cast<const float4*>(src);
-            float4 p1 = *reinterpret_cast<const float4*>(src + 4);
-            v[0] += p0.x; v[1] += p0.y; v[2] += p0.z; v[3] += p0.w;
-            v[4] += p1.x; v[5] += p1.y; v[6] += p1.z; v[7] += p1.w;
+        for (int rr = 0; rr < 4; ++rr) {
+            const int row = rbase + rr * 8 + rl;
+            if (row < a.M) {
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = 0.f;
+                for (int z = 0; z < a.nsplit; ++z) {
+                    const float* src = a.partial + ((long)z * a.M + row) * a.N + col0;
+                    float4 p0 = *reinterpret_cast<const float4*>(src);
+                    float4 p1 = *reinterpret_cast<const float4*>(src + 4);
+                    v[0] += p0.x; v[1] += p0.y; v[2] += p0.z; v[3] += p0.w;
+                    v[4] += p1.x; v[5] += p1.y; v[6] += p1.z; v[7] += p1.w;
+                }
+                epilogue_vec8<T>(a, row, col0, v);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) csum[e] += v[e];
+            }
         }
-        epilogue_vec8<T>(a, row, col0, v);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) csum[e] += v[e];
     }
     if (a.colsum) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) atomicAdd(a.colsum + col0 + e, csum[e]);
+        for (int e = 0; e < 8; ++e) cs[rl][cl * 8 + e] = csum[e];
+        __syncthreads();
+        const int c = threadIdx.x;
+        const int col = blockIdx.x * 256 + c;
+        if (col < a.N) {
+            float t = 0.f;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) t += cs[r][c];
+            atomicAdd(a.colsum + col, t);
+        }
     }
 }
 
@@ -313,43 +472,88 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmArgs a, int
 // ---------------------------------------------------------------------------------------------
 static constexpr int kNumCU = 256;  // MI355X
 
+// Tile configurations of the 16-bit direct-to-LDS kernel (4 waves, 2 x 2).  Index 0 is the
+// register-staged kernel (fp32, and the reference point for the others in tests).
+struct TileCfg { int bm, bn, bk, stages; };
+static const TileCfg kCfgs[] = {
+    {64, 64, 64, 2},     // 0: register-staged kernel's 16-bit tile (fp32 uses 64 x 64 x 16)
+    {256, 256, 64, 2},   // 1
+    {256, 128, 64, 3},   // 2
+    {128, 256, 64, 3},   // 3
+    {128, 128, 64, 4},   // 4
+    {128, 128, 64, 2},   // 5
+    {128, 64, 64, 4},    // 6
+    {64, 128, 64, 4},    // 7
+    {64, 64, 64, 4},     // 8
+};
+static constexpr int kNumCfgs = (int)(sizeof(kCfgs) / sizeof(kCfgs[0]));
+
 struct GemmPlan {
-    int cfg;      // 0: 128x128 tile, 1: 64x64 tile
+    int cfg;
     int nsplit;
     int kper;
     int gx, gy;
 };
 
-static GemmPlan plan_gemm(const tp_gemm_desc* d) {
-    GemmPlan p;
-    const int bk = (d->dtype == TP_F32) ? 16 : 64;  // k granularity shared by both tile configs
-    long t128 = (long)((d->M + 127) / 128) * ((d->N + 127) / 128);
-    long t64 = (long)((d->M + 63) / 64) * ((d->N + 63) / 64);
-    if (d->dtype != TP_F32 && t128 >= kNumCU) {
-        p.cfg = 0;
-        p.gx = (d->N + 127) / 128; p.gy = (d->M + 127) / 128;
-    } else {
-        p.cfg = 1;
-        p.gx = (d->N + 63) / 64; p.gy = (d->M + 63) / 64;
-    }
-    long tiles = (long)p.gx * p.gy;
-    int nsplit = 1;
-    // split K until about two workgroups per CU exist, keeping at least 4 k-tiles per split;
-    // read-modify-write and scatter epilogues run in the reduce kernel just the same.
-    if (tiles < 2 * kNumCU) {
-        long want = (2 * kNumCU + tiles - 1) / tiles;
-        long kt = (d->K + bk - 1) / bk;
-        long maxs = kt / 4 > 0 ? kt / 4 : 1;
-        nsplit = (int)(want < maxs ? want : maxs);
-        if (nsplit > 16) nsplit = 16;
-        if (nsplit < 1) nsplit = 1;
-    }
-    (void)t64;
+static void finish_plan(const tp_gemm_desc* d, GemmPlan& p, int bk, int nsplit) {
     long kt = (d->K + bk - 1) / bk;
+    if (nsplit > kt) nsplit = (int)kt;
+    if (nsplit < 1) nsplit = 1;
     long per = (kt + nsplit - 1) / nsplit;
     p.kper = (int)(per * bk);
     p.nsplit = (int)((d->K + p.kper - 1) / p.kper);
-    if (p.nsplit < 1) { p.nsplit = 1; p.kper = bk; }
+}
+
+static GemmPlan plan_gemm(const tp_gemm_desc* d) {
+    GemmPlan p;
+    if (d->dtype == TP_F32) {
+        p.cfg = 0;
+        p.gx = (d->N + 63) / 64; p.gy = (d->M + 63) / 64;
+        long tiles = (long)p.gx * p.gy;
+        int nsplit = 1;
+        if (tiles < 2 * kNumCU) {
+            long want = (2 * kNumCU + tiles - 1) / tiles;
+            long kt = (d->K + 15) / 16;
+            long maxs = kt / 8 > 0 ? kt / 8 : 1;
+            nsplit = (int)(want < maxs ? want : maxs);
+            if (nsplit > 16) nsplit = 16;
+        }
+        finish_plan(d, p, 16, nsplit);
+        return p;
+    }
+    // reserved: bits 0-7 force a tile configuration (1-based index + 1 so that 0 means automatic),
+    // bits 8-15 force the number of k splits.  For tuning and tests.
+    int forced_cfg = (d->reserved & 0xff) - 1;
+    int forced_split = (d->reserved >> 8) & 0xff;
+    // Measured on MI355X: the 128 x 128 x 64 two-stage tile (two workgroups per CU) wins whenever its
+    // tile count comes near the CU count, 64 x 64 x 64 otherwise; k is split to reach about two
+    // workgroups per CU as long as every split keeps at least 2048 (small tiles) / 1024 (large) of k.
+    const long t128 = (long)((d->M + 127) / 128) * ((d->N + 127) / 128);
+    const long t64 = (long)((d->M + 63) / 64) * ((d->N + 63) / 64);
+    int cfg, ns = 1;
+    if (t128 >= 96) {
+        cfg = 5;
+        if (t128 < 224) {
+            ns = (int)(448 / t128);
+            int maxs = d->K / 1024;
+            if (ns > maxs) ns = maxs;
+        }
+    } else {
+        cfg = 8;
+        if (t64 < 384) {
+            ns = (int)(512 / t64);
+            int maxs = d->K / 2048;
+            if (ns > maxs) ns = maxs;
+        }
+    }
+    if (ns < 1) ns = 1;
+    if (ns > 16) ns = 16;
+    if (forced_cfg >= 0 && forced_cfg < kNumCfgs) cfg = forced_cfg;
+    if (forced_split) ns = forced_split;
+    p.cfg = cfg;
+    p.gx = (d->N + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn;
+    p.gy = (d->M + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm;
+    finish_plan(d, p, kCfgs[cfg].bk, ns);
     return p;
 }
 
@@ -359,8 +563,17 @@ static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
     if constexpr (sizeof(T) == 4) {
         gemm_kernel<T, AKM, BKM, 64, 64, 16, 2, 2><<<grid, 256, 0, s>>>(a);
     } else {
-        if (p.cfg == 0) gemm_kernel<T, AKM, BKM, 128, 128, 32, 2, 2><<<grid, 256, 0, s>>>(a);
-        else gemm_kernel<T, AKM, BKM, 64, 64, 64, 2, 2><<<grid, 256, 0, s>>>(a);
+        switch (p.cfg) {
+        case 1: gemm_dma_kernel<T, AKM, BKM, 256, 256, 64, 2, 2, 2><<<grid, 256, 0, s>>>(a); break;
+        case 2: gemm_dma_kernel<T, AKM, BKM, 256, 128, 64, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
+        case 3: gemm_dma_kernel<T, AKM, BKM, 128, 256, 64, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
+        case 4: gemm_dma_kernel<T, AKM, BKM, 128, 128, 64, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
+        case 5: gemm_dma_kernel<T, AKM, BKM, 128, 128, 64, 2, 2, 2><<<grid, 256, 0, s>>>(a); break;
+        case 6: gemm_dma_kernel<T, AKM, BKM, 128, 64, 64, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
+        case 7: gemm_dma_kernel<T, AKM, BKM, 64, 128, 64, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
+        case 8: gemm_dma_kernel<T, AKM, BKM, 64, 64, 64, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
+        default: gemm_kernel<T, AKM, BKM, 64, 64, 64, 2, 2><<<grid, 256, 0, s>>>(a); break;
+        }
     }
 }
 
@@ -372,9 +585,8 @@ static void launch_gemm(const tp_gemm_desc* d, const GemmPlan& p, const GemmArgs
     default: launch_cfg<T, false, false>(p, a, s); break;
     }
     if (p.nsplit > 1) {
-        int rpb = 8;
-        dim3 grid((d->N / 8 + 255) / 256, (d->M + rpb - 1) / rpb);
-        gemm_splitk_reduce_kernel<T><<<grid, 256, 0, s>>>(a, rpb);
+        dim3 grid((d->N + 255) / 256, (d->M + 31) / 32);
+        gemm_splitk_reduce_kernel<T><<<grid, 256, 0, s>>>(a);
     }
 }
 

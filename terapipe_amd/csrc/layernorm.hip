@@ -169,12 +169,61 @@ __global__ __launch_bounds__(1024) void ln_bwd_kernel(const T* __restrict__ dy, 
 #pragma unroll
             for (int e = 0; e < CH; ++e) {
                 long col = (long)c * CH + e;
-                atomicAdd(dgamma + col, a_dg[i][e]);
-                atomicAdd(dbeta + col, a_db[i][e]);
+                if (dgamma) {
+                    atomicAdd(dgamma + col, a_dg[i][e]);
+                    atomicAdd(dbeta + col, a_db[i][e]);
+                }
                 if (cs_dres && dres) atomicAdd(cs_dres + col, a_dr[i][e]);
                 if (cs_dx) atomicAdd(cs_dx + col, a_dx[i][e]);
             }
         }
+    }
+}
+
+// dgamma / dbeta over a block of rows: 256 threads = 32 column chunks (8 columns each) x 8 row lanes,
+// 64 rows per block, row lanes combined in LDS, one atomic per column per block.
+template <typename T>
+__global__ __launch_bounds__(256) void ln_param_grads_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                                             const float* __restrict__ mean,
+                                                             const float* __restrict__ rstd, float* dgamma,
+                                                             float* dbeta, int M, int E) {
+    __shared__ float sg[8][256], sb[8][256];
+    const int cl = threadIdx.x & 31, rl = threadIdx.x >> 5;
+    const int col0 = (blockIdx.x * 32 + cl) * 8;
+    const int rbase = blockIdx.y * 64;
+    float ag[8], ab[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { ag[e] = 0.f; ab[e] = 0.f; }
+    if (col0 < E) {
+        for (int rr = 0; rr < 8; ++rr) {
+            const int row = rbase + rr * 8 + rl;
+            if (row < M) {
+                const float mu = mean[row], rs = rstd[row];
+                float d[8], xv[8];
+                if constexpr (sizeof(T) == 2) {
+                    load_chunk<T>(dy + (long)row * E + col0, d);
+                    load_chunk<T>(x + (long)row * E + col0, xv);
+                } else {
+                    load_chunk<T>(dy + (long)row * E + col0, d);
+                    load_chunk<T>(dy + (long)row * E + col0 + 4, d + 4);
+                    load_chunk<T>(x + (long)row * E + col0, xv);
+                    load_chunk<T>(x + (long)row * E + col0 + 4, xv + 4);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { ag[e] += d[e] * (xv[e] - mu) * rs; ab[e] += d[e]; }
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { sg[rl][cl * 8 + e] = ag[e]; sb[rl][cl * 8 + e] = ab[e]; }
+    __syncthreads();
+    const int c = threadIdx.x, col = blockIdx.x * 256 + c;
+    if (col < E) {
+        float tg = 0.f, tb = 0.f;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) { tg += sg[r][c]; tb += sb[r][c]; }
+        atomicAdd(dgamma + col, tg);
+        atomicAdd(dbeta + col, tb);
     }
 }
 
@@ -243,14 +292,17 @@ extern "C" int tp_layernorm_bwd(const void* dy, const void* x, const float* mean
                                 float* dbeta_acc, float* colsum_dres_acc, float* colsum_dx_acc, int M, int E,
                                 int dtype, void* stream) {
     using namespace tp;
-    if (!dy || !x || !mean || !rstd || !gamma || !dx || !dgamma_acc || !dbeta_acc) { set_error("tp_layernorm_bwd: null pointer"); return TP_ERR_ARG; }
+    if (!dy || !x || !mean || !rstd || !gamma || !dx) { set_error("tp_layernorm_bwd: null pointer"); return TP_ERR_ARG; }
+    if ((dgamma_acc == nullptr) != (dbeta_acc == nullptr)) { set_error("tp_layernorm_bwd: dgamma_acc and dbeta_acc must both be given or both be NULL"); return TP_ERR_ARG; }
     if (M <= 0) { set_error("tp_layernorm_bwd: M=%d", M); return TP_ERR_ARG; }
     if (dtype < TP_F32 || dtype > TP_BF16) { set_error("tp_layernorm_bwd: bad dtype %d", dtype); return TP_ERR_ARG; }
     if (((uintptr_t)dy | (uintptr_t)x | (uintptr_t)gamma | (uintptr_t)dres | (uintptr_t)dx) & 15) { set_error("tp_layernorm_bwd: pointers must be 16-byte aligned"); return TP_ERR_ARG; }
     int nt, maxc;
     int rc = ln_geometry(E, dtype, &nt, &maxc);
     if (rc != TP_OK) return rc;
-    int grid = M < 128 ? M : 128;
+    // with accumulators every block ends in E atomics per array, so fewer blocks sweep more rows each;
+    // without them one block per row
+    int grid = (dgamma_acc || colsum_dres_acc || colsum_dx_acc) ? (M < 128 ? M : 128) : M;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     switch (dtype) {
     case TP_F32: launch_ln_bwd<float>(maxc, nt, grid, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc, M, E, s); break;
@@ -258,4 +310,21 @@ extern "C" int tp_layernorm_bwd(const void* dy, const void* x, const float* mean
     default: launch_ln_bwd<bf16>(maxc, nt, grid, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc, M, E, s); break;
     }
     return check_launch("tp_layernorm_bwd");
+}
+
+extern "C" int tp_ln_param_grads(const void* dy, const void* x, const float* mean, const float* rstd,
+                                 float* dgamma_acc, float* dbeta_acc, int M, int E, int dtype, void* stream) {
+    using namespace tp;
+    if (!dy || !x || !mean || !rstd || !dgamma_acc || !dbeta_acc) { set_error("tp_ln_param_grads: null pointer"); return TP_ERR_ARG; }
+    if (M <= 0 || E <= 0 || E % 8) { set_error("tp_ln_param_grads: M=%d, E=%d (E must be a multiple of 8)", M, E); return TP_ERR_ARG; }
+    if (dtype < TP_F32 || dtype > TP_BF16) { set_error("tp_ln_param_grads: bad dtype %d", dtype); return TP_ERR_ARG; }
+    if (((uintptr_t)dy | (uintptr_t)x) & 15) { set_error("tp_ln_param_grads: pointers must be 16-byte aligned"); return TP_ERR_ARG; }
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    dim3 grid((E + 255) / 256, (M + 63) / 64);
+    switch (dtype) {
+    case TP_F32: ln_param_grads_kernel<float><<<grid, 256, 0, s>>>((const float*)dy, (const float*)x, mean, rstd, dgamma_acc, dbeta_acc, M, E); break;
+    case TP_F16: ln_param_grads_kernel<f16><<<grid, 256, 0, s>>>((const f16*)dy, (const f16*)x, mean, rstd, dgamma_acc, dbeta_acc, M, E); break;
+    default: ln_param_grads_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)dy, (const bf16*)x, mean, rstd, dgamma_acc, dbeta_acc, M, E); break;
+    }
+    return check_launch("tp_ln_param_grads");
 }

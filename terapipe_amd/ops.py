@@ -95,12 +95,12 @@ class Workspace:
         return buf
 
 
-def layernorm_fwd(x2d, gamma, beta, eps=1e-5):
+def layernorm_fwd(x2d, gamma, beta, eps=1e-5, out=None, mean=None, rstd=None):
     _require_cuda(x2d, gamma, beta)
     M, E = x2d.shape
-    y = torch.empty_like(x2d)
-    mean = torch.empty(M, dtype=torch.float32, device=x2d.device)
-    rstd = torch.empty(M, dtype=torch.float32, device=x2d.device)
+    y = torch.empty_like(x2d) if out is None else out
+    mean = torch.empty(M, dtype=torch.float32, device=x2d.device) if mean is None else mean
+    rstd = torch.empty(M, dtype=torch.float32, device=x2d.device) if rstd is None else rstd
     lib = _lib.load()
     with _timed("layernorm_fwd", (M, E)):
         _lib.check(lib.tp_layernorm_fwd(_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps,
@@ -109,10 +109,12 @@ def layernorm_fwd(x2d, gamma, beta, eps=1e-5):
 
 
 def layernorm_bwd(dy, x2d, mean, rstd, gamma, dres, dgamma_acc, dbeta_acc, colsum_dres_acc=None,
-                  colsum_dx_acc=None):
+                  colsum_dx_acc=None, out=None):
+    """dgamma_acc / dbeta_acc may be None: then only dx is computed (the parameter gradients are left
+    to ln_param_grads over all rows)."""
     _require_cuda(dy, x2d, gamma)
     M, E = x2d.shape
-    dx = torch.empty_like(x2d)
+    dx = torch.empty_like(x2d) if out is None else out
     lib = _lib.load()
     with _timed("layernorm_bwd", (M, E)):
         _lib.check(lib.tp_layernorm_bwd(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx),
@@ -122,9 +124,10 @@ def layernorm_bwd(dy, x2d, mean, rstd, gamma, dres, dgamma_acc, dbeta_acc, colsu
 
 
 def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=None, aux=None, aux_out=None,
-         colsum_acc=None, qkv=None):
+         colsum_acc=None, qkv=None, tile_cfg=None, ksplit=None):
     """Runs one GEMM.  A, B, C, residual, aux are 2-D row-major tensors (stride(1) == 1).
-    qkv = dict(q, k_cache, v_cache, batch, heads, head_dim, cache_len, cache_rows, q_scale)."""
+    qkv = dict(q, k_cache, v_cache, batch, heads, head_dim, cache_len, cache_rows, q_scale).
+    tile_cfg / ksplit force a tile configuration / k-split count (tuning and tests); default automatic."""
     _require_cuda(A, B, C)
     d = GemmDesc()
     d.op, d.dtype, d.epilogue = op, tp_dtype(A.dtype), epilogue
@@ -145,6 +148,8 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
         d.q, d.k_cache, d.v_cache = qkv["q"].data_ptr(), qkv["k_cache"].data_ptr(), qkv["v_cache"].data_ptr()
         d.batch, d.heads, d.head_dim = qkv["batch"], qkv["heads"], qkv["head_dim"]
         d.cache_len, d.cache_rows, d.q_scale = qkv["cache_len"], qkv["cache_rows"], qkv["q_scale"]
+    if tile_cfg is not None or ksplit is not None:
+        d.reserved = ((tile_cfg + 1) if tile_cfg is not None else 0) | ((ksplit or 0) << 8)
     lib = _lib.load()
     need = lib.tp_gemm_workspace_bytes(ctypes.byref(d))
     ws = Workspace.get(need, A.device) if need else None
@@ -163,12 +168,13 @@ def _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len
     return d
 
 
-def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q_scale):
+def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q_scale, out=None, lse=None):
     """q [B*H, T, Dh] (pre-scaled); caches [B*H, L, Dh] with rows [0, cache_len+T) valid.
     Returns o [T, B, H*Dh] and lse [B*H, T]."""
     _require_cuda(q, k_cache, v_cache)
-    o = torch.empty(T, batch, heads * head_dim, dtype=q.dtype, device=q.device)
-    lse = torch.empty(batch * heads, T, dtype=torch.float32, device=q.device)
+    o = torch.empty(T, batch, heads * head_dim, dtype=q.dtype, device=q.device) if out is None else out
+    if lse is None:
+        lse = torch.empty(batch * heads, T, dtype=torch.float32, device=q.device)
     d = _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale)
     lib = _lib.load()
     need = lib.tp_attn_fwd_workspace_bytes(ctypes.byref(d))
@@ -180,10 +186,12 @@ def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q
 
 
 def attn_prefix_bwd(q, k_cache, v_cache, o, lse, d_o, dqkv, dk_cache, dv_cache, batch, heads, head_dim, T,
-                    cache_len, q_scale, accumulate_prefix, has_incoming, zero_slice_rows, colsum_dqkv_acc=None):
+                    cache_len, q_scale, accumulate_prefix, has_incoming, zero_slice_rows, colsum_dqkv_acc=None,
+                    delta=None):
     """Writes dqkv [T*B, 3*H*Dh]; updates rows [0, cache_len) of the gradient caches."""
     _require_cuda(q, k_cache, v_cache, d_o, dqkv)
-    delta = torch.empty(batch * heads, T, dtype=torch.float32, device=q.device)
+    if delta is None:
+        delta = torch.empty(batch * heads, T, dtype=torch.float32, device=q.device)
     d = _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale)
     d.d_o, d.delta, d.dqkv = d_o.data_ptr(), delta.data_ptr(), dqkv.data_ptr()
     d.dk_cache, d.dv_cache = _p(dk_cache), _p(dv_cache)
@@ -194,6 +202,16 @@ def attn_prefix_bwd(q, k_cache, v_cache, o, lse, d_o, dqkv, dk_cache, dv_cache, 
     with _timed("attn_bwd", (batch, heads, head_dim, T, cache_len)):
         _lib.check(lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()), "tp_attn_prefix_bwd")
     return dqkv
+
+
+def ln_param_grads(dy, x2d, mean, rstd, dgamma_acc, dbeta_acc):
+    """dgamma_acc[E] += sum_m dy * xhat, dbeta_acc[E] += sum_m dy over all M rows (fp32 accumulators)."""
+    _require_cuda(dy, x2d, dgamma_acc, dbeta_acc)
+    M, E = x2d.shape
+    lib = _lib.load()
+    with _timed("ln_param_grads", (M, E)):
+        _lib.check(lib.tp_ln_param_grads(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(dgamma_acc), _p(dbeta_acc), M, E,
+                                         tp_dtype(x2d.dtype), _stream()), "tp_ln_param_grads")
 
 
 def accum_cast(dst, src_f32, accumulate):

@@ -2,12 +2,12 @@
 ``TransformerLayers`` (terapipe.py:52-95) and ``TeraPipe`` (terapipe.py:219-271) with the reverse-order
 slice backward of ``TeraPipeBackwardPassHook`` (terapipe.py:154-212).
 
-``TeraPipe.forward`` runs the whole slice grid inside ONE autograd node.  Its backward walks the slices
-in reverse, hands dK/dV of the prefix rows from slice i+1 to slice i through persistent fp32 gradient
-caches (instead of a full-length clone per slice, reference transformer_models.py:188), and can defer
-the weight-gradient GEMMs to one GEMM per weight over all tokens (dW = dY_all^T X_all equals the sum
-over slices of dY_i^T X_i).  Pipeline send/recv, process groups and the optimizer are not part of
-this path.
+``TeraPipe.forward`` runs the whole slice grid inside ONE autograd node on buffers allocated once per
+runner.  Its backward walks the slices in reverse, hands dK/dV of the prefix rows from slice i+1 to
+slice i through persistent fp32 gradient caches (instead of a full-length clone per slice, reference
+transformer_models.py:188), and computes the parameter gradients once over all tokens at the end
+(dW = dY_all^T X_all equals the sum over slices of dY_i^T X_i).  Pipeline send/recv, process groups
+and the optimizer are not part of this path.
 """
 import numpy as np
 import torch
@@ -15,7 +15,7 @@ import torch.nn as nn
 
 from . import _layer_core as core
 from . import ops
-from ._lib import TP_EPI_STORE, TP_GEMM_TN
+from ._lib import TP_EPI_ACCUMULATE, TP_EPI_STORE, TP_GEMM_TN
 from .transformer_models import ModelParallelTransformerLayer, grid_slice_batch_and_sequence
 
 
@@ -70,105 +70,160 @@ class TransformerLayers(nn.Module):
         return fn((seq_len, batch_size, self.embedding_dim), device=device, dtype=self.dtype)
 
 
+class _StackBuffers:
+    """Per-runner device buffers, allocated once and reused by every step: for each batch slice and
+    layer the saved activations and the intermediate gradients of the WHOLE sequence, so that a slice
+    works on a row range of them (slice i of a [L, Bs, E] tensor is rows [P*Bs, (P+T)*Bs)), the K/V
+    caches, the fp32 (or cache-dtype) gradient caches, and the parameter-gradient accumulators."""
+
+    def __init__(self, runner, dtype, device):
+        layers = runner.layers
+        nl, E, F, H = layers.n_layers, layers.embedding_dim, layers.ffn_embedding_dim, layers.num_attention_heads
+        L, Dh = runner.seq_len, layers.embedding_dim // layers.num_attention_heads
+        self.dtype, self.device = dtype, device
+        gdt = torch.float32 if runner.fp32_grad_cache else dtype
+        kw = dict(dtype=dtype, device=device)
+        f32 = dict(dtype=torch.float32, device=device)
+        self.per_batch = []
+        for Bs in runner.batch_slices:
+            R = L * Bs
+            b = {}
+            b["x"] = [torch.empty(R, E, **kw) for _ in range(nl + 1)]      # x[l] input of layer l; x[nl] output
+            b["dx"] = [torch.empty(R, E, **kw) for _ in range(nl + 1)]     # gradient of the same
+            for name, width in (("xn", E), ("q", E), ("o", E), ("h", E), ("hn", E), ("a", F),
+                                ("dz1", F), ("dhn", E), ("dh", E), ("dqkv", 3 * E), ("dxn", E)):
+                b[name] = [torch.empty(R, width, **kw) for _ in range(nl)]
+            b["z"] = [torch.empty(R, F, **kw) if layers.layers[l].activation == "gelu" else None for l in range(nl)]
+            for name in ("mean1", "rstd1", "mean2", "rstd2"):
+                b[name] = [torch.empty(R, **f32) for _ in range(nl)]
+            b["lse"] = [torch.empty(R * H, **f32) for _ in range(nl)]
+            b["d_o"] = torch.empty(max(runner.seq_slices) * Bs, E, **kw)
+            b["delta"] = torch.empty(max(runner.seq_slices) * Bs * H, **f32)
+            # zero-filled once: rows beyond the current slice are read only under the causal mask, but
+            # they must hold finite values (reference create_attn_cache zero-fills, transformer_models.py:257-261)
+            b["cache"] = [torch.zeros(Bs * H, L, Dh, **kw) for _ in range(2 * nl)]
+            b["gcache"] = [torch.empty(Bs * H, L, Dh, dtype=gdt, device=device) for _ in range(2 * nl)]
+            self.per_batch.append(b)
+        self.small = torch.zeros(nl, core.small_acc_numel(E, F), **f32)
+        self.small_views = [core.small_acc_views(self.small[l], E, F) for l in range(nl)]
+
+
 class _TeraPipeFunction(torch.autograd.Function):
     """forward: every (batch slice, sequence slice) through the whole layer stack, slice-major.
-    backward: reverse-order slices (terapipe.py:182-191 of the reference)."""
+    backward: reverse-order slices (terapipe.py:182-191 of the reference), then one weight-gradient
+    GEMM per weight and one reduction per vector parameter over all tokens."""
 
     @staticmethod
     def forward(ctx, runner, inputs, *flat_params):
         layers = runner.layers
-        n_layers = layers.n_layers
-        heads = layers.num_attention_heads
-        ws = [dict(zip(core.PARAM_NAMES, flat_params[12 * i:12 * i + 12])) for i in range(n_layers)]
+        nl, heads = layers.n_layers, layers.num_attention_heads
+        E, H = layers.embedding_dim, heads
+        ws = [dict(zip(core.PARAM_NAMES, flat_params[12 * i:12 * i + 12])) for i in range(nl)]
         act = [l.activation for l in layers.layers]
-        need_state = any(ctx.needs_input_grad)
-        xs = grid_slice_batch_and_sequence(inputs, runner.batch_slices, runner.seq_slices, requires_grad=False,
-                                           batch_dim=runner.batch_dim, sequence_dim=runner.sequence_dim)
+        bufs = runner._stack_buffers(inputs.dtype, inputs.device)
         nb, ns = len(runner.batch_slices), len(runner.seq_slices)
         states = np.empty((nb, ns), dtype="O")
-        outs = np.empty((nb, ns), dtype="O")
-        caches = []
+        b0 = 0
         for b in range(nb):
-            cache = layers.create_cache(runner.batch_slices[b], runner.seq_len)      # terapipe.py:251
-            cache_len = 0
+            Bs = runner.batch_slices[b]
+            pb = bufs.per_batch[b]
+            # the batch slice as [L*Bs, E] rows (t, b_local): a copy, as grid_slice_batch_and_sequence makes
+            pb["x"][0].view(runner.seq_len, Bs, E).copy_(inputs[:, b0:b0 + Bs, :])
+            cache = pb["cache"]
+            P = 0
             for i in range(ns):
-                x = xs[b, i]
+                T = runner.seq_slices[i]
+                r0, r1 = P * Bs, (P + T) * Bs
                 sts = []
-                for l in range(n_layers):
-                    x, st = core.layer_fwd(ws[l], x, heads, cache[2 * l], cache[2 * l + 1], cache_len, act[l],
-                                           need_state=need_state)
+                for l in range(nl):
+                    bf = core.Bufs(xn=pb["xn"][l][r0:r1], mean1=pb["mean1"][l][r0:r1], rstd1=pb["rstd1"][l][r0:r1],
+                                   q=pb["q"][l][r0:r1].view(Bs * H, T, E // H), o=pb["o"][l][r0:r1].view(T, Bs, E),
+                                   lse=pb["lse"][l][r0 * H:r1 * H].view(Bs * H, T), h=pb["h"][l][r0:r1],
+                                   mean2=pb["mean2"][l][r0:r1], rstd2=pb["rstd2"][l][r0:r1], hn=pb["hn"][l][r0:r1],
+                                   a=pb["a"][l][r0:r1], z=None if pb["z"][l] is None else pb["z"][l][r0:r1],
+                                   out=pb["x"][l + 1][r0:r1])
+                    _, st = core.layer_fwd(ws[l], pb["x"][l][r0:r1].view(T, Bs, E), heads, cache[2 * l],
+                                           cache[2 * l + 1], P, act[l], need_state=True, buf=bf)
                     sts.append(st)
                 states[b, i] = sts
-                outs[b, i] = x
-                cache_len += runner.seq_slices[i]                                    # terapipe.py:264
-            caches.append(cache)
-        runner.last_caches = caches
+                P += T                                                               # terapipe.py:264
+            b0 += Bs
+        runner.last_caches = [pb["cache"] for pb in bufs.per_batch]
         if runner.keep_states:
             runner.last_states = states.copy()
-        y = torch.cat([torch.cat(list(outs[b]), dim=runner.sequence_dim) for b in range(nb)], dim=runner.batch_dim)
-        ctx.runner, ctx.ws, ctx.act, ctx.states = runner, ws, act, states
-        ctx.in_shape = inputs.shape
+        if nb == 1:
+            y = bufs.per_batch[0]["x"][nl].view(runner.seq_len, runner.batch_slices[0], E).clone()
+        else:
+            y = torch.cat([pb["x"][nl].view(runner.seq_len, Bs, E)
+                           for pb, Bs in zip(bufs.per_batch, runner.batch_slices)], dim=1)
+        ctx.runner, ctx.ws, ctx.act, ctx.states, ctx.bufs = runner, ws, act, states, bufs
         return y
 
     @staticmethod
     def backward(ctx, grad_y):
-        runner, ws, act, states = ctx.runner, ctx.ws, ctx.act, ctx.states
+        runner, ws, act, states, bufs = ctx.runner, ctx.ws, ctx.act, ctx.states, ctx.bufs
         layers = runner.layers
-        n_layers, heads = layers.n_layers, layers.num_attention_heads
-        E, F = layers.embedding_dim, layers.ffn_embedding_dim
-        Dh = E // heads
-        dev, dt = grad_y.device, grad_y.dtype
+        nl, heads = layers.n_layers, layers.num_attention_heads
+        E, F, H = layers.embedding_dim, layers.ffn_embedding_dim, heads
         nb, ns = len(runner.batch_slices), len(runner.seq_slices)
-        dys = grid_slice_batch_and_sequence(grad_y, runner.batch_slices, runner.seq_slices,
-                                            batch_dim=runner.batch_dim, sequence_dim=runner.sequence_dim)
-        gdt = torch.float32 if runner.fp32_grad_cache else dt
-        nsmall = core.small_acc_numel(E, F)
-        small = torch.zeros(n_layers, nsmall, dtype=torch.float32, device=dev)
-        small_views = [core.small_acc_views(small[l], E, F) for l in range(n_layers)]
-        wgrads = [{n: torch.empty_like(ws[l][n]) for n in core.BIG_PARAMS} for l in range(n_layers)]
-        defer = runner.defer_weight_grads
-        stash = [[{n: [] for n in core.BIG_PARAMS} for _ in range(n_layers)]] if defer else None
-        dxs = np.empty((nb, ns), dtype="O")
-        first = True
+        L = runner.seq_len
+        ops.zero_(bufs.small)
+        b0 = sum(runner.batch_slices)
         for b in reversed(range(nb)):
             Bs = runner.batch_slices[b]
-            # gradient caches of this batch slice: every row is written (=) before it is read (+=),
-            # because the last slice covers all rows, so no zero fill is needed
-            gks = [torch.empty(Bs * heads, runner.seq_len, Dh, dtype=gdt, device=dev) for _ in range(2 * n_layers)]
+            b0 -= Bs
+            pb = bufs.per_batch[b]
+            pb["dx"][nl].view(L, Bs, E).copy_(grad_y[:, b0:b0 + Bs, :])
+            gc = pb["gcache"]
+            P = L
             for i in reversed(range(ns)):
+                T = runner.seq_slices[i]
+                P -= T
+                r0, r1 = P * Bs, (P + T) * Bs
                 last = i == ns - 1
-                dx = dys[b, i]
-                for l in reversed(range(n_layers)):
-                    d = {} if defer else None
-                    dx = core.layer_bwd(ws[l], states[b, i][l], dx, heads, gks[2 * l], gks[2 * l + 1], wgrads[l],
-                                        not first, small_views[l], accumulate_prefix=not last,
-                                        has_incoming=not last, zero_slice_rows=False, activation=act[l], defer=d)
-                    if defer:
-                        for n in core.BIG_PARAMS:
-                            stash[0][l][n].append(d[n])
-                states[b, i] = None
-                dxs[b, i] = dx
-                first = False
-        if defer:
-            for l in range(n_layers):
-                for n in core.BIG_PARAMS:
-                    pairs = stash[0][l][n]
-                    dY = torch.cat([p[0] for p in pairs], dim=0)
-                    X = torch.cat([p[1] for p in pairs], dim=0)
-                    ops.gemm(TP_GEMM_TN, dY, X, dY.shape[1], X.shape[1], dY.shape[0], C=wgrads[l][n],
-                             epilogue=TP_EPI_STORE)
+                for l in reversed(range(nl)):
+                    bf = core.Bufs(dz1=pb["dz1"][l][r0:r1], dhn=pb["dhn"][l][r0:r1], dh=pb["dh"][l][r0:r1],
+                                   d_o=pb["d_o"][:T * Bs], dqkv=pb["dqkv"][l][r0:r1], dxn=pb["dxn"][l][r0:r1],
+                                   dx=pb["dx"][l][r0:r1], delta=pb["delta"][:T * Bs * H].view(Bs * H, T))
+                    # the gradient caches need no zero fill: the last slice (processed first) writes every
+                    # prefix row with '=', the earlier ones add to rows that were written before
+                    core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), heads,
+                                   gc[2 * l], gc[2 * l + 1], None, False, None, accumulate_prefix=not last,
+                                   has_incoming=not last, zero_slice_rows=False, activation=act[l], buf=bf)
+        # parameter gradients over all tokens: dW = dY_all^T X_all (one GEMM per weight and batch slice),
+        # bias gradients = column sums of dY_all, LayerNorm gradients from (dy, x, mean, rstd) of all rows
         grads = []
-        for l in range(n_layers):
-            g = dict(wgrads[l])
+        for l in range(nl):
+            sv = bufs.small_views[l]
+            g = {n: torch.empty_like(ws[l][n]) for n in core.BIG_PARAMS}
+            for bi, pb in enumerate(bufs.per_batch):
+                R = L * runner.batch_slices[bi]
+                epi = TP_EPI_STORE if bi == 0 else TP_EPI_ACCUMULATE
+                dy_out = pb["dx"][l + 1]
+                ops.gemm(TP_GEMM_TN, pb["dqkv"][l], pb["xn"][l], 3 * E, E, R, C=g["attn.in_proj.weight"], epilogue=epi)
+                ops.gemm(TP_GEMM_TN, pb["dh"][l], pb["o"][l], E, E, R, C=g["attn.out_proj.weight"], epilogue=epi)
+                ops.gemm(TP_GEMM_TN, pb["dz1"][l], pb["hn"][l], F, E, R, C=g["fc1.weight"], epilogue=epi)
+                ops.gemm(TP_GEMM_TN, dy_out, pb["a"][l], E, F, R, C=g["fc2.weight"], epilogue=epi)
+                ops.colsum_acc(pb["dqkv"][l], sv["attn.in_proj.bias"])
+                ops.colsum_acc(pb["dh"][l], sv["attn.out_proj.bias"])
+                ops.colsum_acc(pb["dz1"][l], sv["fc1.bias"])
+                ops.colsum_acc(dy_out, sv["fc2.bias"])
+                ops.ln_param_grads(pb["dxn"][l], pb["x"][l], pb["mean1"][l], pb["rstd1"][l], sv["attn_ln.weight"],
+                                   sv["attn_ln.bias"])
+                ops.ln_param_grads(pb["dhn"][l], pb["h"][l], pb["mean2"][l], pb["rstd2"][l], sv["fc_ln.weight"],
+                                   sv["fc_ln.bias"])
             for n in core.SMALL_PARAMS:
                 t = torch.empty_like(ws[l][n])
-                ops.accum_cast(t, small_views[l][n], False)
+                ops.accum_cast(t, sv[n], False)
                 g[n] = t
             grads += [g[n] for n in core.PARAM_NAMES]
         dinputs = None
         if ctx.needs_input_grad[1]:
-            dinputs = torch.cat([torch.cat(list(dxs[b]), dim=runner.sequence_dim) for b in range(nb)],
-                                dim=runner.batch_dim)
+            if nb == 1:
+                dinputs = bufs.per_batch[0]["dx"][0].view(L, runner.batch_slices[0], E).clone()
+            else:
+                dinputs = torch.cat([pb["dx"][0].view(L, Bs, E)
+                                     for pb, Bs in zip(bufs.per_batch, runner.batch_slices)], dim=1)
         ctx.states = None
         return (None, dinputs) + tuple(grads)
 
@@ -179,13 +234,15 @@ class TeraPipe(nn.Module):
     leaves the summed-over-slices gradients in the layers' parameters (and in ``inputs.grad`` when the
     input requires grad).
 
-    defer_weight_grads: run one weight-gradient GEMM per weight over all tokens instead of one per slice.
-    fp32_grad_cache: keep the cross-slice dK/dV accumulators in fp32 (one rounding at the end) instead of
-    the cache dtype the reference uses.
+    The per-slice backward leaves the weight and vector-parameter gradients to one reduction over all
+    tokens at the end of backward (dW = dY_all^T X_all equals the sum over slices of dY_i^T X_i; the
+    layer-level autograd surface in transformer_models.py accumulates per slice instead).
+    fp32_grad_cache: keep the cross-slice dK/dV accumulators in fp32 (one rounding when a slice's own
+    rows are emitted) instead of the cache dtype the reference uses.
     """
 
     def __init__(self, layers, batch_size, seq_len, batch_slices, seq_slices, batch_dim=1, sequence_dim=0,
-                 defer_weight_grads=True, fp32_grad_cache=True):
+                 fp32_grad_cache=True):
         super().__init__()
         assert sum(batch_slices) == batch_size and sum(seq_slices) == seq_len
         assert batch_dim == 1 and sequence_dim == 0, "layers take [seq, batch, embed] inputs"
@@ -193,8 +250,8 @@ class TeraPipe(nn.Module):
         self.batch_slices, self.seq_slices = list(batch_slices), list(seq_slices)
         self.batch_dim, self.sequence_dim = batch_dim, sequence_dim
         self.layers = layers
-        self.defer_weight_grads = defer_weight_grads
         self.fp32_grad_cache = fp32_grad_cache
+        self._sbufs = None
         self.last_caches = None
         self.keep_states = False   # debugging / tests: keep the per-slice saved activations of the last forward
         self.last_states = None
@@ -206,6 +263,11 @@ class TeraPipe(nn.Module):
     @property
     def n_input_slices(self):
         return len(self.seq_slices)
+
+    def _stack_buffers(self, dtype, device):
+        if self._sbufs is None or self._sbufs.dtype != dtype or self._sbufs.device != device:
+            self._sbufs = _StackBuffers(self, dtype, device)
+        return self._sbufs
 
     def forward(self, inputs=None):
         if inputs is None:

@@ -59,6 +59,16 @@ def test_layernorm_fwd_bwd(dtype, M, E):
     acc.zero_()
     dx2 = ops.layernorm_bwd(dyd, xd, mean, rstd, gd, None, acc[0], acc[1], None, None)
     assert_close(dx2, x64.grad, dtype, "ln dx (no dres)")
+    # dx only (no accumulators), parameter gradients by the all-rows reduction
+    out = torch.empty_like(xd)
+    dx3 = ops.layernorm_bwd(dyd, xd, mean, rstd, gd, dresd, None, None, None, None, out=out)
+    assert dx3.data_ptr() == out.data_ptr()
+    assert_close(dx3, dx_ref, dtype, "ln dx (no accumulators)")
+    if E % 8 == 0:
+        acc.zero_()
+        ops.ln_param_grads(dyd, xd, mean, rstd, acc[0], acc[1])
+        assert_close(acc[0], g64.grad, torch.float32, "ln_param_grads dgamma", 20)
+        assert_close(acc[1], b64.grad, torch.float32, "ln_param_grads dbeta", 20)
 
 
 GEMM_SHAPES = [

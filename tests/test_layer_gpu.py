@@ -232,8 +232,8 @@ def _run_terapipe(ta, layers, x, dy, B, L, bs, ss, keep_states=False, **kw):
     return runner, y.detach(), xd.grad
 
 
-@pytest.mark.parametrize("defer,fp32gc", [(True, True), (False, True), (False, False), (True, False)])
-def test_terapipe_c1_tiny_fp32(defer, fp32gc):
+@pytest.mark.parametrize("fp32gc", [True, False])
+def test_terapipe_c1_tiny_fp32(fp32gc):
     """BASELINE config 1 (layer stack part): 4 layers, hidden 256, 4 heads, FFN 1024, seq 128, batch 2,
     fp32, 8 slices of 16, reverse-slice backward, tolerance 1e-5."""
     ta = _mods()
@@ -244,7 +244,7 @@ def test_terapipe_c1_tiny_fp32(defer, fp32gc):
     x, dy = torch.randn(L, B, E, generator=g), torch.randn(L, B, E, generator=g)
     yo, dxo, fco, go = oracle_run(ps, x, dy, H, [B], ss)
     layers = _build_layers(ta, n_layers, E, Fd, H, torch.float32, ps)
-    runner, y, dx = _run_terapipe(ta, layers, x, dy, B, L, [B], ss, defer_weight_grads=defer, fp32_grad_cache=fp32gc)
+    runner, y, dx = _run_terapipe(ta, layers, x, dy, B, L, [B], ss, fp32_grad_cache=fp32gc)
     assert_close(y, yo, torch.float32, "y")
     assert_close(dx, dxo, torch.float32, "dx")
     for j in range(2 * n_layers):
@@ -326,15 +326,14 @@ def test_terapipe_16bit_reduced_shapes(dtype, case):
     g = torch.Generator().manual_seed(17)
     x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
-    for defer, fp32gc in [(True, True), (False, False)]:
-        runner, y, dx = _run_terapipe(ta, layers, x, dy, B, L, bs, ss, keep_states=True,
-                                      defer_weight_grads=defer, fp32_grad_cache=fp32gc)
+    for fp32gc in (True, False):
+        runner, y, dx = _run_terapipe(ta, layers, x, dy, B, L, bs, ss, keep_states=True, fp32_grad_cache=fp32gc)
         # oracle with the ReLU active set of this run (module docstring)
         leaf = [{k: v.clone().requires_grad_(True) for k, v in p.items()} for p in ps]
         yo, dxo, fco = oracle.terapipe_forward_backward(leaf, x.float(), dy.float(), H, bs, ss,
                                                         relu_masks=_relu_masks_from_states(runner.last_states))
         go = [{k: v.grad for k, v in p.items()} for p in leaf]
-        tag = "%s defer=%s fp32gc=%s" % (case, defer, fp32gc)
+        tag = "%s fp32gc=%s" % (case, fp32gc)
         assert_close(y, yo, dtype, tag + " y")
         assert_close(dx, dxo, dtype, tag + " dx")
         for b in range(len(bs)):
@@ -395,3 +394,26 @@ def test_relu_flip_error_is_not_worse_than_plain_torch_16bit(dtype):
         for n in go[l]:
             e_hip, b = rel_err(got[l][n], go[l][n]), bound(leaf16[l][n].grad, go[l][n])
             assert e_hip <= b, "layer %d d(%s): hip %.3e, plain torch bound %.3e" % (l, n, e_hip, b)
+
+
+def test_runner_buffers_are_reused_across_steps():
+    """The runner keeps its activation / gradient buffers between steps: a second step on different
+    inputs must not see anything of the first (fp32, tolerance 1e-5)."""
+    ta = _mods()
+    n_layers, E, H, Fd, L, B = 2, 256, 4, 1024, 64, 2
+    ss = [16, 32, 16]
+    ps = make_params(n_layers, E, Fd, torch.float32, seed=4)
+    layers = _build_layers(ta, n_layers, E, Fd, H, torch.float32, ps)
+    runner = ta.TeraPipe(layers, B, L, [1, 1], ss)
+    for seed in (1, 2):
+        g = torch.Generator().manual_seed(seed)
+        x, dy = torch.randn(L, B, E, generator=g), torch.randn(L, B, E, generator=g)
+        yo, dxo, _, go = oracle_run(ps, x, dy, H, [1, 1], ss)
+        for p in layers.parameters():
+            p.grad = None
+        xd = x.to(DEV).requires_grad_(True)
+        y = runner(xd)
+        (y * dy.to(DEV)).sum().backward()
+        assert_close(y, yo, torch.float32, "step %d y" % seed)
+        assert_close(xd.grad, dxo, torch.float32, "step %d dx" % seed)
+        _check_param_grads(_param_grads(layers), go, torch.float32, "step %d" % seed)
