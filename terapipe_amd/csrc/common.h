@@ -172,6 +172,33 @@ __device__ __forceinline__ typename Elem<T>::opnd_t fetch_tr(const T* tile, int 
     }
 }
 
+// The same fetches split into "compute the lane's LDS offset once" and "load from a precomputed
+// address", for loops that revisit the same tile positions (the offsets do not depend on the k-tile).
+template <typename T, int COLS>
+__device__ __forceinline__ int km_offset(int row, int k0, int lane) {
+    static_assert(sizeof(T) == 2, "16-bit tiles");
+    return TileLayout<T, COLS>::off(row, k0 + 8 * (lane >> 5));
+}
+template <typename T, int COLS, bool INTERLEAVED>
+__device__ __forceinline__ void tr_offsets(int krow0, int col0, int lane, int& o0, int& o1) {
+    static_assert(sizeof(T) == 2, "16-bit tiles");
+    typedef TileLayout<T, COLS> L;
+    const int g = lane >> 5, p = lane & 15;
+    const int col = col0 + 16 * ((lane & 31) >> 4) + 4 * (p & 3);
+    const int r0 = krow0 + (INTERLEAVED ? 4 * g : 8 * g) + (p >> 2);
+    o0 = L::off(r0, col);
+    o1 = L::off(r0 + (INTERLEAVED ? 8 : 4), col);
+}
+template <typename T> __device__ __forceinline__ uint4 load_km(const T* p) {
+    return *reinterpret_cast<const uint4*>(p);
+}
+template <typename T> __device__ __forceinline__ uint4 load_tr(const T* p0, const T* p1) {
+    short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TP_LDS_PTR(short4v, p0));
+    short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TP_LDS_PTR(short4v, p1));
+    uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+    return make_uint4(l2.x, l2.y, h2.x, h2.y);
+}
+
 // Pack 8 fp32 accumulator values (registers j0 .. j0+7 of a 32x32 block) into one 16-bit MFMA operand.
 template <typename T>
 __device__ __forceinline__ uint4 pack8(const float* v) {
@@ -207,6 +234,108 @@ __device__ __forceinline__ float wave_sum(float v) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
     return v;
 }
+
+// ---------------------------------------------------------------------------------------------
+// Direct global -> LDS tile loads (global_load_lds_dwordx4).  A wave instruction writes 64 consecutive
+// 16-byte chunks of LDS, so the XOR swizzle of the tile layout is applied on the global side: the lane
+// that fills LDS chunk (row, pc) loads the global chunk (row, pc ^ swz(row)).  Chunks outside the matrix
+// are loaded from a zero buffer so that every lane issues every load and the per-tile vmcnt accounting
+// is exact.  The loads are inline asm: the compiler does not see them as LDS writes (it would otherwise
+// force vmcnt(0) before every ds_read); kernels wait with wait_vmcnt<n>() + s_barrier once per tile.
+// ---------------------------------------------------------------------------------------------
+static __device__ __attribute__((aligned(16))) unsigned int g_zero_chunk[4] = {0u, 0u, 0u, 0u};
+
+__device__ __forceinline__ void dma16(const void* gptr, const void* lds_wave_base) {
+    unsigned lds = (unsigned)(unsigned long)(__attribute__((address_space(3))) const void*)lds_wave_base;
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+                 :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory");
+}
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N <= 63, "vmcnt immediate is 6 bits");
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
+template <typename T, int ROWS, int COLS, int NT> struct TileDma {
+    static constexpr int CPR = COLS / 8;
+    static constexpr int TOTAL = ROWS * CPR;
+    static constexpr int N = TOTAL / NT;
+    static_assert(TOTAL % NT == 0 && NT % 64 == 0, "tile must split evenly over the waves");
+    // issues the N loads of this thread for the tile whose first element is (r0, c0)
+    static __device__ __forceinline__ void issue(T* lds, const T* __restrict__ base, long ld, int r0, int c0,
+                                                 int rmax, int cmax, int tid) {
+        const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int p0 = (i * (NT / 64) + wave) * 64;
+            const int p = p0 + lane;
+            const int row = p / CPR, pc = p % CPR;
+            const int lc = pc ^ swz16<COLS>(row);
+            const int gr = r0 + row, gc = c0 + lc * 8;
+            const void* src = (gr < rmax && gc < cmax) ? (const void*)(base + (long)gr * ld + gc)
+                                                       : (const void*)g_zero_chunk;
+            dma16(src, lds + p0 * 8);
+        }
+    }
+};
+
+// The same tile loads for a tile that slides along one axis in equal steps (the k loop of a GEMM, the
+// key loop of attention): the per-lane source pointers are computed once, every step is one 64-bit add
+// per load.  `ALONG_COLS` says whether the tile slides along its columns (k-major operand) or its rows.
+// Lanes whose fixed coordinate is outside the matrix point at the zero chunk with stride 0; the sliding
+// coordinate is checked only on the steps the caller flags as possibly partial.
+template <typename T, int ROWS, int COLS, int NT, bool ALONG_COLS> struct SlidingTileDma {
+    static constexpr int CPR = COLS / 8;
+    static constexpr int TOTAL = ROWS * CPR;
+    static constexpr int N = TOTAL / NT;
+    static_assert(TOTAL % NT == 0 && NT % 64 == 0, "tile must split evenly over the waves");
+    const char* ptr[N];     // source of this lane's chunk in the NEXT tile to issue
+    long step[N];           // bytes to advance per tile (0 for lanes pinned to the zero chunk)
+    int slide[N];           // offset of this lane's chunk along the sliding axis inside a tile
+    int pos;                // sliding coordinate of the next tile to issue, relative to the start
+
+    // fixed0 / fixed_max: first coordinate and bound of the axis that does not slide;
+    // slide0: start of the sliding axis; tile_step: elements to slide per tile.
+    __device__ __forceinline__ void init(const T* __restrict__ base, long ld, int fixed0, int fixed_max,
+                                         int slide0, int tile_step, int tid) {
+        const int lane = tid & 63, wave = tid >> 6;
+        pos = 0;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int p = (i * (NT / 64) + wave) * 64 + lane;
+            const int row = p / CPR, pc = p % CPR;
+            const int lc = pc ^ swz16<COLS>(row);
+            const int fx = ALONG_COLS ? row : lc * 8;
+            slide[i] = ALONG_COLS ? lc * 8 : row;
+            const bool ok = fixed0 + fx < fixed_max;
+            const long gr = ALONG_COLS ? fixed0 + fx : slide0 + slide[i];
+            const long gc = ALONG_COLS ? slide0 + slide[i] : fixed0 + fx;
+            ptr[i] = ok ? reinterpret_cast<const char*>(base + gr * ld + gc)
+                        : reinterpret_cast<const char*>(g_zero_chunk);
+            step[i] = ok ? (ALONG_COLS ? (long)tile_step : (long)tile_step * ld) * (long)sizeof(T) : 0;
+        }
+    }
+    // issues the next tile; `len` is the extent of the sliding axis from its start, `tile_step` as in
+    // init.  Chunks at or beyond len load zeros.
+    __device__ __forceinline__ void issue(T* lds, int len, int tile_step, int tid) {
+        const int wave = tid >> 6;
+        if (pos + tile_step <= len) {          // uniform: the whole tile is inside
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                dma16(ptr[i], lds + (i * (NT / 64) + wave) * 512);
+                ptr[i] += step[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                const void* src = pos + slide[i] < len ? (const void*)ptr[i] : (const void*)g_zero_chunk;
+                dma16(src, lds + (i * (NT / 64) + wave) * 512);
+                ptr[i] += step[i];
+            }
+        }
+        pos += tile_step;
+    }
+};
 
 // error plumbing shared by the host-side entry points
 void set_error(const char* fmt, ...);

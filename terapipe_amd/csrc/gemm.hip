@@ -210,42 +210,6 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, float16v (&acc)
 // compiler does not see them as LDS writes (it would otherwise force vmcnt(0) before every ds_read),
 // and the kernel waits with explicit s_waitcnt vmcnt(n) + s_barrier once per k-tile.
 // ---------------------------------------------------------------------------------------------
-__device__ __attribute__((aligned(16))) unsigned int g_zero_chunk[4] = {0u, 0u, 0u, 0u};
-
-__device__ __forceinline__ void dma16(const void* gptr, const void* lds_wave_base) {
-    unsigned lds = (unsigned)(unsigned long)(__attribute__((address_space(3))) const void*)lds_wave_base;
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
-                 :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory");
-}
-
-template <int N> __device__ __forceinline__ void wait_vmcnt() {
-    static_assert(N >= 0 && N <= 63, "vmcnt immediate is 6 bits");
-    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
-}
-
-template <typename T, int ROWS, int COLS, int NT> struct TileDma {
-    static constexpr int CPR = COLS / 8;
-    static constexpr int TOTAL = ROWS * CPR;
-    static constexpr int N = TOTAL / NT;
-    static_assert(TOTAL % NT == 0 && NT % 64 == 0, "tile must split evenly over the waves");
-    // issues the N loads of this thread for the tile whose first element is (r0, c0)
-    static __device__ __forceinline__ void issue(T* lds, const T* __restrict__ base, long ld, int r0, int c0,
-                                                 int rmax, int cmax, int tid) {
-        const int lane = tid & 63, wave = tid >> 6;
-#pragma unroll
-        for (int i = 0; i < N; ++i) {
-            const int p0 = (i * (NT / 64) + wave) * 64;
-            const int p = p0 + lane;
-            const int row = p / CPR, pc = p % CPR;
-            const int lc = pc ^ swz16<COLS>(row);
-            const int gr = r0 + row, gc = c0 + lc * 8;
-            const void* src = (gr < rmax && gc < cmax) ? (const void*)(base + (long)gr * ld + gc)
-                                                       : (const void*)g_zero_chunk;
-            dma16(src, lds + p0 * 8);
-        }
-    }
-};
-
 template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN, int STAGES>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_dma_kernel(GemmArgs a) {
     typedef Elem<T> E;
@@ -256,8 +220,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_dma_kernel(GemmArgs a) {
     constexpr int BR = BKM ? BN : BK, BC = BKM ? BK : BN;
     constexpr int A_ELEMS = AR * AC, B_ELEMS = BR * BC;
     constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
-    typedef TileDma<T, AR, AC, NT> DA;
-    typedef TileDma<T, BR, BC, NT> DB;
+    typedef SlidingTileDma<T, AR, AC, NT, AKM> DA;
+    typedef SlidingTileDma<T, BR, BC, NT, BKM> DB;
     constexpr int NLOAD = DA::N + DB::N;                 // DMA instructions per thread per k-tile
     static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
     constexpr int TILE_BYTES = STAGES * STAGE_ELEMS * 2;
@@ -274,14 +238,15 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_dma_kernel(GemmArgs a) {
     const T* A = reinterpret_cast<const T*>(a.A);
     const T* B = reinterpret_cast<const T*>(a.B);
 
-    auto issue = [&](int kt, int stage) {
+    DA da;
+    DB db;
+    da.init(A, a.lda, m0, a.M, kbeg, BK, tid);
+    db.init(B, a.ldb, n0, a.N, kbeg, BK, tid);
+    const int klen = kend - kbeg;
+    auto issue = [&](int stage) {      // tiles are issued in k order; tiles past the end load zeros
         T* sA = tiles + stage * STAGE_ELEMS;
-        T* sB = sA + A_ELEMS;
-        const int k0 = kbeg + kt * BK;
-        if constexpr (AKM) DA::issue(sA, A, a.lda, m0, k0, a.M, kend, tid);
-        else DA::issue(sA, A, a.lda, k0, m0, kend, a.M, tid);
-        if constexpr (BKM) DB::issue(sB, B, a.ldb, n0, k0, a.N, kend, tid);
-        else DB::issue(sB, B, a.ldb, k0, n0, kend, a.N, tid);
+        da.issue(sA, klen, BK, tid);
+        db.issue(sA + A_ELEMS, klen, BK, tid);
     };
 
     float16v acc[TM][TN];
@@ -292,40 +257,80 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_dma_kernel(GemmArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+    // LDS addresses of this lane's operand fetches inside stage 0 (they do not depend on the k-tile;
+    // with the stage loop unrolled the stage base folds into the instruction's immediate offset)
+    constexpr int NKSTEP = BK / E::KSTEP;
+    constexpr int NPA = AKM ? 1 : 2, NPB = BKM ? 1 : 2;
+    const T* pa[NKSTEP][TM][NPA];
+    const T* pb[NKSTEP][TN][NPB];
+#pragma unroll
+    for (int ks = 0; ks < NKSTEP; ++ks) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int mb = (wm * TM + i) * 32;
+            if constexpr (AKM) {
+                pa[ks][i][0] = tiles + km_offset<T, AC>(mb + (lane & 31), ks * E::KSTEP, lane);
+            } else {
+                int o0, o1;
+                tr_offsets<T, AC, false>(ks * E::KSTEP, mb, lane, o0, o1);
+                pa[ks][i][0] = tiles + o0;
+                pa[ks][i][NPA - 1] = tiles + o1;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int nb = (wn * TN + j) * 32;
+            if constexpr (BKM) {
+                pb[ks][j][0] = tiles + A_ELEMS + km_offset<T, BC>(nb + (lane & 31), ks * E::KSTEP, lane);
+            } else {
+                int o0, o1;
+                tr_offsets<T, BC, false>(ks * E::KSTEP, nb, lane, o0, o1);
+                pb[ks][j][0] = tiles + A_ELEMS + o0;
+                pb[ks][j][NPB - 1] = tiles + A_ELEMS + o1;
+            }
+        }
+    }
+
     const int nk = (kend - kbeg + BK - 1) / BK;
     // prologue: tiles 0 .. STAGES-2 in flight (tiles past the end load zeros; keeps the counts uniform)
 #pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) issue(s, s);
+    for (int s = 0; s < STAGES - 1; ++s) issue(s);
 
-    for (int kt = 0; kt < nk; ++kt) {
-        // tile kt has landed once at most the loads of the STAGES-2 younger tiles are outstanding
-        wait_vmcnt<NLOAD * (STAGES - 2)>();
-        __builtin_amdgcn_s_barrier();   // every wave's part of tile kt is in LDS; tile kt-1 is no longer read
-        asm volatile("" ::: "memory");
-        issue(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);   // refills the buffer tile kt-1 used
-        const T* tA = tiles + (kt % STAGES) * STAGE_ELEMS;
-        const T* tB = tA + A_ELEMS;
+    for (int kt0 = 0; kt0 < nk; kt0 += STAGES) {
 #pragma unroll
-        for (int ks = 0; ks < BK / E::KSTEP; ++ks) {
-            typename E::opnd_t fa[TM], fb[TN];
+        for (int s = 0; s < STAGES; ++s) {        // stage index is a compile-time constant in here
+            if (kt0 + s < nk) {
+                // tile kt has landed once at most the loads of the STAGES-2 younger tiles are outstanding
+                wait_vmcnt<NLOAD * (STAGES - 2)>();
+                __builtin_amdgcn_s_barrier();   // every wave's part of the tile is in LDS; the previous tile is no longer read
+                asm volatile("" ::: "memory");
+                issue((s + STAGES - 1) % STAGES);   // tile kt + STAGES - 1 refills the buffer of tile kt - 1
+                // all operand fetches of the tile are issued before the first MFMA, so their LDS latency
+                // overlaps instead of being paid once per k-step (one wave per SIMD has nothing else to hide it)
+                typename E::opnd_t fa[NKSTEP][TM], fb[NKSTEP][TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                int mb = (wm * TM + i) * 32;
-                if constexpr (AKM) fa[i] = fetch_km<T, AC>(tA, mb + (lane & 31), ks * E::KSTEP, lane);
-                else fa[i] = fetch_tr<T, AC, false>(tA, ks * E::KSTEP, mb, lane);
+                for (int ks = 0; ks < NKSTEP; ++ks) {
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) {
+                        if constexpr (AKM) fa[ks][i] = load_km<T>(pa[ks][i][0] + s * STAGE_ELEMS);
+                        else fa[ks][i] = load_tr<T>(pa[ks][i][0] + s * STAGE_ELEMS, pa[ks][i][NPA - 1] + s * STAGE_ELEMS);
+                    }
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) {
+                        if constexpr (BKM) fb[ks][j] = load_km<T>(pb[ks][j][0] + s * STAGE_ELEMS);
+                        else fb[ks][j] = load_tr<T>(pb[ks][j][0] + s * STAGE_ELEMS, pb[ks][j][NPB - 1] + s * STAGE_ELEMS);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);   // keep the scheduler from sinking the fetches to their uses
+#pragma unroll
+                for (int ks = 0; ks < NKSTEP; ++ks)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) acc[i][j] = E::mfma(fa[ks][i], fb[ks][j], acc[i][j]);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave's LDS reads of the tile are done
             }
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                int nb = (wn * TN + j) * 32;
-                if constexpr (BKM) fb[j] = fetch_km<T, BC>(tB, nb + (lane & 31), ks * E::KSTEP, lane);
-                else fb[j] = fetch_tr<T, BC, false>(tB, ks * E::KSTEP, nb, lane);
-            }
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = E::mfma(fa[i], fb[j], acc[i][j]);
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave's LDS reads of tile kt are done
     }
     // drain the zero-tile loads still in flight before LDS is reused for the epilogue
     wait_vmcnt<0>();
@@ -485,6 +490,11 @@ static const TileCfg kCfgs[] = {
     {128, 64, 64, 4},    // 6
     {64, 128, 64, 4},    // 7
     {64, 64, 64, 4},     // 8
+    {64, 64, 64, 8},     // 9
+    {128, 128, 32, 4},   // 10
+    {128, 64, 64, 6},    // 11
+    {64, 64, 128, 4},    // 12
+    {128, 128, 64, 3},   // 13
 };
 static constexpr int kNumCfgs = (int)(sizeof(kCfgs) / sizeof(kCfgs[0]));
 
@@ -531,7 +541,7 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     const long t128 = (long)((d->M + 127) / 128) * ((d->N + 127) / 128);
     const long t64 = (long)((d->M + 63) / 64) * ((d->N + 63) / 64);
     int cfg, ns = 1;
-    if (t128 >= 96) {
+    if (t128 >= 144) {
         cfg = 5;
         if (t128 < 224) {
             ns = (int)(448 / t128);
@@ -542,7 +552,7 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
         cfg = 8;
         if (t64 < 384) {
             ns = (int)(512 / t64);
-            int maxs = d->K / 2048;
+            int maxs = d->K / 3072;
             if (ns > maxs) ns = maxs;
         }
     }
@@ -572,6 +582,11 @@ static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
         case 6: gemm_dma_kernel<T, AKM, BKM, 128, 64, 64, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
         case 7: gemm_dma_kernel<T, AKM, BKM, 64, 128, 64, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
         case 8: gemm_dma_kernel<T, AKM, BKM, 64, 64, 64, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
+        case 9: gemm_dma_kernel<T, AKM, BKM, 64, 64, 64, 2, 2, 8><<<grid, 256, 0, s>>>(a); break;
+        case 10: gemm_dma_kernel<T, AKM, BKM, 128, 128, 32, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
+        case 11: gemm_dma_kernel<T, AKM, BKM, 128, 64, 64, 2, 2, 6><<<grid, 256, 0, s>>>(a); break;
+        case 12: gemm_dma_kernel<T, AKM, BKM, 64, 64, 128, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
+        case 13: gemm_dma_kernel<T, AKM, BKM, 128, 128, 64, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
         default: gemm_kernel<T, AKM, BKM, 64, 64, 64, 2, 2><<<grid, 256, 0, s>>>(a); break;
         }
     }
