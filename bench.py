@@ -121,6 +121,8 @@ def main():
     ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--eager", action="store_true",
+                    help="launch every kernel from the host each step instead of replaying the runner's HIP graphs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -135,6 +137,7 @@ def main():
     from terapipe_amd import ops
 
     layers, runner, x, R = build_model(w, device)
+    runner.use_hip_graph = not args.eager
     for _ in range(args.warmup):
         one_step(layers, runner, x, R)
     torch.cuda.synchronize()
@@ -153,39 +156,71 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w["dtype"], "data": "synthetic",
         "config": {"workload": "%s: %s" % (args.workload, w["desc"]),
-                   "loss": "sum(y * R), R ~ N(0,1) fixed", "optimizer_step": "not part of the path"},
+                   "loss": "sum(y * R), R ~ N(0,1) fixed", "optimizer_step": "not part of the path",
+                   "launch": "eager" if args.eager else "HIP-graph replay of forward and of backward"},
     }
 
     if not args.no_roofline:
-        # one instrumented step: every library call bracketed by HIP events on the launch stream
-        with ops.KernelTimer() as kt:
+        # Kernel time per kind, measured live with HIP events: one step is recorded (every library call
+        # with its descriptor and buffers), then all calls of one kind are replayed back to back inside
+        # a HIP graph on the launch stream and the replay is bracketed by two events.  Replaying from a
+        # graph keeps host launch gaps out of the figure (events around single eager launches would
+        # include the time the GPU waits for the host).
+        runner.use_hip_graph = False
+        with ops.CallRecorder() as rec:
             one_step(layers, runner, x, R)
+        torch.cuda.synchronize()
+
+        def replay_ms(tag, reps=3):
+            calls = rec.by_tag(tag)
+            if not calls:
+                return 0, 0.0, []
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _, _, fn in calls[:4]:
+                    fn()
+            torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize()
-        summ = kt.summary()
-        g_calls, g_ms, _ = summ.get("gemm", (0, 0.0, []))
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for _, _, fn in calls:
+                    fn()
+            g.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            return len(calls), e0.elapsed_time(e1) / reps, [m for _, m, _ in calls]
+
+        g_calls, g_ms, _ = replay_ms("gemm")
         flops = gemm_flops_per_step(w)
         peak = PEAK_MFMA_FP32 if w["dtype"] == "f32" else PEAK_MFMA_16BIT
         achieved = flops / (g_ms * 1e-3) if g_ms > 0 else 0.0
         out["roofline"] = {
-            "kernel": "tp::gemm_kernel (all NT/NN/TN launches of one step, split-K reduce included)",
+            "kernel": "tp::gemm_dma_kernel / tp::gemm_kernel (all NT/NN/TN launches of one step, split-K reduce included)",
             "bound": "mfma", "achieved": achieved / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
             "frac": achieved / peak, "traffic": None,
             "launches": g_calls, "avg_launch_us": g_ms * 1e3 / max(g_calls, 1),
             "algorithmic_flops_per_step": flops, "kernel_ms_per_step": g_ms,
+            "method": "graph replay of the step's GEMM calls between two HIP events",
         }
-        # prefix attention: algorithmic bytes / kernel time, over all calls of the step
-        a_bytes = {"attn_fwd": 0.0, "attn_bwd": 0.0}
-        for tag in a_bytes:
-            for (_b, _h, _d, T, P) in summ.get(tag, (0, 0.0, []))[2]:
-                a_bytes[tag] += attn_bytes_per_call(w, T, P, tag == "attn_bwd")
         attn = {}
-        for tag in a_bytes:
-            c, ms, _ = summ.get(tag, (0, 0.0, []))
-            gbs = a_bytes[tag] / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
-            attn[tag] = {"calls": c, "kernel_ms_per_step": ms, "algorithmic_GB_per_step": a_bytes[tag] / 1e9,
+        kt = {"gemm": round(g_ms, 3)}
+        for tag in ("attn_fwd", "attn_bwd"):
+            c, ms, metas = replay_ms(tag)
+            nbytes = sum(attn_bytes_per_call(w, T, P, tag == "attn_bwd") for (_b, _h, _d, T, P) in metas)
+            gbs = nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+            attn[tag] = {"calls": c, "kernel_ms_per_step": ms, "algorithmic_GB_per_step": nbytes / 1e9,
                          "achieved_GBps": gbs, "frac_of_hbm_peak": gbs * 1e9 / PEAK_HBM}
+            kt[tag] = round(ms, 3)
+        for tag in ("layernorm_fwd", "layernorm_bwd"):
+            kt[tag] = round(replay_ms(tag)[1], 3)
         out["roofline_attention"] = {"bound": "hbm", "peak": PEAK_HBM / 1e9, "unit": "GB/s", **attn}
-        out["kernel_time_ms_per_step"] = {k: round(v[1], 3) for k, v in summ.items()}
+        out["kernel_time_ms_per_step"] = kt
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)

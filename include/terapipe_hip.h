@@ -147,6 +147,8 @@ typedef struct tp_attn_desc {
                                            (grad_cache.data[index] = 0, transformer_models.py:189) */
     float q_scale;
     float* colsum_dqkv_acc;             /* optional [3*H*Dh] fp32: += column sums of dqkv (in_proj bias grad) */
+    int32_t reserved;                   /* 0 = automatic; bits 0-7: number of key-range splits of the forward (tuning, tests) */
+    int32_t reserved2;
 } tp_attn_desc;
 
 size_t tp_attn_fwd_workspace_bytes(const tp_attn_desc* d);

@@ -52,6 +52,7 @@ class AttnDesc(ctypes.Structure):
         ("has_incoming", c_int32), ("zero_slice_rows", c_int32),
         ("q_scale", c_float),
         ("colsum_dqkv_acc", c_void_p),
+        ("reserved", c_int32), ("reserved2", c_int32),
     ]
 
 

@@ -25,6 +25,9 @@ struct AttnArgs {
 
 static constexpr float kLog2e = 1.4426950408889634f;
 
+// v_exp_f32: 2^x at hardware precision (about 1 ulp), results below the normal range flush to zero
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 template <typename T, int DH>
 __device__ __forceinline__ void load_row_operands(typename Elem<T>::opnd_t* reg, const T* rowptr, bool valid, int g) {
     typedef Elem<T> E;
@@ -495,34 +498,44 @@ __device__ __forceinline__ void attn_fwd_tile(const T* sK, const T* sV, const ty
         for (int ks = 0; ks < NKS; ++ks) sacc[kb] = E::mfma(kop[ks], qreg[ks], sacc[kb]);
     }
     float mt = -INFINITY;
+    if (key0 + NKB * 32 - 1 > P + (tq - li)) {      // wave-uniform: some key of the tile is masked for some row
 #pragma unroll
-    for (int kb = 0; kb < NKB; ++kb)
+        for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            int key = key0 + kb * 32 + acc_row(j, g);
-            float sc = key > P + tq ? -INFINITY : sacc[kb][j];
-            sacc[kb][j] = sc;
-            mt = fmaxf(mt, sc);
-        }
+            for (int j = 0; j < 16; ++j) {
+                int key = key0 + kb * 32 + acc_row(j, g);
+                float sc = key > P + tq ? -INFINITY : sacc[kb][j];
+                sacc[kb][j] = sc;
+                mt = fmaxf(mt, sc);
+            }
+    } else {
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) mt = fmaxf(mt, sacc[kb][j]);
+    }
     mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
     const float m_new = fmaxf(m, mt);
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = exp2f((m - m_safe) * kLog2e);
+    const float alpha = fast_exp2((m - m_safe) * kLog2e);
+    const float mneg = -m_safe * kLog2e;
     float psum = 0.f;
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
-            float p = exp2f((sacc[kb][j] - m_safe) * kLog2e);
+            float p = fast_exp2(fmaf(sacc[kb][j], kLog2e, mneg));   // exp(s - m); -inf -> 0
             sacc[kb][j] = p;
             psum += p;
         }
     lsum = lsum * alpha + psum;
     m = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {   // wave-uniform: some row's running maximum moved
 #pragma unroll
-    for (int db = 0; db < NDB; ++db)
+        for (int db = 0; db < NDB; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+            for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+    }
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb) mfma_acc_as_b<T, DH>(oacc, sV, kb * 32, sacc[kb], lane);
 }
@@ -533,7 +546,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_dma_kernel(AttnArgs a) {
     static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
     constexpr int NT = NW * 64, NKB = BN / 32, NDB = DH / 32, NKS = DH / E::KSTEP;
     constexpr int TILE = BN * DH;                       // elements of one K or V tile
-    typedef TileDma<T, BN, DH, NT> D;
+    typedef RowSlideDma<T, BN, DH, NT> D;
     constexpr int NLOAD = 2 * D::N;
     static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
     __shared__ __attribute__((aligned(16))) T ring[STAGES * 2 * TILE];
@@ -563,13 +576,15 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_dma_kernel(AttnArgs a) {
 
     const T* Kb = reinterpret_cast<const T*>(a.kc) + (long)bh * a.cache_rows * DH;
     const T* Vb = reinterpret_cast<const T*>(a.vc) + (long)bh * a.cache_rows * DH;
+    D dma;
+    dma.init(DH, tid);
     auto issue = [&](int it) {
-        // tile index past the range loads zeros (rmax = 0): keeps the per-tile load count uniform
+        // rows past S are clamped to row S-1 (finite, masked); tiles past the range reload the last
+        // rows, which keeps the per-tile load count uniform
         const int stage = it % STAGES;
         const int row0 = (t_beg + it) * BN;
-        const int rmax = it < nt ? S : 0;
-        D::issue(ring + stage * 2 * TILE, Kb, DH, row0, 0, rmax, DH, tid);
-        D::issue(ring + stage * 2 * TILE + TILE, Vb, DH, row0, 0, rmax, DH, tid);
+        dma.issue(ring + stage * 2 * TILE, Kb, row0, S, tid);
+        dma.issue(ring + stage * 2 * TILE + TILE, Vb, row0, S, tid);
     };
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) issue(s);
@@ -626,7 +641,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_dma_kernel(AttnArgs a) {
     static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
     constexpr int NT = NW * 64, NKB = BN / 32, NDB = DH / 32, NKS = DH / E::KSTEP;
     constexpr int TILE = BN * DH;
-    typedef TileDma<T, BN, DH, NT> D;
+    typedef RowSlideDma<T, BN, DH, NT> D;
     constexpr int NLOAD = 2 * D::N;
     static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
     __shared__ __attribute__((aligned(16))) T ring[STAGES * 2 * TILE];
@@ -646,6 +661,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_dma_kernel(AttnArgs a) {
     load_row_operands<T, DH>(doreg, reinterpret_cast<const T*>(a.d_o) + ((long)tq * a.B + b) * EE + (long)h * DH, tq < T_, g);
     const float lse_q = tq < T_ ? a.lse[(long)bh * T_ + tq] : 0.f;
     const float delta_q = tq < T_ ? a.delta[(long)bh * T_ + tq] : 0.f;
+    const float lse_neg = -lse_q * kLog2e;
     wait_vmcnt<0>();
 
     float16v dq[NDB];
@@ -656,11 +672,12 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_dma_kernel(AttnArgs a) {
 
     const T* Kb = reinterpret_cast<const T*>(a.kc) + (long)bh * a.cache_rows * DH;
     const T* Vb = reinterpret_cast<const T*>(a.vc) + (long)bh * a.cache_rows * DH;
+    D dma;
+    dma.init(DH, tid);
     auto issue = [&](int it) {
         const int stage = it % STAGES;
-        const int rmax = it < nt ? S : 0;
-        D::issue(ring + stage * 2 * TILE, Kb, DH, it * BN, 0, rmax, DH, tid);
-        D::issue(ring + stage * 2 * TILE + TILE, Vb, DH, it * BN, 0, rmax, DH, tid);
+        dma.issue(ring + stage * 2 * TILE, Kb, it * BN, S, tid);
+        dma.issue(ring + stage * 2 * TILE + TILE, Vb, it * BN, S, tid);
     };
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) issue(s);
@@ -690,11 +707,19 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_dma_kernel(AttnArgs a) {
                     sacc = E::mfma(kop[ks], qreg[ks], sacc);
                     pacc = E::mfma(vop[ks], doreg[ks], pacc);
                 }
+                if (key0 + kb * 32 + 31 > P + q0w) {     // wave-uniform: the block touches the causal boundary
 #pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    int key = key0 + kb * 32 + acc_row(j, g);
-                    float p = key > P + tq ? 0.f : exp2f((sacc[j] - lse_q) * kLog2e);
-                    pacc[j] = p * (pacc[j] - delta_q);
+                    for (int j = 0; j < 16; ++j) {
+                        int key = key0 + kb * 32 + acc_row(j, g);
+                        float p = key > P + tq ? 0.f : fast_exp2(fmaf(sacc[j], kLog2e, lse_neg));
+                        pacc[j] = p * (pacc[j] - delta_q);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        float p = fast_exp2(fmaf(sacc[j], kLog2e, lse_neg));
+                        pacc[j] = p * (pacc[j] - delta_q);
+                    }
                 }
                 mfma_acc_as_b<T, DH>(dq, sK, kb * 32, pacc, lane);
             }
@@ -725,7 +750,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_dma_kernel(AttnArgs a) 
     static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
     constexpr int NT = NW * 64, NDB = DH / 32, NKS = DH / E::KSTEP;
     constexpr int TILE = 32 * DH;
-    typedef TileDma<T, 32, DH, NT> D;
+    typedef RowSlideDma<T, 32, DH, NT> D;
     constexpr int NLOAD = 2 * D::N;
     static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
     __shared__ __attribute__((aligned(16))) T ring[STAGES * 2 * TILE];
@@ -747,7 +772,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_dma_kernel(AttnArgs a) 
     load_row_operands<T, DH>(kreg, reinterpret_cast<const T*>(a.kc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
     load_row_operands<T, DH>(vreg, reinterpret_cast<const T*>(a.vc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
     for (int t = tid; t < Tpad; t += NT) {
-        sLse[t] = t < T_ ? a.lse[(long)bh * T_ + t] : 0.f;
+        sLse[t] = t < T_ ? -a.lse[(long)bh * T_ + t] * kLog2e : 0.f;     // stored as -lse * log2(e)
         sDelta[t] = t < T_ ? a.delta[(long)bh * T_ + t] : 0.f;
     }
     wait_vmcnt<0>();
@@ -763,11 +788,14 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_dma_kernel(AttnArgs a) 
     const T* dOb = reinterpret_cast<const T*>(a.d_o) + (long)b * EE + (long)h * DH;  // row t at stride B*E
     const int qb_start = key0wg > P ? (key0wg - P) / 32 : 0;
     const int nt = nqb - qb_start;
+    D dmaq, dmado;
+    dmaq.init(DH, tid);
+    dmado.init((long)a.B * EE, tid);
     auto issue = [&](int it) {
+        // query rows past T are clamped to row T-1: finite data whose P and dS are forced to zero
         const int stage = it % STAGES;
-        const int rmax = it < nt ? T_ : 0;
-        D::issue(ring + stage * 2 * TILE, Qb, DH, (qb_start + it) * 32, 0, rmax, DH, tid);
-        D::issue(ring + stage * 2 * TILE + TILE, dOb, (long)a.B * EE, (qb_start + it) * 32, 0, rmax, DH, tid);
+        dmaq.issue(ring + stage * 2 * TILE, Qb, (qb_start + it) * 32, T_, tid);
+        dmado.issue(ring + stage * 2 * TILE + TILE, dOb, (qb_start + it) * 32, T_, tid);
     };
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) issue(s);
@@ -801,12 +829,17 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_dma_kernel(AttnArgs a) 
                 float4 d4 = *reinterpret_cast<const float4*>(sDelta + qb * 32 + 8 * jq + 4 * g);
                 const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
                 const float dl[4] = {d4.x, d4.y, d4.z, d4.w};
+                // wave-uniform: every (query, key) pair of the block is visible and in range
+                const bool all_visible = (qb * 32 + 32 <= T_) && (key0w + 31 <= P + qb * 32) && (key0w + 32 <= S);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     int j = 4 * jq + e;
                     int t = qb * 32 + 8 * jq + 4 * g + e;
-                    bool vis = (t < T_) && (key <= P + t) && (key < S);
-                    float p = vis ? exp2f((sacc[j] - lv[e]) * kLog2e) : 0.f;
+                    float p = fast_exp2(fmaf(sacc[j], kLog2e, lv[e]));
+                    if (!all_visible) {
+                        bool vis = (t < T_) && (key <= P + t) && (key < S);
+                        p = vis ? p : 0.f;
+                    }
                     float ds = p * (pacc[j] - dl[e]);
                     sacc[j] = p;
                     pacc[j] = ds;
@@ -900,6 +933,7 @@ static FwdPlan plan_fwd(const tp_attn_desc* d) {
         if (ns > 32) ns = 32;
         if (ns < 1) ns = 1;
     }
+    if (d->reserved & 0xff) ns = d->reserved & 0xff;
     p.nsplit = ns;
     return p;
 }

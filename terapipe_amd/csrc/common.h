@@ -337,6 +337,58 @@ template <typename T, int ROWS, int COLS, int NT, bool ALONG_COLS> struct Slidin
     }
 };
 
+// Tile loads for a ROWS x COLS tile (COLS = the full row of the source: no column bound) that slides
+// down the rows of a matrix: the source is a wave-uniform 64-bit base in SGPRs plus a loop-invariant
+// 32-bit per-lane byte offset, so a full tile costs no vector ALU work at all.  Rows at or beyond rmax
+// are CLAMPED to the last valid row instead of zero-filled: the caller must tolerate duplicated (finite)
+// data there -- the attention kernels do, every such row is masked.
+__device__ __forceinline__ void dma16_saddr(unsigned off, const void* sbase, const void* lds_wave_base) {
+    unsigned lds = (unsigned)(unsigned long)(__attribute__((address_space(3))) const void*)lds_wave_base;
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(off), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory");
+}
+
+template <typename T, int ROWS, int COLS, int NT> struct RowSlideDma {
+    static constexpr int CPR = COLS / 8;
+    static constexpr int TOTAL = ROWS * CPR;
+    static constexpr int N = TOTAL / NT;
+    static_assert(TOTAL % NT == 0 && NT % 64 == 0, "tile must split evenly over the waves");
+    unsigned off[N];     // byte offset of this lane's chunk from the tile's first row
+    short row[N];        // its row inside the tile
+    unsigned col_bytes[N];
+    long ld_bytes;
+
+    __device__ __forceinline__ void init(long ld_elems, int tid) {
+        const int lane = tid & 63, wave = tid >> 6;
+        ld_bytes = ld_elems * (long)sizeof(T);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int p = (i * (NT / 64) + wave) * 64 + lane;
+            const int r = p / CPR, pc = p % CPR;
+            const int lc = pc ^ swz16<COLS>(r);
+            row[i] = (short)r;
+            col_bytes[i] = (unsigned)(lc * 8 * sizeof(T));
+            off[i] = (unsigned)(r * ld_bytes) + col_bytes[i];
+        }
+    }
+    // loads the tile whose first row is row0 of the matrix at `base` (row 0 of the matrix, wave-uniform)
+    __device__ __forceinline__ void issue(T* lds, const T* base, int row0, int rmax, int tid) const {
+        const int wave = tid >> 6;
+        if (row0 + ROWS <= rmax) {
+            const char* sbase = reinterpret_cast<const char*>(base) + (long)row0 * ld_bytes;
+#pragma unroll
+            for (int i = 0; i < N; ++i) dma16_saddr(off[i], sbase, lds + (i * (NT / 64) + wave) * 512);
+        } else {
+            const int last = rmax > 0 ? rmax - 1 : 0;
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                const int r = min(row0 + (int)row[i], last);
+                dma16_saddr((unsigned)(r * ld_bytes) + col_bytes[i], base, lds + (i * (NT / 64) + wave) * 512);
+            }
+        }
+    }
+};
+
 // error plumbing shared by the host-side entry points
 void set_error(const char* fmt, ...);
 

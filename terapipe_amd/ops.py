@@ -62,6 +62,31 @@ class KernelTimer:
         return out
 
 
+class CallRecorder:
+    """Records every library call made while active as (tag, meta, replay) where replay() issues the
+    same call again on the then-current stream with the same descriptor and buffers.  bench.py replays
+    all calls of one kind back to back inside a HIP graph to time that kind of kernel without host gaps."""
+    active = None
+
+    def __init__(self):
+        self.calls = []
+
+    def __enter__(self):
+        CallRecorder.active = self
+        return self
+
+    def __exit__(self, *exc):
+        CallRecorder.active = None
+
+    def by_tag(self, tag):
+        return [c for c in self.calls if c[0] == tag]
+
+
+def _record(tag, meta, replay):
+    if CallRecorder.active is not None:
+        CallRecorder.active.calls.append((tag, meta, replay))
+
+
 class _timed:
     __slots__ = ("tag", "meta", "e0")
 
@@ -105,6 +130,9 @@ def layernorm_fwd(x2d, gamma, beta, eps=1e-5, out=None, mean=None, rstd=None):
     with _timed("layernorm_fwd", (M, E)):
         _lib.check(lib.tp_layernorm_fwd(_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps,
                                         tp_dtype(x2d.dtype), _stream()), "tp_layernorm_fwd")
+    if CallRecorder.active is not None:
+        a = (_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps, tp_dtype(x2d.dtype))
+        _record("layernorm_fwd", (M, E), lambda: lib.tp_layernorm_fwd(*a, _stream()))
     return y, mean, rstd
 
 
@@ -120,6 +148,10 @@ def layernorm_bwd(dy, x2d, mean, rstd, gamma, dres, dgamma_acc, dbeta_acc, colsu
         _lib.check(lib.tp_layernorm_bwd(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx),
                                         _p(dgamma_acc), _p(dbeta_acc), _p(colsum_dres_acc), _p(colsum_dx_acc),
                                         M, E, tp_dtype(x2d.dtype), _stream()), "tp_layernorm_bwd")
+    if CallRecorder.active is not None:
+        a = (_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx), _p(dgamma_acc), _p(dbeta_acc),
+             _p(colsum_dres_acc), _p(colsum_dx_acc), M, E, tp_dtype(x2d.dtype))
+        _record("layernorm_bwd", (M, E), lambda: lib.tp_layernorm_bwd(*a, _stream()))
     return dx
 
 
@@ -155,6 +187,9 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
     ws = Workspace.get(need, A.device) if need else None
     with _timed("gemm", (op, M, N, K)):
         _lib.check(lib.tp_gemm(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()), "tp_gemm")
+    if CallRecorder.active is not None:
+        wsp, wsn = _p(ws), (ws.numel() if ws is not None else 0)
+        _record("gemm", (op, M, N, K), lambda: lib.tp_gemm(ctypes.byref(d), wsp, wsn, _stream()))
     return C
 
 
@@ -168,7 +203,8 @@ def _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len
     return d
 
 
-def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q_scale, out=None, lse=None):
+def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q_scale, out=None, lse=None,
+                    nsplit=None):
     """q [B*H, T, Dh] (pre-scaled); caches [B*H, L, Dh] with rows [0, cache_len+T) valid.
     Returns o [T, B, H*Dh] and lse [B*H, T]."""
     _require_cuda(q, k_cache, v_cache)
@@ -176,12 +212,18 @@ def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q
     if lse is None:
         lse = torch.empty(batch * heads, T, dtype=torch.float32, device=q.device)
     d = _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale)
+    if nsplit:
+        d.reserved = int(nsplit)
     lib = _lib.load()
     need = lib.tp_attn_fwd_workspace_bytes(ctypes.byref(d))
     ws = Workspace.get(need, q.device) if need else None
     with _timed("attn_fwd", (batch, heads, head_dim, T, cache_len)):
         _lib.check(lib.tp_attn_prefix_fwd(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()),
                    "tp_attn_prefix_fwd")
+    if CallRecorder.active is not None:
+        wsp, wsn = _p(ws), (ws.numel() if ws is not None else 0)
+        _record("attn_fwd", (batch, heads, head_dim, T, cache_len),
+                lambda: lib.tp_attn_prefix_fwd(ctypes.byref(d), wsp, wsn, _stream()))
     return o, lse
 
 
@@ -201,6 +243,8 @@ def attn_prefix_bwd(q, k_cache, v_cache, o, lse, d_o, dqkv, dk_cache, dv_cache, 
     lib = _lib.load()
     with _timed("attn_bwd", (batch, heads, head_dim, T, cache_len)):
         _lib.check(lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()), "tp_attn_prefix_bwd")
+    _record("attn_bwd", (batch, heads, head_dim, T, cache_len),
+            lambda: lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()))
     return dqkv
 
 

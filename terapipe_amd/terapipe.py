@@ -76,7 +76,7 @@ class _StackBuffers:
     works on a row range of them (slice i of a [L, Bs, E] tensor is rows [P*Bs, (P+T)*Bs)), the K/V
     caches, the fp32 (or cache-dtype) gradient caches, and the parameter-gradient accumulators."""
 
-    def __init__(self, runner, dtype, device):
+    def __init__(self, runner, dtype, device, ws):
         layers = runner.layers
         nl, E, F, H = layers.n_layers, layers.embedding_dim, layers.ffn_embedding_dim, layers.num_attention_heads
         L, Dh = runner.seq_len, layers.embedding_dim // layers.num_attention_heads
@@ -106,48 +106,130 @@ class _StackBuffers:
             self.per_batch.append(b)
         self.small = torch.zeros(nl, core.small_acc_numel(E, F), **f32)
         self.small_views = [core.small_acc_views(self.small[l], E, F) for l in range(nl)]
+        # parameter-gradient results (copied out to autograd after every backward)
+        self.wgrads = [{n: torch.empty_like(ws[l][n]) for n in core.BIG_PARAMS} for l in range(nl)]
+        self.sgrads = [{n: torch.empty_like(ws[l][n]) for n in core.SMALL_PARAMS} for l in range(nl)]
+        self.param_ptrs = [t.data_ptr() for w in ws for t in w.values()]
+        self.fwd_graph = self.bwd_graph = None
+        self.states = None
+
+
+def _forward_body(runner, ws, act, bufs, states):
+    """Every (batch slice, sequence slice) through the whole layer stack, slice-major, reading the batch
+    slices from bufs x[0] and leaving the outputs in bufs x[n_layers].  Launches kernels only (no
+    allocation, no host synchronisation), so it can be recorded into a HIP graph."""
+    layers = runner.layers
+    nl, H, E = layers.n_layers, layers.num_attention_heads, layers.embedding_dim
+    for b, Bs in enumerate(runner.batch_slices):
+        pb = bufs.per_batch[b]
+        cache = pb["cache"]
+        P = 0
+        for i, T in enumerate(runner.seq_slices):
+            r0, r1 = P * Bs, (P + T) * Bs
+            sts = []
+            for l in range(nl):
+                bf = core.Bufs(xn=pb["xn"][l][r0:r1], mean1=pb["mean1"][l][r0:r1], rstd1=pb["rstd1"][l][r0:r1],
+                               q=pb["q"][l][r0:r1].view(Bs * H, T, E // H), o=pb["o"][l][r0:r1].view(T, Bs, E),
+                               lse=pb["lse"][l][r0 * H:r1 * H].view(Bs * H, T), h=pb["h"][l][r0:r1],
+                               mean2=pb["mean2"][l][r0:r1], rstd2=pb["rstd2"][l][r0:r1], hn=pb["hn"][l][r0:r1],
+                               a=pb["a"][l][r0:r1], z=None if pb["z"][l] is None else pb["z"][l][r0:r1],
+                               out=pb["x"][l + 1][r0:r1])
+                _, st = core.layer_fwd(ws[l], pb["x"][l][r0:r1].view(T, Bs, E), H, cache[2 * l], cache[2 * l + 1],
+                                       P, act[l], need_state=True, buf=bf)
+                sts.append(st)
+            states[b, i] = sts
+            P += T                                                               # terapipe.py:264
+
+
+def _backward_body(runner, ws, act, bufs, states):
+    """Reverse-order slices (terapipe.py:182-191 of the reference) reading the output gradient from bufs
+    dx[n_layers], then one weight-gradient GEMM per weight and one reduction per vector parameter over
+    all tokens, into bufs.wgrads / bufs.sgrads.  Launches kernels only."""
+    layers = runner.layers
+    nl, H = layers.n_layers, layers.num_attention_heads
+    E, F = layers.embedding_dim, layers.ffn_embedding_dim
+    nb, ns = len(runner.batch_slices), len(runner.seq_slices)
+    L = runner.seq_len
+    ops.zero_(bufs.small)
+    for b in reversed(range(nb)):
+        Bs = runner.batch_slices[b]
+        pb = bufs.per_batch[b]
+        gc = pb["gcache"]
+        P = L
+        for i in reversed(range(ns)):
+            T = runner.seq_slices[i]
+            P -= T
+            r0, r1 = P * Bs, (P + T) * Bs
+            last = i == ns - 1
+            for l in reversed(range(nl)):
+                bf = core.Bufs(dz1=pb["dz1"][l][r0:r1], dhn=pb["dhn"][l][r0:r1], dh=pb["dh"][l][r0:r1],
+                               d_o=pb["d_o"][:T * Bs], dqkv=pb["dqkv"][l][r0:r1], dxn=pb["dxn"][l][r0:r1],
+                               dx=pb["dx"][l][r0:r1], delta=pb["delta"][:T * Bs * H].view(Bs * H, T))
+                # the gradient caches need no zero fill: the last slice (processed first) writes every
+                # prefix row with '=', the earlier ones add to rows that were written before
+                core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), H,
+                               gc[2 * l], gc[2 * l + 1], None, False, None, accumulate_prefix=not last,
+                               has_incoming=not last, zero_slice_rows=False, activation=act[l], buf=bf)
+    # parameter gradients over all tokens: dW = dY_all^T X_all (one GEMM per weight and batch slice),
+    # bias gradients = column sums of dY_all, LayerNorm gradients from (dy, x, mean, rstd) of all rows
+    for l in range(nl):
+        sv = bufs.small_views[l]
+        g = bufs.wgrads[l]
+        for bi, pb in enumerate(bufs.per_batch):
+            R = L * runner.batch_slices[bi]
+            epi = TP_EPI_STORE if bi == 0 else TP_EPI_ACCUMULATE
+            dy_out = pb["dx"][l + 1]
+            ops.gemm(TP_GEMM_TN, pb["dqkv"][l], pb["xn"][l], 3 * E, E, R, C=g["attn.in_proj.weight"], epilogue=epi)
+            ops.gemm(TP_GEMM_TN, pb["dh"][l], pb["o"][l], E, E, R, C=g["attn.out_proj.weight"], epilogue=epi)
+            ops.gemm(TP_GEMM_TN, pb["dz1"][l], pb["hn"][l], F, E, R, C=g["fc1.weight"], epilogue=epi)
+            ops.gemm(TP_GEMM_TN, dy_out, pb["a"][l], E, F, R, C=g["fc2.weight"], epilogue=epi)
+            ops.colsum_acc(pb["dqkv"][l], sv["attn.in_proj.bias"])
+            ops.colsum_acc(pb["dh"][l], sv["attn.out_proj.bias"])
+            ops.colsum_acc(pb["dz1"][l], sv["fc1.bias"])
+            ops.colsum_acc(dy_out, sv["fc2.bias"])
+            ops.ln_param_grads(pb["dxn"][l], pb["x"][l], pb["mean1"][l], pb["rstd1"][l], sv["attn_ln.weight"],
+                               sv["attn_ln.bias"])
+            ops.ln_param_grads(pb["dhn"][l], pb["h"][l], pb["mean2"][l], pb["rstd2"][l], sv["fc_ln.weight"],
+                               sv["fc_ln.bias"])
+        for n in core.SMALL_PARAMS:
+            ops.accum_cast(bufs.sgrads[l][n], sv[n], False)
+
+
+def _capture(fn):
+    """Records fn()'s kernel launches into a HIP graph (after the caller has run fn() eagerly once, so
+    that every buffer and workspace already exists)."""
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    return g
 
 
 class _TeraPipeFunction(torch.autograd.Function):
-    """forward: every (batch slice, sequence slice) through the whole layer stack, slice-major.
-    backward: reverse-order slices (terapipe.py:182-191 of the reference), then one weight-gradient
-    GEMM per weight and one reduction per vector parameter over all tokens."""
+    """One autograd node around the whole slice grid (see _forward_body / _backward_body)."""
 
     @staticmethod
     def forward(ctx, runner, inputs, *flat_params):
         layers = runner.layers
-        nl, heads = layers.n_layers, layers.num_attention_heads
-        E, H = layers.embedding_dim, heads
+        nl, E = layers.n_layers, layers.embedding_dim
         ws = [dict(zip(core.PARAM_NAMES, flat_params[12 * i:12 * i + 12])) for i in range(nl)]
         act = [l.activation for l in layers.layers]
-        bufs = runner._stack_buffers(inputs.dtype, inputs.device)
+        bufs = runner._stack_buffers(inputs.dtype, inputs.device, ws)
         nb, ns = len(runner.batch_slices), len(runner.seq_slices)
-        states = np.empty((nb, ns), dtype="O")
         b0 = 0
-        for b in range(nb):
-            Bs = runner.batch_slices[b]
-            pb = bufs.per_batch[b]
+        for b, Bs in enumerate(runner.batch_slices):
             # the batch slice as [L*Bs, E] rows (t, b_local): a copy, as grid_slice_batch_and_sequence makes
-            pb["x"][0].view(runner.seq_len, Bs, E).copy_(inputs[:, b0:b0 + Bs, :])
-            cache = pb["cache"]
-            P = 0
-            for i in range(ns):
-                T = runner.seq_slices[i]
-                r0, r1 = P * Bs, (P + T) * Bs
-                sts = []
-                for l in range(nl):
-                    bf = core.Bufs(xn=pb["xn"][l][r0:r1], mean1=pb["mean1"][l][r0:r1], rstd1=pb["rstd1"][l][r0:r1],
-                                   q=pb["q"][l][r0:r1].view(Bs * H, T, E // H), o=pb["o"][l][r0:r1].view(T, Bs, E),
-                                   lse=pb["lse"][l][r0 * H:r1 * H].view(Bs * H, T), h=pb["h"][l][r0:r1],
-                                   mean2=pb["mean2"][l][r0:r1], rstd2=pb["rstd2"][l][r0:r1], hn=pb["hn"][l][r0:r1],
-                                   a=pb["a"][l][r0:r1], z=None if pb["z"][l] is None else pb["z"][l][r0:r1],
-                                   out=pb["x"][l + 1][r0:r1])
-                    _, st = core.layer_fwd(ws[l], pb["x"][l][r0:r1].view(T, Bs, E), heads, cache[2 * l],
-                                           cache[2 * l + 1], P, act[l], need_state=True, buf=bf)
-                    sts.append(st)
-                states[b, i] = sts
-                P += T                                                               # terapipe.py:264
+            bufs.per_batch[b]["x"][0].view(runner.seq_len, Bs, E).copy_(inputs[:, b0:b0 + Bs, :])
             b0 += Bs
+        if runner.use_hip_graph and bufs.fwd_graph is not None:
+            bufs.fwd_graph.replay()
+            states = bufs.states
+        else:
+            states = np.empty((nb, ns), dtype="O")
+            _forward_body(runner, ws, act, bufs, states)
+            if runner.use_hip_graph:
+                bufs.states = states
+                bufs.fwd_graph = _capture(lambda: _forward_body(runner, ws, act, bufs, np.empty((nb, ns), dtype="O")))
         runner.last_caches = [pb["cache"] for pb in bufs.per_batch]
         if runner.keep_states:
             runner.last_states = states.copy()
@@ -163,63 +245,27 @@ class _TeraPipeFunction(torch.autograd.Function):
     def backward(ctx, grad_y):
         runner, ws, act, states, bufs = ctx.runner, ctx.ws, ctx.act, ctx.states, ctx.bufs
         layers = runner.layers
-        nl, heads = layers.n_layers, layers.num_attention_heads
-        E, F, H = layers.embedding_dim, layers.ffn_embedding_dim, heads
-        nb, ns = len(runner.batch_slices), len(runner.seq_slices)
+        nl, E = layers.n_layers, layers.embedding_dim
         L = runner.seq_len
-        ops.zero_(bufs.small)
-        b0 = sum(runner.batch_slices)
-        for b in reversed(range(nb)):
-            Bs = runner.batch_slices[b]
-            b0 -= Bs
-            pb = bufs.per_batch[b]
-            pb["dx"][nl].view(L, Bs, E).copy_(grad_y[:, b0:b0 + Bs, :])
-            gc = pb["gcache"]
-            P = L
-            for i in reversed(range(ns)):
-                T = runner.seq_slices[i]
-                P -= T
-                r0, r1 = P * Bs, (P + T) * Bs
-                last = i == ns - 1
-                for l in reversed(range(nl)):
-                    bf = core.Bufs(dz1=pb["dz1"][l][r0:r1], dhn=pb["dhn"][l][r0:r1], dh=pb["dh"][l][r0:r1],
-                                   d_o=pb["d_o"][:T * Bs], dqkv=pb["dqkv"][l][r0:r1], dxn=pb["dxn"][l][r0:r1],
-                                   dx=pb["dx"][l][r0:r1], delta=pb["delta"][:T * Bs * H].view(Bs * H, T))
-                    # the gradient caches need no zero fill: the last slice (processed first) writes every
-                    # prefix row with '=', the earlier ones add to rows that were written before
-                    core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), heads,
-                                   gc[2 * l], gc[2 * l + 1], None, False, None, accumulate_prefix=not last,
-                                   has_incoming=not last, zero_slice_rows=False, activation=act[l], buf=bf)
-        # parameter gradients over all tokens: dW = dY_all^T X_all (one GEMM per weight and batch slice),
-        # bias gradients = column sums of dY_all, LayerNorm gradients from (dy, x, mean, rstd) of all rows
+        b0 = 0
+        for b, Bs in enumerate(runner.batch_slices):
+            bufs.per_batch[b]["dx"][nl].view(L, Bs, E).copy_(grad_y[:, b0:b0 + Bs, :])
+            b0 += Bs
+        if runner.use_hip_graph and bufs.bwd_graph is not None:
+            bufs.bwd_graph.replay()
+        else:
+            _backward_body(runner, ws, act, bufs, states)
+            if runner.use_hip_graph:
+                bufs.bwd_graph = _capture(lambda: _backward_body(runner, ws, act, bufs, states))
+        # the gradient buffers are reused by the next step: hand autograd copies
         grads = []
         for l in range(nl):
-            sv = bufs.small_views[l]
-            g = {n: torch.empty_like(ws[l][n]) for n in core.BIG_PARAMS}
-            for bi, pb in enumerate(bufs.per_batch):
-                R = L * runner.batch_slices[bi]
-                epi = TP_EPI_STORE if bi == 0 else TP_EPI_ACCUMULATE
-                dy_out = pb["dx"][l + 1]
-                ops.gemm(TP_GEMM_TN, pb["dqkv"][l], pb["xn"][l], 3 * E, E, R, C=g["attn.in_proj.weight"], epilogue=epi)
-                ops.gemm(TP_GEMM_TN, pb["dh"][l], pb["o"][l], E, E, R, C=g["attn.out_proj.weight"], epilogue=epi)
-                ops.gemm(TP_GEMM_TN, pb["dz1"][l], pb["hn"][l], F, E, R, C=g["fc1.weight"], epilogue=epi)
-                ops.gemm(TP_GEMM_TN, dy_out, pb["a"][l], E, F, R, C=g["fc2.weight"], epilogue=epi)
-                ops.colsum_acc(pb["dqkv"][l], sv["attn.in_proj.bias"])
-                ops.colsum_acc(pb["dh"][l], sv["attn.out_proj.bias"])
-                ops.colsum_acc(pb["dz1"][l], sv["fc1.bias"])
-                ops.colsum_acc(dy_out, sv["fc2.bias"])
-                ops.ln_param_grads(pb["dxn"][l], pb["x"][l], pb["mean1"][l], pb["rstd1"][l], sv["attn_ln.weight"],
-                                   sv["attn_ln.bias"])
-                ops.ln_param_grads(pb["dhn"][l], pb["h"][l], pb["mean2"][l], pb["rstd2"][l], sv["fc_ln.weight"],
-                                   sv["fc_ln.bias"])
-            for n in core.SMALL_PARAMS:
-                t = torch.empty_like(ws[l][n])
-                ops.accum_cast(t, sv[n], False)
-                g[n] = t
-            grads += [g[n] for n in core.PARAM_NAMES]
+            for n in core.PARAM_NAMES:
+                src = bufs.wgrads[l][n] if n in bufs.wgrads[l] else bufs.sgrads[l][n]
+                grads.append(src.clone())
         dinputs = None
         if ctx.needs_input_grad[1]:
-            if nb == 1:
+            if len(runner.batch_slices) == 1:
                 dinputs = bufs.per_batch[0]["dx"][0].view(L, runner.batch_slices[0], E).clone()
             else:
                 dinputs = torch.cat([pb["dx"][0].view(L, Bs, E)
@@ -239,10 +285,14 @@ class TeraPipe(nn.Module):
     layer-level autograd surface in transformer_models.py accumulates per slice instead).
     fp32_grad_cache: keep the cross-slice dK/dV accumulators in fp32 (one rounding when a slice's own
     rows are emitted) instead of the cache dtype the reference uses.
+    use_hip_graph: after the first (eager) step, record the kernel launches of forward and of backward
+    into two HIP graphs and replay them on later steps.  The runner's buffers are static and the
+    launches depend only on shapes, so the replays compute the same thing without the per-launch host
+    work; parameters must keep their storage (in-place optimizer updates are fine).
     """
 
     def __init__(self, layers, batch_size, seq_len, batch_slices, seq_slices, batch_dim=1, sequence_dim=0,
-                 fp32_grad_cache=True):
+                 fp32_grad_cache=True, use_hip_graph=False):
         super().__init__()
         assert sum(batch_slices) == batch_size and sum(seq_slices) == seq_len
         assert batch_dim == 1 and sequence_dim == 0, "layers take [seq, batch, embed] inputs"
@@ -251,6 +301,7 @@ class TeraPipe(nn.Module):
         self.batch_dim, self.sequence_dim = batch_dim, sequence_dim
         self.layers = layers
         self.fp32_grad_cache = fp32_grad_cache
+        self.use_hip_graph = use_hip_graph
         self._sbufs = None
         self.last_caches = None
         self.keep_states = False   # debugging / tests: keep the per-slice saved activations of the last forward
@@ -264,9 +315,11 @@ class TeraPipe(nn.Module):
     def n_input_slices(self):
         return len(self.seq_slices)
 
-    def _stack_buffers(self, dtype, device):
-        if self._sbufs is None or self._sbufs.dtype != dtype or self._sbufs.device != device:
-            self._sbufs = _StackBuffers(self, dtype, device)
+    def _stack_buffers(self, dtype, device, ws):
+        ptrs = [t.data_ptr() for w in ws for t in w.values()]
+        if (self._sbufs is None or self._sbufs.dtype != dtype or self._sbufs.device != device
+                or self._sbufs.param_ptrs != ptrs):     # recorded graphs hold the parameter addresses
+            self._sbufs = _StackBuffers(self, dtype, device, ws)
         return self._sbufs
 
     def forward(self, inputs=None):
