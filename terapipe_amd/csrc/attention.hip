@@ -891,6 +891,737 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_dma_kernel(AttnArgs a) 
     }
 }
 
+// Workgroups are dealt to the eight XCDs round-robin by linear id.  This maps the linear id to
+// (batch*head, block) so that all blocks of one (batch, head) run on the same XCD and its K / V / Q / dO
+// rows are fetched into one L2 only.  Launch with xcd_grid(BH, nblocks) workgroups; false = no work.
+__device__ __forceinline__ bool xcd_map(int BH, int& bh, int& blk) {
+    const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+    const int nbh8 = (BH + 7) >> 3;
+    bh = xcd + 8 * (slot % nbh8);
+    blk = slot / nbh8;
+    return bh < BH;
+}
+static inline unsigned xcd_grid(int BH, int nblocks) { return 8u * ((BH + 7) / 8) * nblocks; }
+
+// ---- shared pieces of the second-generation 16-bit attention kernels -------------------------------
+
+// Wave-private transpose of a [DH x 32] fp32 accumulator set (register j of block db = row db*32 +
+// acc_row(j, g), column lane & 31) into row-major [32][DH] through LDS, so that global memory is then
+// touched in full rows.  `buf` is the wave's own 32 x (DH + 4) floats.  After the call lane l holds, for
+// i in [0, DH / 8): row 2 * i' ... see rows_read.
+template <int DH>
+__device__ __forceinline__ void acc_to_lds_rows(const float16v* acc, float* buf, int lane) {
+    constexpr int NDB = DH / 32, LD = DH + 4;
+    const int g = lane >> 5, li = lane & 31;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int jq = 0; jq < 4; ++jq)
+            *reinterpret_cast<float4*>(buf + li * LD + db * 32 + 8 * jq + 4 * g) =
+                make_float4(acc[db][4 * jq], acc[db][4 * jq + 1], acc[db][4 * jq + 2], acc[db][4 * jq + 3]);
+}
+// piece i of the row-major read-back: row and first column of the four floats this lane gets
+template <int DH> __device__ __forceinline__ void row_piece(int i, int lane, int& row, int& col) {
+    constexpr int LPR = DH / 4;            // lanes per row
+    const int idx = i * 64 + lane;
+    row = idx / LPR;
+    col = (idx % LPR) * 4;
+}
+
+// dK / dV, second generation: stage-unrolled ring (LDS addresses are lane constants plus immediates),
+// scalar-base tile loads, row-contiguous epilogue.
+template <typename T, typename GT, int DH, int NW, int STAGES>
+__global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv2_kernel(AttnArgs a) {
+    typedef Elem<T> E;
+    static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
+    constexpr int NDB = DH / 32, NKS = DH / 16;
+    constexpr int TILE = 32 * DH;                       // elements of one Q or dO tile
+    constexpr int CPR = DH / 8;                         // 16-byte chunks per row
+    constexpr int NLD = 32 * CPR / (NW * 64);           // loads per thread per tile
+    static_assert(32 * CPR % (NW * 64) == 0, "tile must split evenly");
+    constexpr int NLOAD = 2 * NLD;
+    static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
+    constexpr int RING_BYTES = STAGES * 2 * TILE * 2;
+    constexpr int EPI_LD = DH + 4;
+    constexpr int EPI_BYTES = NW * 32 * EPI_LD * 4;
+    constexpr int SMEM = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM];
+    extern __shared__ __attribute__((aligned(16))) float stats[];   // -lse*log2e [Tpad], delta[Tpad]
+    T* ring = reinterpret_cast<T*>(smem);
+    const unsigned ring_lds = lds_addr(smem);
+
+    const int tid = threadIdx.x, lane = tid & 63, g = lane >> 5, li = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int bh, kblk;
+    if (!xcd_map(a.B * a.H, bh, kblk)) return;
+    const int b = bh / a.H, h = bh - b * a.H;
+    const int T_ = a.T, P = a.P, S = a.P + a.T;
+    const long EE = (long)a.H * DH;
+    const int key0wg = kblk * NW * 32;
+    const int key0w = key0wg + wave * 32;
+    const int key = key0w + li;
+    const int nqb = (T_ + 31) / 32;
+    const int Tpad = nqb * 32;
+    float* sLse = stats;
+    float* sDelta = stats + Tpad;
+
+    typename E::opnd_t kreg[NKS], vreg[NKS];
+    load_row_operands<T, DH>(kreg, reinterpret_cast<const T*>(a.kc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
+    load_row_operands<T, DH>(vreg, reinterpret_cast<const T*>(a.vc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
+    for (int t = tid; t < Tpad; t += NW * 64) {
+        sLse[t] = t < T_ ? -a.lse[(long)bh * T_ + t] * kLog2e : 0.f;
+        sDelta[t] = t < T_ ? a.delta[(long)bh * T_ + t] : 0.f;
+    }
+
+    // lane-constant LDS addresses inside stage 0's Q tile (the dO tile and the other stages are
+    // compile-time offsets from these)
+    const T* pkm[NKS];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) pkm[ks] = ring + km_offset<T, DH>(li, ks * 16, lane);
+    const T* ptr0[NDB];
+    const T* ptr1[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+        int o0, o1;
+        tr_offsets<T, DH, true>(0, db * 32, lane, o0, o1);
+        ptr0[db] = ring + o0;
+        ptr1[db] = ring + o1;
+    }
+    // tile loads: per-lane byte offsets from the tile's first row
+    unsigned qoff[NLD], dooff[NLD];
+    const unsigned ldo_bytes = (unsigned)((long)a.B * EE * 2);
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int p = (i * NW + wave) * 64 + lane;
+        const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+        qoff[i] = (unsigned)(r * DH * 2 + lc * 16);
+        dooff[i] = (unsigned)(r * ldo_bytes + lc * 16);
+    }
+    const char* Qb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.q) + (long)bh * T_ * DH));
+    const char* dOb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.d_o) + (long)b * EE + (long)h * DH));
+    const int qb_start = key0wg > P ? (key0wg - P) / 32 : 0;
+    const int nt = nqb - qb_start;
+
+    wait_vmcnt<0>();
+    __syncthreads();
+
+    auto issue = [&](int stage, int it) {
+        // query rows past T are clamped to row T-1: finite data whose P and dS are forced to zero
+        const unsigned dq_ = ring_lds + (unsigned)(stage * 2 * TILE * 2 + wave * 1024);   // this wave's 1 KB of load 0
+        const int row0 = (qb_start + it) * 32;
+        if (row0 + 32 <= T_) {
+            const char* sq = Qb + (long)row0 * (DH * 2);
+            const char* sd = dOb + (long)row0 * ldo_bytes;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) dma16_saddr_lds(qoff[i], sq, dq_ + i * NW * 1024);
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) dma16_saddr_lds(dooff[i], sd, dq_ + TILE * 2 + i * NW * 1024);
+        } else {
+            const int last = T_ - 1;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int p = (i * NW + wave) * 64 + lane;
+                const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+                const int rr = min(row0 + r, last);
+                dma16_saddr_lds((unsigned)(rr * DH * 2 + lc * 16), Qb, dq_ + i * NW * 1024);
+            }
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int p = (i * NW + wave) * 64 + lane;
+                const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+                const int rr = min(row0 + r, last);
+                dma16_saddr_lds((unsigned)(rr * ldo_bytes + lc * 16), dOb, dq_ + TILE * 2 + i * NW * 1024);
+            }
+        }
+    };
+
+    float16v dk[NDB], dv[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
+
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) issue(s, s);
+
+    for (int it0 = 0; it0 < nt; it0 += STAGES) {
+#pragma unroll
+        for (int s = 0; s < STAGES; ++s) {
+            const int it = it0 + s;
+            if (it < nt) {
+                wait_vmcnt<NLOAD * (STAGES - 2)>();
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                issue((s + STAGES - 1) % STAGES, it + STAGES - 1);
+                const int so = s * 2 * TILE;              // compile-time after unrolling
+                const int qb = qb_start + it;
+                if (key0w < S && key0w <= P + qb * 32 + 31) {
+                    typename E::opnd_t qop[NKS], doop[NKS];
+#pragma unroll
+                    for (int ks = 0; ks < NKS; ++ks) {
+                        qop[ks] = load_km<T>(pkm[ks] + so);
+                        doop[ks] = load_km<T>(pkm[ks] + so + TILE);
+                    }
+                    float4 l4[4], d4[4];
+#pragma unroll
+                    for (int jq = 0; jq < 4; ++jq) {
+                        l4[jq] = *reinterpret_cast<const float4*>(sLse + qb * 32 + 8 * jq + 4 * g);
+                        d4[jq] = *reinterpret_cast<const float4*>(sDelta + qb * 32 + 8 * jq + 4 * g);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    float16v sacc, pacc;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+                    for (int ks = 0; ks < NKS; ++ks) {
+                        sacc = E::mfma(qop[ks], kreg[ks], sacc);
+                        pacc = E::mfma(doop[ks], vreg[ks], pacc);
+                    }
+                    // wave-uniform: every (query, key) pair of the block is visible and in range
+                    const bool all_visible = (qb * 32 + 32 <= T_) && (key0w + 31 <= P + qb * 32) && (key0w + 32 <= S);
+                    float pv[16], dsv[16];
+                    if (all_visible) {
+#pragma unroll
+                        for (int jq = 0; jq < 4; ++jq) {
+                            const float lv[4] = {l4[jq].x, l4[jq].y, l4[jq].z, l4[jq].w};
+                            const float dl[4] = {d4[jq].x, d4[jq].y, d4[jq].z, d4[jq].w};
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const int j = 4 * jq + e;
+                                const float p = fast_exp2(fmaf(sacc[j], kLog2e, lv[e]));
+                                pv[j] = p;
+                                dsv[j] = p * (pacc[j] - dl[e]);
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int jq = 0; jq < 4; ++jq) {
+                            const float lv[4] = {l4[jq].x, l4[jq].y, l4[jq].z, l4[jq].w};
+                            const float dl[4] = {d4[jq].x, d4[jq].y, d4[jq].z, d4[jq].w};
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const int j = 4 * jq + e;
+                                const int t = qb * 32 + 8 * jq + 4 * g + e;
+                                const bool vis = (t < T_) && (key <= P + t) && (key < S);
+                                const float p = vis ? fast_exp2(fmaf(sacc[j], kLog2e, lv[e])) : 0.f;
+                                pv[j] = p;
+                                dsv[j] = p * (pacc[j] - dl[e]);
+                            }
+                        }
+                    }
+                    uint4 pop[2], dsop[2];
+                    pop[0] = pack8<T>(pv); pop[1] = pack8<T>(pv + 8);
+                    dsop[0] = pack8<T>(dsv); dsop[1] = pack8<T>(dsv + 8);
+                    // dV^T += dO^T P, dK^T += Q^T dS: all sixteen transposed operand fetches first
+                    uint4 ado[2][NDB], aq[2][NDB];
+#pragma unroll
+                    for (int hs = 0; hs < 2; ++hs)
+#pragma unroll
+                        for (int db = 0; db < NDB; ++db) {
+                            ado[hs][db] = load_tr<T>(ptr0[db] + so + TILE + hs * 16 * DH, ptr1[db] + so + TILE + hs * 16 * DH);
+                            aq[hs][db] = load_tr<T>(ptr0[db] + so + hs * 16 * DH, ptr1[db] + so + hs * 16 * DH);
+                        }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int hs = 0; hs < 2; ++hs)
+#pragma unroll
+                        for (int db = 0; db < NDB; ++db) {
+                            dv[db] = E::mfma(ado[hs][db], pop[hs], dv[db]);
+                            dk[db] = E::mfma(aq[hs][db], dsop[hs], dk[db]);
+                        }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            }
+        }
+    }
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();      // every wave is done with the ring: reuse it for the epilogue
+    asm volatile("" ::: "memory");
+
+    float* ebuf = reinterpret_cast<float*>(smem) + wave * 32 * EPI_LD;
+    GT* gKb = reinterpret_cast<GT*>(a.gk) + ((long)bh * a.cache_rows + key0w) * DH;
+    GT* gVb = reinterpret_cast<GT*>(a.gv) + ((long)bh * a.cache_rows + key0w) * DH;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        acc_to_lds_rows<DH>(which == 0 ? dk : dv, ebuf, lane);
+        GT* gb = which == 0 ? gKb : gVb;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        constexpr int NP = 32 * DH / 256;
+        float4 val[NP];
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            int row, col;
+            row_piece<DH>(i, lane, row, col);
+            val[i] = *reinterpret_cast<const float4*>(ebuf + row * EPI_LD + col);
+        }
+        // incoming gradient of these rows (prefix rows: the accumulator itself; slice rows: what the later
+        // slices left in the gradient cache)
+        float old[NP][4];
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            int row, col;
+            row_piece<DH>(i, lane, row, col);
+            const int kk = key0w + row;
+            old[i][0] = old[i][1] = old[i][2] = old[i][3] = 0.f;
+            const bool rd = kk < S && (kk < P ? a.accumulate_prefix != 0 : a.has_incoming != 0);
+            if (rd) load4<GT>(gb + (long)row * DH + col, old[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            int row, col;
+            row_piece<DH>(i, lane, row, col);
+            const int kk = key0w + row;
+            if (kk < S) {
+                const float r0 = old[i][0] + val[i].x, r1 = old[i][1] + val[i].y, r2 = old[i][2] + val[i].z,
+                            r3 = old[i][3] + val[i].w;
+                if (kk < P) {
+                    store4<GT>(gb + (long)row * DH + col, r0, r1, r2, r3);
+                } else {
+                    T* dst = reinterpret_cast<T*>(a.dqkv) + ((long)(kk - P) * a.B + b) * (3 * EE) + (long)h * 3 * DH +
+                             (which + 1) * DH + col;
+                    store4<T>(dst, r0, r1, r2, r3);
+                    if (a.zero_slice_rows) store4<GT>(gb + (long)row * DH + col, 0.f, 0.f, 0.f, 0.f);
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the buffer is rewritten by the next pass
+    }
+}
+
+// dQ, second generation.  A workgroup owns 32 queries of one (batch, head); its NW waves split the key
+// range, each streaming its own K / V tiles of 32 keys through a private two-stage LDS ring (no
+// workgroup barrier inside the loop), and the NW partial dQ blocks are summed through LDS at the end.
+// The kernel also computes delta = rowsum(dO * O) for its queries and leaves it in a.delta for the
+// dK/dV kernel that follows on the stream.
+template <typename T, int DH, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_bwd_dq2_kernel(AttnArgs a) {
+    typedef Elem<T> E;
+    static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
+    constexpr int NDB = DH / 32, NKS = DH / 16;
+    constexpr int TILE = 32 * DH;                       // elements of one K or V tile
+    constexpr int CPR = DH / 8;
+    constexpr int NLD = 32 * CPR / 64;                  // loads per lane per tile (one wave loads a whole tile)
+    constexpr int NLOAD = 2 * NLD;
+    static_assert(NLOAD <= 63, "too many loads in flight for vmcnt");
+    constexpr int WAVE_RING = 2 * 2 * TILE * 2;         // bytes: two stages of K + V
+    constexpr int EPI_LD = DH + 4;
+    constexpr int EPI_BYTES = NW * 32 * EPI_LD * 4;
+    constexpr int SMEM = NW * WAVE_RING > EPI_BYTES ? NW * WAVE_RING : EPI_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM];
+
+    const int tid = threadIdx.x, lane = tid & 63, g = lane >> 5, li = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int bh, qblk;
+    if (!xcd_map(a.B * a.H, bh, qblk)) return;
+    const int b = bh / a.H, h = bh - b * a.H;
+    const int T_ = a.T, P = a.P, S = a.P + a.T;
+    const long EE = (long)a.H * DH;
+    const int q0 = ((T_ + 31) / 32 - 1 - qblk) * 32;     // the blocks with the longest key range start first
+    const int tq = q0 + li;
+    const bool qok = tq < T_;
+    const int kv_end = P + min(T_, q0 + 32);
+    const int ntiles = (kv_end + 31) / 32;
+    const int tpw = (ntiles + NW - 1) / NW;
+    const int t_beg = wave * tpw, t_end = min(ntiles, t_beg + tpw);
+    const int nt = max(t_end - t_beg, 0);
+
+    T* ring = reinterpret_cast<T*>(smem) + wave * (WAVE_RING / 2);
+    const unsigned ring_lds = lds_addr(smem) + wave * WAVE_RING;
+
+    typename E::opnd_t qreg[NKS], doreg[NKS];
+    const long orow = ((long)tq * a.B + b) * EE + (long)h * DH;
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * T_ + tq) * DH, qok, g);
+    load_row_operands<T, DH>(doreg, reinterpret_cast<const T*>(a.d_o) + orow, qok, g);
+    float delta_q;
+    {
+        typename E::opnd_t oreg[NKS];
+        load_row_operands<T, DH>(oreg, reinterpret_cast<const T*>(a.o) + orow, qok, g);
+        float s = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            const T* x = reinterpret_cast<const T*>(&oreg[ks]);
+            const T* y = reinterpret_cast<const T*>(&doreg[ks]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s = fmaf(E::to_float(x[e]), E::to_float(y[e]), s);
+        }
+        delta_q = s + __shfl_xor(s, 32, 64);
+    }
+    if (wave == 0 && g == 0 && qok) a.delta[(long)bh * T_ + tq] = delta_q;
+    const float lse_neg = qok ? -a.lse[(long)bh * T_ + tq] * kLog2e : 0.f;
+
+    // lane-constant LDS addresses inside stage 0's K tile
+    const T* pkm[NKS];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) pkm[ks] = ring + km_offset<T, DH>(li, ks * 16, lane);
+    const T* ptr0[NDB];
+    const T* ptr1[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+        int o0, o1;
+        tr_offsets<T, DH, true>(0, db * 32, lane, o0, o1);
+        ptr0[db] = ring + o0;
+        ptr1[db] = ring + o1;
+    }
+    unsigned koff[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int p = i * 64 + lane;
+        const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+        koff[i] = (unsigned)(r * DH * 2 + lc * 16);
+    }
+    const char* Kb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.kc) + (long)bh * a.cache_rows * DH));
+    const char* Vb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.vc) + (long)bh * a.cache_rows * DH));
+
+    auto issue = [&](int stage, int tile) {
+        // rows at or past S are clamped to row S-1: finite data, and every such key is masked
+        const unsigned dst = ring_lds + (unsigned)(stage * 2 * TILE * 2);
+        const int row0 = tile * 32;
+        if (row0 + 32 <= S) {
+            const char* sk = Kb + (long)row0 * (DH * 2);
+            const char* sv = Vb + (long)row0 * (DH * 2);
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) dma16_saddr_lds(koff[i], sk, dst + i * 1024);
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) dma16_saddr_lds(koff[i], sv, dst + TILE * 2 + i * 1024);
+        } else {
+            const int last = S - 1;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int p = i * 64 + lane;
+                const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+                const unsigned off = (unsigned)(min(row0 + r, last) * DH * 2 + lc * 16);
+                dma16_saddr_lds(off, Kb, dst + i * 1024);
+            }
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int p = i * 64 + lane;
+                const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+                const unsigned off = (unsigned)(min(row0 + r, last) * DH * 2 + lc * 16);
+                dma16_saddr_lds(off, Vb, dst + TILE * 2 + i * 1024);
+            }
+        }
+    };
+
+    float16v dq[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
+
+    wait_vmcnt<0>();                     // the row operands are in; tile loads are counted from here
+    if (nt > 0) issue(0, t_beg);
+    auto step = [&](auto stage_c, int it) {
+        constexpr int s = decltype(stage_c)::value;
+        // the other stage was last read one iteration ago (lgkmcnt(0) below): refill it, then wait
+        // for this iteration's tile (all but the NLOAD loads just issued)
+        if (it + 1 < nt) {
+            issue(s ^ 1, t_beg + it + 1);
+            wait_vmcnt<NLOAD>();
+        } else {
+            wait_vmcnt<0>();
+        }
+        const int so = s * 2 * TILE;
+        const int key0 = (t_beg + it) * 32;
+        typename E::opnd_t kop[NKS], vop[NKS];
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            kop[ks] = load_km<T>(pkm[ks] + so);
+            vop[ks] = load_km<T>(pkm[ks] + so + TILE);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        float16v sacc, pacc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            sacc = E::mfma(kop[ks], qreg[ks], sacc);
+            pacc = E::mfma(vop[ks], doreg[ks], pacc);
+        }
+        float dsv[16];
+        if (key0 + 31 > P + q0) {        // wave-uniform: the tile touches the causal boundary
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int key = key0 + acc_row(j, g);
+                const float p = key > P + tq ? 0.f : fast_exp2(fmaf(sacc[j], kLog2e, lse_neg));
+                dsv[j] = p * (pacc[j] - delta_q);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const float p = fast_exp2(fmaf(sacc[j], kLog2e, lse_neg));
+                dsv[j] = p * (pacc[j] - delta_q);
+            }
+        }
+        uint4 dsop[2];
+        dsop[0] = pack8<T>(dsv);
+        dsop[1] = pack8<T>(dsv + 8);
+        uint4 ak[2][NDB];
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+                ak[hs][db] = load_tr<T>(ptr0[db] + so + hs * 16 * DH, ptr1[db] + so + hs * 16 * DH);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) dq[db] = E::mfma(ak[hs][db], dsop[hs], dq[db]);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    {
+        int it = 0;
+        for (; it + 1 < nt; it += 2) {
+            step(std::integral_constant<int, 0>(), it);
+            step(std::integral_constant<int, 1>(), it + 1);
+        }
+        if (it < nt) step(std::integral_constant<int, 0>(), it);
+    }
+    wait_vmcnt<0>();
+    __syncthreads();       // every wave is done with its ring: the space is reused for the reduction
+
+    float* ebuf = reinterpret_cast<float*>(smem);
+    acc_to_lds_rows<DH>(dq, ebuf + wave * 32 * EPI_LD, lane);
+    __syncthreads();
+    // thread -> (row, 16 consecutive columns) for DH = 128 with 256 threads; generally 32*DH/(NW*64) columns
+    constexpr int CPT = 32 * DH / (NW * 64);             // columns per thread
+    static_assert(CPT % 4 == 0 && DH % CPT == 0, "bad reduction split");
+    const int row = tid / (DH / CPT), c0 = (tid % (DH / CPT)) * CPT;
+    if (q0 + row < T_) {
+        T* dst = reinterpret_cast<T*>(a.dqkv) + ((long)(q0 + row) * a.B + b) * (3 * EE) + (long)h * 3 * DH + c0;
+#pragma unroll
+        for (int c = 0; c < CPT; c += 4) {
+            float4 acc4 = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const float4 v = *reinterpret_cast<const float4*>(ebuf + (w * 32 + row) * EPI_LD + c0 + c);
+                acc4.x += v.x; acc4.y += v.y; acc4.z += v.z; acc4.w += v.w;
+            }
+            store4<T>(dst + c, acc4.x * a.qscale, acc4.y * a.qscale, acc4.z * a.qscale, acc4.w * a.qscale);
+        }
+    }
+}
+
+// Forward, second generation.  A workgroup owns 32 queries of one (batch, head); its NW waves split the
+// key range, each streaming its own K / V tiles of 32 keys through a private two-stage LDS ring and
+// keeping its own online-softmax state; the NW partial (m, l, O) are merged through LDS at the end.
+template <typename T, int DH, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
+    typedef Elem<T> E;
+    static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
+    constexpr int NDB = DH / 32, NKS = DH / 16;
+    constexpr int TILE = 32 * DH;
+    constexpr int CPR = DH / 8;
+    constexpr int NLD = 32 * CPR / 64;
+    constexpr int NLOAD = 2 * NLD;
+    static_assert(NLOAD <= 63, "too many loads in flight for vmcnt");
+    constexpr int WAVE_RING = 2 * 2 * TILE * 2;
+    constexpr int EPI_LD = DH + 4;
+    constexpr int STAT_FLOATS = 2 * NW * 32;
+    constexpr int EPI_BYTES = (STAT_FLOATS + NW * 32 * EPI_LD) * 4;
+    constexpr int SMEM = NW * WAVE_RING > EPI_BYTES ? NW * WAVE_RING : EPI_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM];
+
+    const int tid = threadIdx.x, lane = tid & 63, g = lane >> 5, li = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int bh, qblk;
+    if (!xcd_map(a.B * a.H, bh, qblk)) return;
+    const int b = bh / a.H, h = bh - b * a.H;
+    const int T_ = a.T, P = a.P, S = a.P + a.T;
+    const long EE = (long)a.H * DH;
+    const int q0 = ((T_ + 31) / 32 - 1 - qblk) * 32;     // the blocks with the longest key range start first
+    const int tq = q0 + li;
+    const bool qok = tq < T_;
+    const int kv_end = P + min(T_, q0 + 32);
+    const int ntiles = (kv_end + 31) / 32;
+    const int tpw = (ntiles + NW - 1) / NW;
+    const int t_beg = wave * tpw, t_end = min(ntiles, t_beg + tpw);
+    const int nt = max(t_end - t_beg, 0);
+
+    T* ring = reinterpret_cast<T*>(smem) + wave * (WAVE_RING / 2);
+    const unsigned ring_lds = lds_addr(smem) + wave * WAVE_RING;
+
+    typename E::opnd_t qreg[NKS];
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * T_ + tq) * DH, qok, g);
+
+    const T* pkm[NKS];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) pkm[ks] = ring + km_offset<T, DH>(li, ks * 16, lane);
+    const T* ptr0[NDB];
+    const T* ptr1[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+        int o0, o1;
+        tr_offsets<T, DH, true>(0, db * 32, lane, o0, o1);
+        ptr0[db] = ring + TILE + o0;          // inside the V tile
+        ptr1[db] = ring + TILE + o1;
+    }
+    unsigned koff[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int p = i * 64 + lane;
+        const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+        koff[i] = (unsigned)(r * DH * 2 + lc * 16);
+    }
+    const char* Kb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.kc) + (long)bh * a.cache_rows * DH));
+    const char* Vb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.vc) + (long)bh * a.cache_rows * DH));
+
+    auto issue = [&](int stage, int tile) {
+        // rows at or past S are clamped to row S-1: finite data, and every such key is masked
+        const unsigned dst = ring_lds + (unsigned)(stage * 2 * TILE * 2);
+        const int row0 = tile * 32;
+        if (row0 + 32 <= S) {
+            const char* sk = Kb + (long)row0 * (DH * 2);
+            const char* sv = Vb + (long)row0 * (DH * 2);
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) dma16_saddr_lds(koff[i], sk, dst + i * 1024);
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) dma16_saddr_lds(koff[i], sv, dst + TILE * 2 + i * 1024);
+        } else {
+            const int last = S - 1;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int p = i * 64 + lane;
+                const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+                const unsigned off = (unsigned)(min(row0 + r, last) * DH * 2 + lc * 16);
+                dma16_saddr_lds(off, Kb, dst + i * 1024);
+            }
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int p = i * 64 + lane;
+                const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+                const unsigned off = (unsigned)(min(row0 + r, last) * DH * 2 + lc * 16);
+                dma16_saddr_lds(off, Vb, dst + TILE * 2 + i * 1024);
+            }
+        }
+    };
+
+    float16v oacc[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+    float m = -INFINITY, lsum = 0.f;
+
+    wait_vmcnt<0>();
+    if (nt > 0) issue(0, t_beg);
+
+    auto step = [&](auto stage_c, int it) {
+        constexpr int s = decltype(stage_c)::value;
+        if (it + 1 < nt) {
+            issue(s ^ 1, t_beg + it + 1);
+            wait_vmcnt<NLOAD>();
+        } else {
+            wait_vmcnt<0>();
+        }
+        constexpr int so = s * 2 * TILE;
+        const int key0 = (t_beg + it) * 32;
+        typename E::opnd_t kop[NKS];
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) kop[ks] = load_km<T>(pkm[ks] + so);
+        // the V^T operands do not depend on the scores: fetch them now, use them after the softmax
+        uint4 av[2][NDB];
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+                av[hs][db] = load_tr<T>(ptr0[db] + so + hs * 16 * DH, ptr1[db] + so + hs * 16 * DH);
+        __builtin_amdgcn_sched_barrier(0);
+        float16v sacc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) sacc = E::mfma(kop[ks], qreg[ks], sacc);
+        float sv[16];
+        float mt = -INFINITY;
+        if (key0 + 31 > P + q0) {            // wave-uniform: the tile touches the causal boundary
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int key = key0 + acc_row(j, g);
+                sv[j] = key > P + tq ? -INFINITY : sacc[j];
+                mt = fmaxf(mt, sv[j]);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) { sv[j] = sacc[j]; mt = fmaxf(mt, sv[j]); }
+        }
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float m_new = fmaxf(m, mt);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = fast_exp2((m - m_safe) * kLog2e);
+        const float mneg = -m_safe * kLog2e;
+        float psum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            sv[j] = fast_exp2(fmaf(sv[j], kLog2e, mneg));   // exp(s - m); -inf -> 0
+            psum += sv[j];
+        }
+        lsum = lsum * alpha + psum;
+        m = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {   // wave-uniform: some row's running maximum moved
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+        }
+        uint4 pop[2];
+        pop[0] = pack8<T>(sv);
+        pop[1] = pack8<T>(sv + 8);
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) oacc[db] = E::mfma(av[hs][db], pop[hs], oacc[db]);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    {
+        int it = 0;
+        for (; it + 1 < nt; it += 2) {
+            step(std::integral_constant<int, 0>(), it);
+            step(std::integral_constant<int, 1>(), it + 1);
+        }
+        if (it < nt) step(std::integral_constant<int, 0>(), it);
+    }
+    wait_vmcnt<0>();
+    __syncthreads();       // every wave is done with its ring: the space is reused for the merge
+
+    float* sM = reinterpret_cast<float*>(smem);
+    float* sL = sM + NW * 32;
+    float* ebuf = sL + NW * 32;
+    const float lw = lsum + __shfl_xor(lsum, 32, 64);
+    if (g == 0) { sM[wave * 32 + li] = m; sL[wave * 32 + li] = lw; }
+    __syncthreads();
+    float m_tot = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) m_tot = fmaxf(m_tot, sM[w * 32 + li]);
+    const float m_ts = m_tot == -INFINITY ? 0.f : m_tot;
+    float L = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) L += sL[w * 32 + li] * fast_exp2((sM[w * 32 + li] - m_ts) * kLog2e);
+    const float f = L > 0.f ? fast_exp2((m - m_ts) * kLog2e) / L : 0.f;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] *= f;
+    acc_to_lds_rows<DH>(oacc, ebuf + wave * 32 * EPI_LD, lane);
+    if (wave == 0 && g == 0 && qok) a.lse[(long)bh * T_ + tq] = L > 0.f ? m_tot + logf(L) : -INFINITY;
+    __syncthreads();
+    constexpr int CPT = 32 * DH / (NW * 64);
+    static_assert(CPT % 4 == 0 && DH % CPT == 0, "bad reduction split");
+    const int row = tid / (DH / CPT), c0 = (tid % (DH / CPT)) * CPT;
+    if (q0 + row < T_) {
+        T* dst = reinterpret_cast<T*>(a.o) + ((long)(q0 + row) * a.B + b) * EE + (long)h * DH + c0;
+#pragma unroll
+        for (int c = 0; c < CPT; c += 4) {
+            float4 acc4 = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const float4 v = *reinterpret_cast<const float4*>(ebuf + (w * 32 + row) * EPI_LD + c0 + c);
+                acc4.x += v.x; acc4.y += v.y; acc4.z += v.z; acc4.w += v.w;
+            }
+            store4<T>(dst + c, acc4.x, acc4.y, acc4.z, acc4.w);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
@@ -918,6 +1649,11 @@ struct FwdPlan { int nw, bn, nsplit, qblocks; };
 
 static FwdPlan plan_fwd(const tp_attn_desc* d) {
     FwdPlan p;
+    if (d->dtype != TP_F32 && !(d->reserved2 & 1)) {
+        // 16-bit: one workgroup per 32 queries whose four waves split the key range and merge in LDS
+        p.nw = 0; p.bn = 32; p.nsplit = 1; p.qblocks = (d->T + 31) / 32;
+        return p;
+    }
     p.nw = d->T > 64 ? 4 : (d->T > 32 ? 2 : 1);
     // few (batch, head) pairs: 64-row workgroups give twice as many of them
     if (p.nw == 4 && (long)((d->T + 127) / 128) * d->batch * d->heads < kNumCU / 2) p.nw = 2;
@@ -953,6 +1689,10 @@ template <typename T, int DH>
 static void launch_fwd(const FwdPlan& p, const AttnArgs& a, hipStream_t s) {
     dim3 grid(p.qblocks, a.B * a.H, p.nsplit);
     if constexpr (sizeof(T) == 2) {
+        if (p.nw == 0) {
+            attn_fwd2_kernel<T, DH, 4><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 256, 0, s>>>(a);
+            return;
+        }
         if (p.nw == 4) attn_fwd_dma_kernel<T, DH, 4, 64, 3><<<grid, 256, 0, s>>>(a);
         else if (p.nw == 2) attn_fwd_dma_kernel<T, DH, 2, 64, 3><<<grid, 128, 0, s>>>(a);
         else attn_fwd_dma_kernel<T, DH, 1, 32, 3><<<grid, 64, 0, s>>>(a);
@@ -971,7 +1711,12 @@ template <typename T, typename GT, int DH>
 static void launch_bwd(const AttnArgs& a, hipStream_t s) {
     const int S = a.P + a.T;
     long rows = (long)a.T * a.B * a.H;
-    attn_bwd_delta_kernel<T, DH><<<(unsigned)((rows + 3) / 4), 256, 0, s>>>(a);
+    if constexpr (sizeof(T) == 2) {
+        // dQ first: it also leaves delta for the dK/dV kernel
+        attn_bwd_dq2_kernel<T, DH, 4><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 256, 0, s>>>(a);
+    } else {
+        attn_bwd_delta_kernel<T, DH><<<(unsigned)((rows + 3) / 4), 256, 0, s>>>(a);
+    }
     {
         // dK/dV: 4 waves x 32 keys per workgroup when that still fills the chip, else 2 or 1
         long bh = (long)a.B * a.H;
@@ -982,9 +1727,10 @@ static void launch_bwd(const AttnArgs& a, hipStream_t s) {
         if (sizeof(T) == 2 && a.T <= kMaxTLds) {
             if constexpr (sizeof(T) == 2) {
                 const size_t dyn = (size_t)2 * ((a.T + 31) / 32) * 32 * sizeof(float);
-                if (nw == 4) attn_bwd_dkdv_dma_kernel<T, GT, DH, 4, 3><<<grid, 256, dyn, s>>>(a);
-                else if (nw == 2) attn_bwd_dkdv_dma_kernel<T, GT, DH, 2, 3><<<grid, 128, dyn, s>>>(a);
-                else attn_bwd_dkdv_dma_kernel<T, GT, DH, 1, 3><<<grid, 64, dyn, s>>>(a);
+                const unsigned g2 = xcd_grid((int)bh, (int)grid.x);
+                if (nw == 4) attn_bwd_dkdv2_kernel<T, GT, DH, 4, 3><<<g2, 256, dyn, s>>>(a);
+                else if (nw == 2) attn_bwd_dkdv2_kernel<T, GT, DH, 2, 3><<<g2, 128, dyn, s>>>(a);
+                else attn_bwd_dkdv2_kernel<T, GT, DH, 1, 3><<<g2, 64, dyn, s>>>(a);
             }
         } else {
             if (nw == 4) attn_bwd_dkdv_kernel<T, GT, DH, 4><<<grid, 256, 0, s>>>(a);
@@ -992,15 +1738,11 @@ static void launch_bwd(const AttnArgs& a, hipStream_t s) {
             else attn_bwd_dkdv_kernel<T, GT, DH, 1><<<grid, 64, 0, s>>>(a);
         }
     }
-    {
+    if constexpr (sizeof(T) == 4) {
         int nw = a.T > 64 ? 4 : (a.T > 32 ? 2 : 1);
         if (nw == 4 && (long)((a.T + 127) / 128) * a.B * a.H < kNumCU / 2) nw = 2;
         dim3 grid((a.T + 32 * nw - 1) / (32 * nw), a.B * a.H);
-        if constexpr (sizeof(T) == 2) {
-            if (nw == 4) attn_bwd_dq_dma_kernel<T, DH, 4, 64, 3><<<grid, 256, 0, s>>>(a);
-            else if (nw == 2) attn_bwd_dq_dma_kernel<T, DH, 2, 64, 3><<<grid, 128, 0, s>>>(a);
-            else attn_bwd_dq_dma_kernel<T, DH, 1, 32, 3><<<grid, 64, 0, s>>>(a);
-        } else {
+        {
             if (nw == 4) attn_bwd_dq_kernel<T, DH, 4, 64><<<grid, 256, 0, s>>>(a);
             else if (nw == 2) attn_bwd_dq_kernel<T, DH, 2, 64><<<grid, 128, 0, s>>>(a);
             else attn_bwd_dq_kernel<T, DH, 1, 32><<<grid, 64, 0, s>>>(a);

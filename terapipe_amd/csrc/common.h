@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 #include "../../include/terapipe_hip.h"
 
@@ -346,6 +347,23 @@ __device__ __forceinline__ void dma16_saddr(unsigned off, const void* sbase, con
     unsigned lds = (unsigned)(unsigned long)(__attribute__((address_space(3))) const void*)lds_wave_base;
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
                  :: "v"(off), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory");
+}
+
+// The same load with the LDS destination (byte address of the wave's first chunk, wave-uniform) given as
+// an integer, which spares the null check of a generic-to-LDS pointer cast per load.
+__device__ __forceinline__ unsigned lds_addr(const void* p) {
+    return (unsigned)(unsigned long)(__attribute__((address_space(3))) const void*)p;
+}
+// Tells the compiler that a pointer is the same in every lane (moves it to scalar registers).
+template <typename P> __device__ __forceinline__ P* uniform_ptr(P* p) {
+    unsigned long v = (unsigned long)p;
+    unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v);
+    unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    return (P*)(((unsigned long)hi << 32) | lo);
+}
+__device__ __forceinline__ void dma16_saddr_lds(unsigned off, const void* sbase, unsigned lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(off), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)) : "memory");
 }
 
 template <typename T, int ROWS, int COLS, int NT> struct RowSlideDma {
