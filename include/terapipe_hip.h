@@ -112,6 +112,8 @@ typedef struct tp_gemm_desc {
     int64_t cache_rows;                 /* L_max: rows per (b,h) in the caches */
     float q_scale;
     int32_t reserved;                   /* 0 = automatic; bits 0-7: tile configuration + 1, bits 8-15: k splits (tuning, tests) */
+    int64_t q_bh_rows;                  /* rows per (b,h) block of q: 0 = T (compact [B*H,T,Dh]); a runner that
+                                           keeps the queries of every slice passes L_max and q offset to row P */
 } tp_gemm_desc;
 
 size_t tp_gemm_workspace_bytes(const tp_gemm_desc* d);
@@ -148,13 +150,41 @@ typedef struct tp_attn_desc {
     float q_scale;
     float* colsum_dqkv_acc;             /* optional [3*H*Dh] fp32: += column sums of dqkv (in_proj bias grad) */
     int32_t reserved;                   /* 0 = automatic; bits 0-7: number of key-range splits of the forward (tuning, tests) */
-    int32_t reserved2;
+    int32_t reserved2;                  /* bit 0: use the tile-sharing forward kernel with a split/merge pass (tuning, tests) */
+    int64_t q_bh_rows;                  /* rows per (b,h) block of q: 0 = T; see tp_gemm_desc.q_bh_rows */
+    int64_t stat_bh_rows;               /* entries per (b,h) block of lse and delta: 0 = T */
+    int32_t dq_only;                    /* backward: 1 = compute delta and the q part of dqkv only; dK/dV of the
+                                           slice are left to tp_attn_suffix_dkdv and no gradient cache is touched */
+    int32_t reserved3;
 } tp_attn_desc;
 
 size_t tp_attn_fwd_workspace_bytes(const tp_attn_desc* d);
 int tp_attn_prefix_fwd(const tp_attn_desc* d, void* workspace, size_t workspace_bytes, void* stream);
 size_t tp_attn_bwd_workspace_bytes(const tp_attn_desc* d);
 int tp_attn_prefix_bwd(const tp_attn_desc* d, void* workspace, size_t workspace_bytes, void* stream);
+
+/* dK / dV of one slice's keys against EVERY query that can see them, in one pass: the sum that
+ * _AssignCache.backward (transformer_models.py:186-190) builds up slice by slice in the gradient caches
+ * when the later slices run their backward first (terapipe.py:182-191).  A stage that keeps q, dO, lse
+ * and delta of all its slices (position-indexed, as the K/V caches are) calls this when slice [P, P+T)
+ * runs its backward -- every later slice has then left its dO and delta -- and needs no gradient cache.
+ * Query position t in [key_begin, q_end) sees key position s <= t.  Writes the k and v parts of dqkv. */
+typedef struct tp_attn_suffix_desc {
+    int32_t dtype;                      /* TP_F16 or TP_BF16 */
+    int32_t batch, heads, head_dim;
+    int32_t key_begin, key_count;       /* P, T of the slice whose keys these are */
+    int32_t q_end;                      /* queries [key_begin, q_end) take part */
+    int32_t reserved;
+    int64_t cache_rows;                 /* rows per (b,h) of k_cache, v_cache */
+    int64_t q_bh_rows;                  /* rows per (b,h) of q_all */
+    int64_t stat_bh_rows;               /* entries per (b,h) of lse_all, delta_all */
+    const void* k_cache; const void* v_cache;
+    const void* q_all;                  /* [B*H, q_bh_rows, Dh], row = position, scaled as in tp_attn_desc.q */
+    const void* d_o_all;                /* [q_end.., B, H*Dh], row = position */
+    const float* lse_all; const float* delta_all;   /* [B*H, stat_bh_rows], entry = position */
+    void* dqkv;                         /* [T*B, 3*H*Dh] of the slice; the k and v parts are written */
+} tp_attn_suffix_desc;
+int tp_attn_suffix_dkdv(const tp_attn_suffix_desc* d, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Small helpers around the kernels above.

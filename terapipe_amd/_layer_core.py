@@ -41,18 +41,22 @@ def small_acc_numel(E, F):
 class SliceState:
     """What one layer keeps from the forward of one slice for its backward."""
     __slots__ = ("x", "mean1", "rstd1", "xn", "q", "o", "lse", "h", "mean2", "rstd2", "hn", "a", "z",
-                 "k_cache", "v_cache", "cache_len", "T", "B")
+                 "k_cache", "v_cache", "cache_len", "T", "B", "q_bh_rows", "stat_bh_rows")
 
 
 class Bufs:
     """Optional preallocated outputs for one layer-slice call (views into the runner's per-layer
-    buffers).  Any attribute left at None is allocated by the call."""
+    buffers).  Any attribute left at None is allocated by the call.  q_bh_rows / stat_bh_rows: q and
+    lse / delta are views, starting at the slice's position, into position-indexed buffers with that many
+    rows per (batch, head) -- 0 means compact [B*H, T, ...] tensors."""
     __slots__ = ("xn", "mean1", "rstd1", "q", "o", "lse", "h", "mean2", "rstd2", "hn", "a", "z", "out",
-                 "dz1", "dhn", "dh", "d_o", "dqkv", "dxn", "dx", "delta")
+                 "dz1", "dhn", "dh", "d_o", "dqkv", "dxn", "dx", "delta", "q_bh_rows", "stat_bh_rows")
 
     def __init__(self, **kw):
         for n in self.__slots__:
             setattr(self, n, kw.get(n))
+        self.q_bh_rows = self.q_bh_rows or 0
+        self.stat_bh_rows = self.stat_bh_rows or 0
 
 
 _NOBUF = Bufs()
@@ -73,8 +77,9 @@ def attention_fwd(w, xn2d, T, B, heads, k_cache, v_cache, cache_len, buf=_NOBUF)
     ops.gemm(TP_GEMM_NT, xn2d, w["attn.in_proj.weight"], M, 3 * E, E, epilogue=TP_EPI_QKV_SCATTER,
              bias=w["attn.in_proj.bias"],
              qkv=dict(q=q, k_cache=k_cache, v_cache=v_cache, batch=B, heads=heads, head_dim=Dh,
-                      cache_len=cache_len, cache_rows=k_cache.shape[1], q_scale=scale))
-    o, lse = ops.attn_prefix_fwd(q, k_cache, v_cache, B, heads, Dh, T, cache_len, scale, out=buf.o, lse=buf.lse)
+                      cache_len=cache_len, cache_rows=k_cache.shape[1], q_scale=scale, q_bh_rows=buf.q_bh_rows))
+    o, lse = ops.attn_prefix_fwd(q, k_cache, v_cache, B, heads, Dh, T, cache_len, scale, out=buf.o, lse=buf.lse,
+                                 q_bh_rows=buf.q_bh_rows, stat_bh_rows=buf.stat_bh_rows)
     return q, o, lse
 
 
@@ -115,6 +120,7 @@ def layer_fwd(w, x, heads, k_cache, v_cache, cache_len, activation="relu", need_
         st.h, st.mean2, st.rstd2, st.hn = h, mean2, rstd2, hn
         st.a, st.z = a, z
         st.k_cache, st.v_cache, st.cache_len, st.T, st.B = k_cache, v_cache, cache_len, T, B
+        st.q_bh_rows, st.stat_bh_rows = buf.q_bh_rows, buf.stat_bh_rows
     return out.view(T, B, E), st
 
 
@@ -124,7 +130,7 @@ def _wgrad(target, accumulate, A, Bm, M_, N_, K_):
 
 
 def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, accumulate_prefix, has_incoming,
-              zero_slice_rows, activation="relu", buf=_NOBUF):
+              zero_slice_rows, activation="relu", buf=_NOBUF, suffix=None):
     """Backward of layer_fwd for one slice.
 
     dout [T, B, E]; gk / gv gradient caches (see tp_attn_desc).  wgrad maps the four weight names to
@@ -132,6 +138,9 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
     parameter names to fp32 accumulators that are added to.  With wgrad None / small_acc None the weight
     / vector-parameter gradients of this slice are NOT computed: the caller keeps the intermediate
     gradients this call leaves in `buf` (dz1, dhn, dh, dqkv, dxn) and reduces over all slices at once.
+    suffix: None, or dict(q_all, d_o_all, lse_all, delta_all, q_end) of position-indexed buffers that hold
+    every slice processed so far (buf.d_o and buf.delta are then views of them at this slice): dK/dV of
+    the slice's keys are computed in one pass over all later query positions and gk / gv are not used.
     Returns dx [T, B, E].
     """
     T, B = st.T, st.B
@@ -164,9 +173,19 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
     if wgrad is not None:
         _wgrad(wgrad["attn.out_proj.weight"], accumulate_wgrad, dh, st.o, E, E, M)
     dqkv = _buf(buf.dqkv, (M, 3 * E), dt, dev)
-    ops.attn_prefix_bwd(st.q, st.k_cache, st.v_cache, st.o, st.lse, d_o, dqkv, gk, gv, B, heads, Dh, T,
-                        st.cache_len, float(Dh) ** -0.5, accumulate_prefix, has_incoming, zero_slice_rows,
-                        colsum_dqkv_acc=sa.get("attn.in_proj.bias"), delta=buf.delta)
+    if suffix is None:
+        ops.attn_prefix_bwd(st.q, st.k_cache, st.v_cache, st.o, st.lse, d_o, dqkv, gk, gv, B, heads, Dh, T,
+                            st.cache_len, float(Dh) ** -0.5, accumulate_prefix, has_incoming, zero_slice_rows,
+                            colsum_dqkv_acc=sa.get("attn.in_proj.bias"), delta=buf.delta,
+                            q_bh_rows=st.q_bh_rows, stat_bh_rows=st.stat_bh_rows)
+    else:
+        ops.attn_prefix_bwd(st.q, st.k_cache, st.v_cache, st.o, st.lse, d_o, dqkv, None, None, B, heads, Dh, T,
+                            st.cache_len, float(Dh) ** -0.5, False, False, False, delta=buf.delta,
+                            q_bh_rows=st.q_bh_rows, stat_bh_rows=st.stat_bh_rows, dq_only=True)
+        ops.attn_suffix_dkdv(st.k_cache, st.v_cache, suffix["q_all"], suffix["d_o_all"], suffix["lse_all"],
+                             suffix["delta_all"], dqkv, B, heads, Dh, st.cache_len, T, suffix["q_end"])
+        if "attn.in_proj.bias" in sa:
+            ops.colsum_acc(dqkv, sa["attn.in_proj.bias"])
     dxn = _buf(buf.dxn, (M, E), dt, dev)
     ops.gemm(TP_GEMM_NN, dqkv, w["attn.in_proj.weight"], M, E, 3 * E, C=dxn)
     if wgrad is not None:

@@ -35,6 +35,7 @@ class GemmDesc(ctypes.Structure):
         ("batch", c_int32), ("heads", c_int32), ("head_dim", c_int32), ("cache_len", c_int32),
         ("cache_rows", c_int64),
         ("q_scale", c_float), ("reserved", c_int32),
+        ("q_bh_rows", c_int64),
     ]
 
 
@@ -53,6 +54,21 @@ class AttnDesc(ctypes.Structure):
         ("q_scale", c_float),
         ("colsum_dqkv_acc", c_void_p),
         ("reserved", c_int32), ("reserved2", c_int32),
+        ("q_bh_rows", c_int64), ("stat_bh_rows", c_int64),
+        ("dq_only", c_int32), ("reserved3", c_int32),
+    ]
+
+
+class AttnSuffixDesc(ctypes.Structure):
+    """Mirror of ``tp_attn_suffix_desc``."""
+    _fields_ = [
+        ("dtype", c_int32), ("batch", c_int32), ("heads", c_int32), ("head_dim", c_int32),
+        ("key_begin", c_int32), ("key_count", c_int32), ("q_end", c_int32), ("reserved", c_int32),
+        ("cache_rows", c_int64), ("q_bh_rows", c_int64), ("stat_bh_rows", c_int64),
+        ("k_cache", c_void_p), ("v_cache", c_void_p),
+        ("q_all", c_void_p), ("d_o_all", c_void_p),
+        ("lse_all", c_void_p), ("delta_all", c_void_p),
+        ("dqkv", c_void_p),
     ]
 
 
@@ -69,6 +85,7 @@ SYMBOLS = {
     "tp_attn_prefix_fwd": (c_int, [ctypes.POINTER(AttnDesc), c_void_p, c_size_t, c_void_p]),
     "tp_attn_bwd_workspace_bytes": (c_size_t, [ctypes.POINTER(AttnDesc)]),
     "tp_attn_prefix_bwd": (c_int, [ctypes.POINTER(AttnDesc), c_void_p, c_size_t, c_void_p]),
+    "tp_attn_suffix_dkdv": (c_int, [ctypes.POINTER(AttnSuffixDesc), c_void_p]),
     "tp_accum_cast": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "tp_colsum_acc": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_void_p]),
     "tp_zero_words": (c_int, [c_void_p, c_int64, c_void_p]),

@@ -20,7 +20,10 @@ struct AttnArgs {
     int nsplit;
     float* part_o; float* part_lse;
     int accumulate_prefix, has_incoming, zero_slice_rows;
+    int dq_only;
     float qscale;
+    long q_bhs;      // elements between consecutive (batch, head) blocks of q
+    long st_bhs;     // floats between consecutive (batch, head) blocks of lse / delta
 };
 
 static constexpr float kLog2e = 1.4426950408889634f;
@@ -100,7 +103,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs a) {
     const int t_beg = blockIdx.z * tps, t_end = min(ntiles, t_beg + tps);
 
     typename E::opnd_t qreg[NKS];
-    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * T_ + tq) * DH, tq < T_, g);
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), tq < T_, g);
 
     float16v oacc[NDB];
 #pragma unroll
@@ -191,7 +194,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs a) {
                     store4<T>(O + dh, oacc[db][4 * jq] * inv, oacc[db][4 * jq + 1] * inv,
                               oacc[db][4 * jq + 2] * inv, oacc[db][4 * jq + 3] * inv);
                 }
-            if (g == 0) a.lse[(long)bh * T_ + tq] = lse;
+            if (g == 0) a.lse[(long)bh * a.st_bhs + tq] = lse;
         } else {
             const long BH = (long)a.B * a.H;
             float* PO = a.part_o + (((long)blockIdx.z * BH + bh) * T_ + tq) * DH;
@@ -236,7 +239,7 @@ __global__ __launch_bounds__(256) void attn_fwd_merge_kernel(AttnArgs a) {
     const float inv = 1.0f / wsum;
 #pragma unroll
     for (int i = 0; i < DH / 64; ++i) O[lane + 64 * i] = Elem<T>::from_float(acc[i] * inv);
-    if (lane == 0) a.lse[row] = mx + logf(wsum);
+    if (lane == 0) a.lse[(long)bh * a.st_bhs + t] = mx + logf(wsum);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -260,7 +263,7 @@ __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(AttnArgs a) {
     for (int i = 0; i < DH / 64; ++i)
         s += Elem<T>::to_float(O[lane + 64 * i]) * Elem<T>::to_float(dO[lane + 64 * i]);
     s = wave_sum(s);
-    if (lane == 0) a.delta[((long)b * a.H + h) * a.T + t] = s;
+    if (lane == 0) a.delta[((long)b * a.H + h) * a.st_bhs + t] = s;
 }
 
 // dK / dV: each wave owns 32 keys and walks over the query blocks that can see them.
@@ -292,7 +295,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_kernel(AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
 
-    const T* Qb = reinterpret_cast<const T*>(a.q) + (long)bh * T_ * DH;
+    const T* Qb = reinterpret_cast<const T*>(a.q) + (long)bh * a.q_bhs;
     const T* dOb = reinterpret_cast<const T*>(a.d_o) + (long)b * EE + (long)h * DH;  // row t at stride B*E
     const int nqb = (T_ + 31) / 32;
     const int qb_start = key0wg > P ? (key0wg - P) / 32 : 0;
@@ -305,8 +308,8 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_kernel(AttnArgs a) {
         cdo.store(sdO, tid);
         if (tid < 32) {
             int t = qb * 32 + tid;
-            sLse[tid] = t < T_ ? a.lse[(long)bh * T_ + t] : 0.f;
-            sDelta[tid] = t < T_ ? a.delta[(long)bh * T_ + t] : 0.f;
+            sLse[tid] = t < T_ ? a.lse[(long)bh * a.st_bhs + t] : 0.f;
+            sDelta[tid] = t < T_ ? a.delta[(long)bh * a.st_bhs + t] : 0.f;
         }
         __syncthreads();
         if (key0w < S && key0w <= P + qb * 32 + 31) {
@@ -401,10 +404,10 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_kernel(AttnArgs a) {
     const int ntiles = (kv_end + BN - 1) / BN;
 
     typename E::opnd_t qreg[NKS], doreg[NKS];
-    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * T_ + tq) * DH, tq < T_, g);
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), tq < T_, g);
     load_row_operands<T, DH>(doreg, reinterpret_cast<const T*>(a.d_o) + ((long)tq * a.B + b) * EE + (long)h * DH, tq < T_, g);
-    const float lse_q = tq < T_ ? a.lse[(long)bh * T_ + tq] : 0.f;
-    const float delta_q = tq < T_ ? a.delta[(long)bh * T_ + tq] : 0.f;
+    const float lse_q = tq < T_ ? a.lse[(long)bh * a.st_bhs + tq] : 0.f;
+    const float delta_q = tq < T_ ? a.delta[(long)bh * a.st_bhs + tq] : 0.f;
 
     float16v dq[NDB];
 #pragma unroll
@@ -564,7 +567,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_dma_kernel(AttnArgs a) {
     const int nt = max(t_end - t_beg, 0);
 
     typename E::opnd_t qreg[NKS];
-    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * T_ + tq) * DH, tq < T_, g);
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), tq < T_, g);
     wait_vmcnt<0>();   // plain loads done before the counted tile loads start
 
     float16v oacc[NDB];
@@ -616,7 +619,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_dma_kernel(AttnArgs a) {
                     store4<T>(O + dh, oacc[db][4 * jq] * inv, oacc[db][4 * jq + 1] * inv,
                               oacc[db][4 * jq + 2] * inv, oacc[db][4 * jq + 3] * inv);
                 }
-            if (g == 0) a.lse[(long)bh * T_ + tq] = lse;
+            if (g == 0) a.lse[(long)bh * a.st_bhs + tq] = lse;
         } else {
             const long BH = (long)a.B * a.H;
             float* PO = a.part_o + (((long)blockIdx.z * BH + bh) * T_ + tq) * DH;
@@ -657,10 +660,10 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_dma_kernel(AttnArgs a) {
     const int nt = (kv_end + BN - 1) / BN;
 
     typename E::opnd_t qreg[NKS], doreg[NKS];
-    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * T_ + tq) * DH, tq < T_, g);
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), tq < T_, g);
     load_row_operands<T, DH>(doreg, reinterpret_cast<const T*>(a.d_o) + ((long)tq * a.B + b) * EE + (long)h * DH, tq < T_, g);
-    const float lse_q = tq < T_ ? a.lse[(long)bh * T_ + tq] : 0.f;
-    const float delta_q = tq < T_ ? a.delta[(long)bh * T_ + tq] : 0.f;
+    const float lse_q = tq < T_ ? a.lse[(long)bh * a.st_bhs + tq] : 0.f;
+    const float delta_q = tq < T_ ? a.delta[(long)bh * a.st_bhs + tq] : 0.f;
     const float lse_neg = -lse_q * kLog2e;
     wait_vmcnt<0>();
 
@@ -772,8 +775,8 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_dma_kernel(AttnArgs a) 
     load_row_operands<T, DH>(kreg, reinterpret_cast<const T*>(a.kc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
     load_row_operands<T, DH>(vreg, reinterpret_cast<const T*>(a.vc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
     for (int t = tid; t < Tpad; t += NT) {
-        sLse[t] = t < T_ ? -a.lse[(long)bh * T_ + t] * kLog2e : 0.f;     // stored as -lse * log2(e)
-        sDelta[t] = t < T_ ? a.delta[(long)bh * T_ + t] : 0.f;
+        sLse[t] = t < T_ ? -a.lse[(long)bh * a.st_bhs + t] * kLog2e : 0.f;     // stored as -lse * log2(e)
+        sDelta[t] = t < T_ ? a.delta[(long)bh * a.st_bhs + t] : 0.f;
     }
     wait_vmcnt<0>();
     __syncthreads();
@@ -784,7 +787,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_dma_kernel(AttnArgs a) 
 #pragma unroll
         for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
 
-    const T* Qb = reinterpret_cast<const T*>(a.q) + (long)bh * T_ * DH;
+    const T* Qb = reinterpret_cast<const T*>(a.q) + (long)bh * a.q_bhs;
     const T* dOb = reinterpret_cast<const T*>(a.d_o) + (long)b * EE + (long)h * DH;  // row t at stride B*E
     const int qb_start = key0wg > P ? (key0wg - P) / 32 : 0;
     const int nt = nqb - qb_start;
@@ -969,8 +972,8 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv2_kernel(AttnArgs a) {
     load_row_operands<T, DH>(kreg, reinterpret_cast<const T*>(a.kc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
     load_row_operands<T, DH>(vreg, reinterpret_cast<const T*>(a.vc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
     for (int t = tid; t < Tpad; t += NW * 64) {
-        sLse[t] = t < T_ ? -a.lse[(long)bh * T_ + t] * kLog2e : 0.f;
-        sDelta[t] = t < T_ ? a.delta[(long)bh * T_ + t] : 0.f;
+        sLse[t] = t < T_ ? -a.lse[(long)bh * a.st_bhs + t] * kLog2e : 0.f;
+        sDelta[t] = t < T_ ? a.delta[(long)bh * a.st_bhs + t] : 0.f;
     }
 
     // lane-constant LDS addresses inside stage 0's Q tile (the dO tile and the other stages are
@@ -997,7 +1000,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv2_kernel(AttnArgs a) {
         qoff[i] = (unsigned)(r * DH * 2 + lc * 16);
         dooff[i] = (unsigned)(r * ldo_bytes + lc * 16);
     }
-    const char* Qb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.q) + (long)bh * T_ * DH));
+    const char* Qb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.q) + (long)bh * a.q_bhs));
     const char* dOb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.d_o) + (long)b * EE + (long)h * DH));
     const int qb_start = key0wg > P ? (key0wg - P) / 32 : 0;
     const int nt = nqb - qb_start;
@@ -1230,7 +1233,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq2_kernel(AttnArgs a) {
 
     typename E::opnd_t qreg[NKS], doreg[NKS];
     const long orow = ((long)tq * a.B + b) * EE + (long)h * DH;
-    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * T_ + tq) * DH, qok, g);
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), qok, g);
     load_row_operands<T, DH>(doreg, reinterpret_cast<const T*>(a.d_o) + orow, qok, g);
     float delta_q;
     {
@@ -1246,8 +1249,8 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq2_kernel(AttnArgs a) {
         }
         delta_q = s + __shfl_xor(s, 32, 64);
     }
-    if (wave == 0 && g == 0 && qok) a.delta[(long)bh * T_ + tq] = delta_q;
-    const float lse_neg = qok ? -a.lse[(long)bh * T_ + tq] * kLog2e : 0.f;
+    if (wave == 0 && g == 0 && qok) a.delta[(long)bh * a.st_bhs + tq] = delta_q;
+    const float lse_neg = qok ? -a.lse[(long)bh * a.st_bhs + tq] * kLog2e : 0.f;
 
     // lane-constant LDS addresses inside stage 0's K tile
     const T* pkm[NKS];
@@ -1441,7 +1444,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
     const unsigned ring_lds = lds_addr(smem) + wave * WAVE_RING;
 
     typename E::opnd_t qreg[NKS];
-    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * T_ + tq) * DH, qok, g);
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), qok, g);
 
     const T* pkm[NKS];
 #pragma unroll
@@ -1602,7 +1605,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[db][r] *= f;
     acc_to_lds_rows<DH>(oacc, ebuf + wave * 32 * EPI_LD, lane);
-    if (wave == 0 && g == 0 && qok) a.lse[(long)bh * T_ + tq] = L > 0.f ? m_tot + logf(L) : -INFINITY;
+    if (wave == 0 && g == 0 && qok) a.lse[(long)bh * a.st_bhs + tq] = L > 0.f ? m_tot + logf(L) : -INFINITY;
     __syncthreads();
     constexpr int CPT = 32 * DH / (NW * 64);
     static_assert(CPT % 4 == 0 && DH % CPT == 0, "bad reduction split");
@@ -1623,6 +1626,249 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// dK / dV of one slice's keys against every query position that can see them (tp_attn_suffix_dkdv).
+// A workgroup owns 32 keys of one (batch, head); its NW waves split the query blocks [key .. q_end),
+// each streaming its own Q / dO tiles of 32 positions (plus their lse and delta) through a private
+// two-stage LDS ring, and the NW partial dK / dV blocks are summed through LDS at the end.
+// ------------------------------------------------------------------------------------------------
+struct SuffixArgs {
+    const void* kc; const void* vc; const void* q; const void* d_o;
+    const float* lse; const float* delta; void* dqkv;
+    int B, H, P, T, Lq;
+    long cache_rows, q_bhs, st_bhs;
+};
+
+__device__ __forceinline__ void dma4(const void* gptr, unsigned lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off"
+                 :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)) : "memory");
+}
+
+template <typename T, int DH, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_suffix_dkdv_kernel(SuffixArgs a) {
+    typedef Elem<T> E;
+    static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
+    constexpr int NDB = DH / 32, NKS = DH / 16;
+    constexpr int TILE = 32 * DH;                       // elements of one Q or dO tile
+    constexpr int CPR = DH / 8;
+    constexpr int NLD = 32 * CPR / 64;
+    constexpr int NLOAD = 2 * NLD + 1;                  // Q, dO and the stats row
+    static_assert(NLOAD <= 63, "too many loads in flight for vmcnt");
+    constexpr int WAVE_RING = 2 * 2 * TILE * 2;         // bytes: two stages of Q + dO
+    constexpr int STAT_BYTES = 2 * 256;                 // per wave: two stages of 32 lse + 32 delta
+    constexpr int EPI_LD = DH + 4;
+    constexpr int EPI_BYTES = NW * 32 * EPI_LD * 4;
+    constexpr int RING_ALL = NW * (WAVE_RING + STAT_BYTES);
+    constexpr int SMEM = RING_ALL > EPI_BYTES ? RING_ALL : EPI_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM];
+
+    const int tid = threadIdx.x, lane = tid & 63, g = lane >> 5, li = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int bh, kblk;
+    if (!xcd_map(a.B * a.H, bh, kblk)) return;
+    const int b = bh / a.H, h = bh - b * a.H;
+    const int P = a.P, S = a.P + a.T, Lq = a.Lq;
+    const long EE = (long)a.H * DH;
+    const int key0 = P + kblk * 32;
+    const int key = key0 + li;
+    const int nqb = (Lq - key0 + 31) / 32;              // query blocks start at the key block's position
+    const int tpw = (nqb + NW - 1) / NW;
+    const int j_beg = wave * tpw, j_end = min(nqb, j_beg + tpw);
+    const int nt = max(j_end - j_beg, 0);
+
+    T* ring = reinterpret_cast<T*>(smem) + wave * (WAVE_RING / 2);
+    const unsigned ring_lds = lds_addr(smem) + wave * WAVE_RING;
+    const float* sstat = reinterpret_cast<const float*>(smem + NW * WAVE_RING + wave * STAT_BYTES);
+    const unsigned stat_lds = lds_addr(smem) + NW * WAVE_RING + wave * STAT_BYTES;
+
+    typename E::opnd_t kreg[NKS], vreg[NKS];
+    load_row_operands<T, DH>(kreg, reinterpret_cast<const T*>(a.kc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
+    load_row_operands<T, DH>(vreg, reinterpret_cast<const T*>(a.vc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
+
+    const T* pkm[NKS];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) pkm[ks] = ring + km_offset<T, DH>(li, ks * 16, lane);
+    const T* ptr0[NDB];
+    const T* ptr1[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+        int o0, o1;
+        tr_offsets<T, DH, true>(0, db * 32, lane, o0, o1);
+        ptr0[db] = ring + o0;
+        ptr1[db] = ring + o1;
+    }
+    unsigned qoff[NLD], dooff[NLD];
+    const unsigned ldo_bytes = (unsigned)((long)a.B * EE * 2);
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int p = i * 64 + lane;
+        const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+        qoff[i] = (unsigned)(r * DH * 2 + lc * 16);
+        dooff[i] = (unsigned)(r * ldo_bytes + lc * 16);
+    }
+    const char* Qb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.q) + (long)bh * a.q_bhs));
+    const char* dOb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.d_o) + (long)b * EE + (long)h * DH));
+    const float* statb = (g == 0 ? a.lse : a.delta) + (long)bh * a.st_bhs;   // lanes 0-31 fetch lse, 32-63 delta
+
+    auto issue = [&](int stage, int j) {
+        // positions at or past q_end are clamped to q_end - 1: finite data whose P and dS are forced to zero
+        const unsigned dst = ring_lds + (unsigned)(stage * 2 * TILE * 2);
+        const int row0 = key0 + j * 32;
+        if (row0 + 32 <= Lq) {
+            const char* sq = Qb + (long)row0 * (DH * 2);
+            const char* sd = dOb + (long)row0 * ldo_bytes;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) dma16_saddr_lds(qoff[i], sq, dst + i * 1024);
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) dma16_saddr_lds(dooff[i], sd, dst + TILE * 2 + i * 1024);
+        } else {
+            const int last = Lq - 1;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int p = i * 64 + lane;
+                const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+                dma16_saddr_lds((unsigned)(min(row0 + r, last) * DH * 2 + lc * 16), Qb, dst + i * 1024);
+            }
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int p = i * 64 + lane;
+                const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+                dma16_saddr_lds((unsigned)(min(row0 + r, last) * ldo_bytes + lc * 16), dOb, dst + TILE * 2 + i * 1024);
+            }
+        }
+        dma4(statb + min(row0 + li, Lq - 1), stat_lds + stage * 256);
+    };
+
+    float16v dk[NDB], dv[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
+
+    wait_vmcnt<0>();
+    if (nt > 0) issue(0, j_beg);
+
+    auto step = [&](auto stage_c, int it) {
+        constexpr int s = decltype(stage_c)::value;
+        if (it + 1 < nt) {
+            issue(s ^ 1, j_beg + it + 1);
+            wait_vmcnt<NLOAD>();
+        } else {
+            wait_vmcnt<0>();
+        }
+        constexpr int so = s * 2 * TILE;
+        const int t0 = key0 + (j_beg + it) * 32;        // first query position of the block
+        typename E::opnd_t qop[NKS], doop[NKS];
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            qop[ks] = load_km<T>(pkm[ks] + so);
+            doop[ks] = load_km<T>(pkm[ks] + so + TILE);
+        }
+        float4 l4[4], d4[4];
+#pragma unroll
+        for (int jq = 0; jq < 4; ++jq) {
+            l4[jq] = *reinterpret_cast<const float4*>(sstat + s * 64 + 8 * jq + 4 * g);
+            d4[jq] = *reinterpret_cast<const float4*>(sstat + s * 64 + 32 + 8 * jq + 4 * g);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        float16v sacc, pacc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            sacc = E::mfma(qop[ks], kreg[ks], sacc);
+            pacc = E::mfma(doop[ks], vreg[ks], pacc);
+        }
+        // wave-uniform: every (query, key) pair of the block is visible and in range
+        const bool all_visible = (t0 + 32 <= Lq) && (key0 + 31 <= t0) && (key0 + 32 <= S);
+        float pv[16], dsv[16];
+        if (all_visible) {
+#pragma unroll
+            for (int jq = 0; jq < 4; ++jq) {
+                const float lv[4] = {l4[jq].x, l4[jq].y, l4[jq].z, l4[jq].w};
+                const float dl[4] = {d4[jq].x, d4[jq].y, d4[jq].z, d4[jq].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int j = 4 * jq + e;
+                    const float p = fast_exp2((sacc[j] - lv[e]) * kLog2e);
+                    pv[j] = p;
+                    dsv[j] = p * (pacc[j] - dl[e]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int jq = 0; jq < 4; ++jq) {
+                const float lv[4] = {l4[jq].x, l4[jq].y, l4[jq].z, l4[jq].w};
+                const float dl[4] = {d4[jq].x, d4[jq].y, d4[jq].z, d4[jq].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int j = 4 * jq + e;
+                    const int t = t0 + 8 * jq + 4 * g + e;
+                    const bool vis = (t < Lq) && (key <= t) && (key < S);
+                    const float p = vis ? fast_exp2((sacc[j] - lv[e]) * kLog2e) : 0.f;
+                    pv[j] = p;
+                    dsv[j] = vis ? p * (pacc[j] - dl[e]) : 0.f;
+                }
+            }
+        }
+        uint4 pop[2], dsop[2];
+        pop[0] = pack8<T>(pv); pop[1] = pack8<T>(pv + 8);
+        dsop[0] = pack8<T>(dsv); dsop[1] = pack8<T>(dsv + 8);
+        uint4 ado[2][NDB], aq[2][NDB];
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) {
+                ado[hs][db] = load_tr<T>(ptr0[db] + so + TILE + hs * 16 * DH, ptr1[db] + so + TILE + hs * 16 * DH);
+                aq[hs][db] = load_tr<T>(ptr0[db] + so + hs * 16 * DH, ptr1[db] + so + hs * 16 * DH);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) {
+                dv[db] = E::mfma(ado[hs][db], pop[hs], dv[db]);
+                dk[db] = E::mfma(aq[hs][db], dsop[hs], dk[db]);
+            }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    {
+        int it = 0;
+        for (; it + 1 < nt; it += 2) {
+            step(std::integral_constant<int, 0>(), it);
+            step(std::integral_constant<int, 1>(), it + 1);
+        }
+        if (it < nt) step(std::integral_constant<int, 0>(), it);
+    }
+    wait_vmcnt<0>();
+    __syncthreads();       // every wave is done with its ring: the space is reused for the reduction
+
+    float* ebuf = reinterpret_cast<float*>(smem);
+    constexpr int CPT = 32 * DH / (NW * 64);
+    static_assert(CPT % 4 == 0 && DH % CPT == 0, "bad reduction split");
+    const int row = tid / (DH / CPT), c0 = (tid % (DH / CPT)) * CPT;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        acc_to_lds_rows<DH>(which == 0 ? dk : dv, ebuf + wave * 32 * EPI_LD, lane);
+        __syncthreads();
+        if (key0 + row < S) {
+            T* dst = reinterpret_cast<T*>(a.dqkv) + ((long)(key0 + row - P) * a.B + b) * (3 * EE) + (long)h * 3 * DH +
+                     (which + 1) * DH + c0;
+#pragma unroll
+            for (int c = 0; c < CPT; c += 4) {
+                float4 acc4 = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int w = 0; w < NW; ++w) {
+                    const float4 v = *reinterpret_cast<const float4*>(ebuf + (w * 32 + row) * EPI_LD + c0 + c);
+                    acc4.x += v.x; acc4.y += v.y; acc4.z += v.z; acc4.w += v.w;
+                }
+                store4<T>(dst + c, acc4.x, acc4.y, acc4.z, acc4.w);
+            }
+        }
+        __syncthreads();   // the buffer is rewritten by the next pass
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
 static constexpr int kNumCU = 256;
@@ -1639,7 +1885,7 @@ static int validate_attn(const tp_attn_desc* d, bool bwd) {
     if (bwd) {
         if (!d->d_o || !d->delta || !d->dqkv) { set_error("%s: null gradient tensor", who); return TP_ERR_ARG; }
         if (((uintptr_t)d->d_o | (uintptr_t)d->dqkv | (uintptr_t)d->dk_cache | (uintptr_t)d->dv_cache) & 15) { set_error("%s: tensors must be 16-byte aligned", who); return TP_ERR_ARG; }
-        if ((d->cache_len > 0 || d->has_incoming || d->zero_slice_rows) && (!d->dk_cache || !d->dv_cache)) { set_error("%s: gradient caches required", who); return TP_ERR_ARG; }
+        if (!d->dq_only && (d->cache_len > 0 || d->has_incoming || d->zero_slice_rows) && (!d->dk_cache || !d->dv_cache)) { set_error("%s: gradient caches required", who); return TP_ERR_ARG; }
         if (d->grad_cache_dtype != d->dtype && d->grad_cache_dtype != TP_F32) { set_error("%s: grad_cache_dtype must be dtype or fp32", who); return TP_ERR_ARG; }
     }
     return TP_OK;
@@ -1682,6 +1928,9 @@ static AttnArgs make_args(const tp_attn_desc* d) {
     a.nsplit = 1; a.part_o = nullptr; a.part_lse = nullptr;
     a.accumulate_prefix = d->accumulate_prefix; a.has_incoming = d->has_incoming;
     a.zero_slice_rows = d->zero_slice_rows; a.qscale = d->q_scale;
+    a.dq_only = d->dq_only;
+    a.q_bhs = (d->q_bh_rows > 0 ? d->q_bh_rows : (long)d->T) * d->head_dim;
+    a.st_bhs = d->stat_bh_rows > 0 ? d->stat_bh_rows : (long)d->T;
     return a;
 }
 
@@ -1717,7 +1966,7 @@ static void launch_bwd(const AttnArgs& a, hipStream_t s) {
     } else {
         attn_bwd_delta_kernel<T, DH><<<(unsigned)((rows + 3) / 4), 256, 0, s>>>(a);
     }
-    {
+    if (!a.dq_only) {
         // dK/dV: 4 waves x 32 keys per workgroup when that still fills the chip, else 2 or 1
         long bh = (long)a.B * a.H;
         int nw = 4;
@@ -1825,9 +2074,45 @@ extern "C" int tp_attn_prefix_bwd(const tp_attn_desc* d, void* workspace, size_t
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("tp_attn_prefix_bwd: launch failed: %s", hipGetErrorString(e)); return TP_ERR_LAUNCH; }
-    if (d->colsum_dqkv_acc) {
+    if (d->colsum_dqkv_acc && !d->dq_only) {
         return tp_colsum_acc(d->dqkv, 3L * d->heads * d->head_dim, d->colsum_dqkv_acc, d->T * d->batch,
                              3 * d->heads * d->head_dim, d->dtype, stream);
     }
+    return TP_OK;
+}
+
+extern "C" int tp_attn_suffix_dkdv(const tp_attn_suffix_desc* d, void* stream) {
+    using namespace tp;
+    const char* who = "tp_attn_suffix_dkdv";
+    if (!d) { set_error("%s: null descriptor", who); return TP_ERR_ARG; }
+    if (d->dtype != TP_F16 && d->dtype != TP_BF16) { set_error("%s: dtype %d not supported (fp16 / bf16)", who, d->dtype); return TP_ERR_UNSUPPORTED; }
+    if (d->head_dim != 64 && d->head_dim != 128) { set_error("%s: head_dim %d not supported (64 or 128)", who, d->head_dim); return TP_ERR_UNSUPPORTED; }
+    if (d->batch <= 0 || d->heads <= 0 || d->key_begin < 0 || d->key_count <= 0 || d->q_end < d->key_begin + d->key_count) {
+        set_error("%s: bad geometry B=%d H=%d keys [%d, +%d) q_end=%d", who, d->batch, d->heads, d->key_begin, d->key_count, d->q_end);
+        return TP_ERR_ARG;
+    }
+    if ((long)d->key_begin + d->key_count > d->cache_rows || d->q_end > d->q_bh_rows || d->q_end > d->stat_bh_rows) {
+        set_error("%s: positions up to %d do not fit cache_rows %ld / q_bh_rows %ld / stat_bh_rows %ld", who, d->q_end,
+                  (long)d->cache_rows, (long)d->q_bh_rows, (long)d->stat_bh_rows);
+        return TP_ERR_ARG;
+    }
+    if (!d->k_cache || !d->v_cache || !d->q_all || !d->d_o_all || !d->lse_all || !d->delta_all || !d->dqkv) { set_error("%s: null tensor", who); return TP_ERR_ARG; }
+    if (((uintptr_t)d->k_cache | (uintptr_t)d->v_cache | (uintptr_t)d->q_all | (uintptr_t)d->d_o_all | (uintptr_t)d->dqkv) & 15) { set_error("%s: tensors must be 16-byte aligned", who); return TP_ERR_ARG; }
+    SuffixArgs a;
+    a.kc = d->k_cache; a.vc = d->v_cache; a.q = d->q_all; a.d_o = d->d_o_all;
+    a.lse = d->lse_all; a.delta = d->delta_all; a.dqkv = d->dqkv;
+    a.B = d->batch; a.H = d->heads; a.P = d->key_begin; a.T = d->key_count; a.Lq = d->q_end;
+    a.cache_rows = d->cache_rows; a.q_bhs = d->q_bh_rows * d->head_dim; a.st_bhs = d->stat_bh_rows;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const unsigned grid = xcd_grid(d->batch * d->heads, (d->key_count + 31) / 32);
+    if (d->dtype == TP_F16) {
+        if (d->head_dim == 64) attn_suffix_dkdv_kernel<f16, 64, 4><<<grid, 256, 0, s>>>(a);
+        else attn_suffix_dkdv_kernel<f16, 128, 4><<<grid, 256, 0, s>>>(a);
+    } else {
+        if (d->head_dim == 64) attn_suffix_dkdv_kernel<bf16, 64, 4><<<grid, 256, 0, s>>>(a);
+        else attn_suffix_dkdv_kernel<bf16, 128, 4><<<grid, 256, 0, s>>>(a);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("%s: launch failed: %s", who, hipGetErrorString(e)); return TP_ERR_LAUNCH; }
     return TP_OK;
 }

@@ -19,6 +19,7 @@ struct GemmArgs {
     void* q; void* kc; void* vc;
     int batch, heads, hd, T, P;
     long cache_rows;
+    long q_rows;     // rows per (batch, head) block of q
     float qscale;
     int kper;        // k extent handled by one split
     int nsplit;
@@ -124,7 +125,7 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& a, int row, int co
         if (part == 0) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) t[e] = v[e] * a.qscale;
-            st8(a.q, (bh * a.T + tt) * a.hd + d, t);
+            st8(a.q, (bh * a.q_rows + tt) * a.hd + d, t);
         } else {
             st8(part == 1 ? a.kc : a.vc, (bh * a.cache_rows + a.P + tt) * a.hd + d, v);
         }
@@ -698,6 +699,7 @@ extern "C" int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_
     a.q = d->q; a.kc = d->k_cache; a.vc = d->v_cache;
     a.batch = d->batch; a.heads = d->heads; a.hd = d->head_dim;
     a.T = d->epilogue == TP_EPI_QKV_SCATTER ? d->M / d->batch : 0;
+    a.q_rows = d->q_bh_rows > 0 ? d->q_bh_rows : a.T;
     a.P = d->cache_len; a.cache_rows = d->cache_rows; a.qscale = d->q_scale;
     a.kper = p.kper; a.nsplit = p.nsplit; a.partial = reinterpret_cast<float*>(workspace);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);

@@ -180,6 +180,7 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
         d.q, d.k_cache, d.v_cache = qkv["q"].data_ptr(), qkv["k_cache"].data_ptr(), qkv["v_cache"].data_ptr()
         d.batch, d.heads, d.head_dim = qkv["batch"], qkv["heads"], qkv["head_dim"]
         d.cache_len, d.cache_rows, d.q_scale = qkv["cache_len"], qkv["cache_rows"], qkv["q_scale"]
+        d.q_bh_rows = qkv.get("q_bh_rows", 0)
     if tile_cfg is not None or ksplit is not None:
         d.reserved = ((tile_cfg + 1) if tile_cfg is not None else 0) | ((ksplit or 0) << 8)
     lib = _lib.load()
@@ -193,8 +194,12 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
     return C
 
 
-def _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale):
+def _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale, q_bh_rows=0,
+               stat_bh_rows=0):
+    """q_bh_rows / stat_bh_rows: rows per (batch, head) block of q / of lse and delta when these are views
+    into position-indexed buffers that hold every slice (0 = compact [B*H, T, ...])."""
     d = AttnDesc()
+    d.q_bh_rows, d.stat_bh_rows = q_bh_rows, stat_bh_rows
     d.dtype = tp_dtype(q.dtype)
     d.batch, d.heads, d.head_dim, d.T, d.cache_len = batch, heads, head_dim, T, cache_len
     d.cache_rows = k_cache.shape[1]
@@ -204,14 +209,14 @@ def _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len
 
 
 def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q_scale, out=None, lse=None,
-                    nsplit=None):
+                    nsplit=None, q_bh_rows=0, stat_bh_rows=0):
     """q [B*H, T, Dh] (pre-scaled); caches [B*H, L, Dh] with rows [0, cache_len+T) valid.
     Returns o [T, B, H*Dh] and lse [B*H, T]."""
     _require_cuda(q, k_cache, v_cache)
     o = torch.empty(T, batch, heads * head_dim, dtype=q.dtype, device=q.device) if out is None else out
     if lse is None:
         lse = torch.empty(batch * heads, T, dtype=torch.float32, device=q.device)
-    d = _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale)
+    d = _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale, q_bh_rows, stat_bh_rows)
     if nsplit:
         d.reserved = int(nsplit)
     lib = _lib.load()
@@ -229,12 +234,14 @@ def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q
 
 def attn_prefix_bwd(q, k_cache, v_cache, o, lse, d_o, dqkv, dk_cache, dv_cache, batch, heads, head_dim, T,
                     cache_len, q_scale, accumulate_prefix, has_incoming, zero_slice_rows, colsum_dqkv_acc=None,
-                    delta=None):
-    """Writes dqkv [T*B, 3*H*Dh]; updates rows [0, cache_len) of the gradient caches."""
+                    delta=None, q_bh_rows=0, stat_bh_rows=0, dq_only=False):
+    """Writes dqkv [T*B, 3*H*Dh]; updates rows [0, cache_len) of the gradient caches.  dq_only: delta and
+    the q part of dqkv only (the k and v parts are then attn_suffix_dkdv's; no gradient cache is touched)."""
     _require_cuda(q, k_cache, v_cache, d_o, dqkv)
     if delta is None:
         delta = torch.empty(batch * heads, T, dtype=torch.float32, device=q.device)
-    d = _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale)
+    d = _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale, q_bh_rows, stat_bh_rows)
+    d.dq_only = int(dq_only)
     d.d_o, d.delta, d.dqkv = d_o.data_ptr(), delta.data_ptr(), dqkv.data_ptr()
     d.dk_cache, d.dv_cache = _p(dk_cache), _p(dv_cache)
     d.grad_cache_dtype = tp_dtype(dk_cache.dtype) if dk_cache is not None else d.dtype
@@ -245,6 +252,28 @@ def attn_prefix_bwd(q, k_cache, v_cache, o, lse, d_o, dqkv, dk_cache, dv_cache, 
         _lib.check(lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()), "tp_attn_prefix_bwd")
     _record("attn_bwd", (batch, heads, head_dim, T, cache_len),
             lambda: lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()))
+    return dqkv
+
+
+def attn_suffix_dkdv(k_cache, v_cache, q_all, d_o_all, lse_all, delta_all, dqkv, batch, heads, head_dim,
+                     key_begin, key_count, q_end):
+    """dK / dV of the keys [key_begin, key_begin + key_count) against every query position in
+    [key_begin, q_end), written into the k and v parts of dqkv [key_count * B, 3 * H * Dh].
+    q_all [B*H, Lq, Dh], lse_all / delta_all [B*H, Ls], d_o_all [>= q_end, B, H*Dh]: all indexed by position."""
+    _require_cuda(k_cache, v_cache, q_all, d_o_all, dqkv)
+    d = _lib.AttnSuffixDesc()
+    d.dtype = tp_dtype(q_all.dtype)
+    d.batch, d.heads, d.head_dim = batch, heads, head_dim
+    d.key_begin, d.key_count, d.q_end = key_begin, key_count, q_end
+    d.cache_rows, d.q_bh_rows, d.stat_bh_rows = k_cache.shape[1], q_all.shape[1], lse_all.shape[1]
+    d.k_cache, d.v_cache = k_cache.data_ptr(), v_cache.data_ptr()
+    d.q_all, d.d_o_all = q_all.data_ptr(), d_o_all.data_ptr()
+    d.lse_all, d.delta_all, d.dqkv = lse_all.data_ptr(), delta_all.data_ptr(), dqkv.data_ptr()
+    lib = _lib.load()
+    with _timed("attn_bwd", (batch, heads, head_dim, key_count, key_begin)):
+        _lib.check(lib.tp_attn_suffix_dkdv(ctypes.byref(d), _stream()), "tp_attn_suffix_dkdv")
+    _record("attn_bwd_dkdv", (batch, heads, head_dim, key_count, key_begin),
+            lambda: lib.tp_attn_suffix_dkdv(ctypes.byref(d), _stream()))
     return dqkv
 
 

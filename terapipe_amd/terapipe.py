@@ -81,6 +81,7 @@ class _StackBuffers:
         nl, E, F, H = layers.n_layers, layers.embedding_dim, layers.ffn_embedding_dim, layers.num_attention_heads
         L, Dh = runner.seq_len, layers.embedding_dim // layers.num_attention_heads
         self.dtype, self.device = dtype, device
+        self.position_indexed = runner.suffix_dkdv and dtype != torch.float32     # the one-pass kernel is 16-bit
         gdt = torch.float32 if runner.fp32_grad_cache else dtype
         kw = dict(dtype=dtype, device=device)
         f32 = dict(dtype=torch.float32, device=device)
@@ -90,19 +91,29 @@ class _StackBuffers:
             b = {}
             b["x"] = [torch.empty(R, E, **kw) for _ in range(nl + 1)]      # x[l] input of layer l; x[nl] output
             b["dx"] = [torch.empty(R, E, **kw) for _ in range(nl + 1)]     # gradient of the same
-            for name, width in (("xn", E), ("q", E), ("o", E), ("h", E), ("hn", E), ("a", F),
+            for name, width in (("xn", E), ("o", E), ("h", E), ("hn", E), ("a", F),
                                 ("dz1", F), ("dhn", E), ("dh", E), ("dqkv", 3 * E), ("dxn", E)):
                 b[name] = [torch.empty(R, width, **kw) for _ in range(nl)]
             b["z"] = [torch.empty(R, F, **kw) if layers.layers[l].activation == "gelu" else None for l in range(nl)]
             for name in ("mean1", "rstd1", "mean2", "rstd2"):
                 b[name] = [torch.empty(R, **f32) for _ in range(nl)]
-            b["lse"] = [torch.empty(R * H, **f32) for _ in range(nl)]
-            b["d_o"] = torch.empty(max(runner.seq_slices) * Bs, E, **kw)
-            b["delta"] = torch.empty(max(runner.seq_slices) * Bs * H, **f32)
+            if self.position_indexed:
+                # q, lse, delta and dO of every slice, indexed by position like the K/V caches: the dK/dV of
+                # a slice's keys are then one pass over all later positions and no gradient cache exists
+                b["q"] = [torch.zeros(Bs * H, L, Dh, **kw) for _ in range(nl)]
+                b["lse"] = [torch.zeros(Bs * H, L, **f32) for _ in range(nl)]
+                b["delta"] = [torch.zeros(Bs * H, L, **f32) for _ in range(nl)]
+                b["d_o"] = [torch.zeros(R, E, **kw) for _ in range(nl)]
+            else:
+                b["q"] = [torch.empty(R, E, **kw) for _ in range(nl)]
+                b["lse"] = [torch.empty(R * H, **f32) for _ in range(nl)]
+                b["d_o"] = torch.empty(max(runner.seq_slices) * Bs, E, **kw)
+                b["delta"] = torch.empty(max(runner.seq_slices) * Bs * H, **f32)
             # zero-filled once: rows beyond the current slice are read only under the causal mask, but
             # they must hold finite values (reference create_attn_cache zero-fills, transformer_models.py:257-261)
             b["cache"] = [torch.zeros(Bs * H, L, Dh, **kw) for _ in range(2 * nl)]
-            b["gcache"] = [torch.empty(Bs * H, L, Dh, dtype=gdt, device=device) for _ in range(2 * nl)]
+            b["gcache"] = (None if self.position_indexed else
+                           [torch.empty(Bs * H, L, Dh, dtype=gdt, device=device) for _ in range(2 * nl)])
             self.per_batch.append(b)
         self.small = torch.zeros(nl, core.small_acc_numel(E, F), **f32)
         self.small_views = [core.small_acc_views(self.small[l], E, F) for l in range(nl)]
@@ -128,9 +139,13 @@ def _forward_body(runner, ws, act, bufs, states):
             r0, r1 = P * Bs, (P + T) * Bs
             sts = []
             for l in range(nl):
+                if bufs.position_indexed:
+                    qv, lv, rows = pb["q"][l][:, P:], pb["lse"][l][:, P:], runner.seq_len
+                else:
+                    qv, lv, rows = pb["q"][l][r0:r1].view(Bs * H, T, E // H), pb["lse"][l][r0 * H:r1 * H].view(Bs * H, T), 0
                 bf = core.Bufs(xn=pb["xn"][l][r0:r1], mean1=pb["mean1"][l][r0:r1], rstd1=pb["rstd1"][l][r0:r1],
-                               q=pb["q"][l][r0:r1].view(Bs * H, T, E // H), o=pb["o"][l][r0:r1].view(T, Bs, E),
-                               lse=pb["lse"][l][r0 * H:r1 * H].view(Bs * H, T), h=pb["h"][l][r0:r1],
+                               q=qv, o=pb["o"][l][r0:r1].view(T, Bs, E), lse=lv, q_bh_rows=rows, stat_bh_rows=rows,
+                               h=pb["h"][l][r0:r1],
                                mean2=pb["mean2"][l][r0:r1], rstd2=pb["rstd2"][l][r0:r1], hn=pb["hn"][l][r0:r1],
                                a=pb["a"][l][r0:r1], z=None if pb["z"][l] is None else pb["z"][l][r0:r1],
                                out=pb["x"][l + 1][r0:r1])
@@ -162,6 +177,15 @@ def _backward_body(runner, ws, act, bufs, states):
             r0, r1 = P * Bs, (P + T) * Bs
             last = i == ns - 1
             for l in reversed(range(nl)):
+                if bufs.position_indexed:
+                    bf = core.Bufs(dz1=pb["dz1"][l][r0:r1], dhn=pb["dhn"][l][r0:r1], dh=pb["dh"][l][r0:r1],
+                                   d_o=pb["d_o"][l][r0:r1], dqkv=pb["dqkv"][l][r0:r1], dxn=pb["dxn"][l][r0:r1],
+                                   dx=pb["dx"][l][r0:r1], delta=pb["delta"][l][:, P:])
+                    core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), H, None, None,
+                                   None, False, None, False, False, False, activation=act[l], buf=bf,
+                                   suffix=dict(q_all=pb["q"][l], d_o_all=pb["d_o"][l], lse_all=pb["lse"][l],
+                                               delta_all=pb["delta"][l], q_end=L))
+                    continue
                 bf = core.Bufs(dz1=pb["dz1"][l][r0:r1], dhn=pb["dhn"][l][r0:r1], dh=pb["dh"][l][r0:r1],
                                d_o=pb["d_o"][:T * Bs], dqkv=pb["dqkv"][l][r0:r1], dxn=pb["dxn"][l][r0:r1],
                                dx=pb["dx"][l][r0:r1], delta=pb["delta"][:T * Bs * H].view(Bs * H, T))
@@ -285,6 +309,11 @@ class TeraPipe(nn.Module):
     layer-level autograd surface in transformer_models.py accumulates per slice instead).
     fp32_grad_cache: keep the cross-slice dK/dV accumulators in fp32 (one rounding when a slice's own
     rows are emitted) instead of the cache dtype the reference uses.
+    suffix_dkdv (fp16 / bf16): keep q, lse, delta and dO of every slice in position-indexed buffers and
+    compute the dK/dV of a slice's keys, when its backward runs, in one pass over all later query
+    positions (every later slice has run its backward by then) -- the same sum that the reference builds
+    up through the cache gradients, without gradient caches and their read-modify-write per slice.  With
+    False (and always in fp32) the gradient caches are used.
     use_hip_graph: after the first (eager) step, record the kernel launches of forward and of backward
     into two HIP graphs and replay them on later steps.  The runner's buffers are static and the
     launches depend only on shapes, so the replays compute the same thing without the per-launch host
@@ -292,7 +321,7 @@ class TeraPipe(nn.Module):
     """
 
     def __init__(self, layers, batch_size, seq_len, batch_slices, seq_slices, batch_dim=1, sequence_dim=0,
-                 fp32_grad_cache=True, use_hip_graph=False):
+                 fp32_grad_cache=True, use_hip_graph=False, suffix_dkdv=True):
         super().__init__()
         assert sum(batch_slices) == batch_size and sum(seq_slices) == seq_len
         assert batch_dim == 1 and sequence_dim == 0, "layers take [seq, batch, embed] inputs"
@@ -302,6 +331,7 @@ class TeraPipe(nn.Module):
         self.layers = layers
         self.fp32_grad_cache = fp32_grad_cache
         self.use_hip_graph = use_hip_graph
+        self.suffix_dkdv = suffix_dkdv
         self._sbufs = None
         self.last_caches = None
         self.keep_states = False   # debugging / tests: keep the per-slice saved activations of the last forward

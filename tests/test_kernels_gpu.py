@@ -248,6 +248,65 @@ def test_attn_prefix_fwd_bwd(dtype, T, B, H, Dh, P, L):
             assert_close(acc, dqkv.double().sum(0), dtype, "dqkv colsum" + tag)
 
 
+SUFFIX_CASES = [
+    # B, H, Dh, L (cache rows), slices
+    (2, 2, 64, 96, [32, 32, 32]),
+    (1, 2, 128, 256, [64, 96, 32, 64]),
+    (1, 3, 128, 200, [40, 7, 100, 33]),      # ragged: nothing aligned to the 32-row blocks
+    (2, 1, 64, 64, [5, 1, 20]),              # caches longer than the sequence
+    (1, 2, 128, 512, [128, 128, 128, 128]),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("B,H,Dh,L,slices", SUFFIX_CASES)
+def test_attn_position_indexed_and_suffix_dkdv(dtype, B, H, Dh, L, slices):
+    """The layout a runner uses that keeps every slice: q, lse, delta and dO live in position-indexed
+    buffers (as the K/V caches do); each slice's forward and dQ work on views of them (q_bh_rows /
+    stat_bh_rows), and dK/dV of a slice's keys come from ONE pass over all later query positions
+    (tp_attn_suffix_dkdv) instead of the gradient caches.  Slices run forward in order and backward in
+    reverse order, as terapipe.py:182-191 does; the check is the fp64 causal attention over the whole
+    sequence through the oracle's attention_core."""
+    ops = _ops()
+    E, BH, Ltot = H * Dh, B * H, sum(slices)
+    g = torch.Generator().manual_seed(Ltot + Dh)
+    q = _rnd((BH, L, Dh), dtype, g, 1.0)
+    kc, vc = _rnd((BH, L, Dh), dtype, g, Dh ** -0.25), _rnd((BH, L, Dh), dtype, g)
+    d_o = _rnd((Ltot, B, E), dtype, g)
+    qd, kd, vd, dod = q.to(DEV), kc.to(DEV), vc.to(DEV), d_o.to(DEV)
+    o_all = torch.empty(Ltot, B, E, dtype=dtype, device=DEV)
+    lse_all = torch.full((BH, L), 123.0, dtype=torch.float32, device=DEV)
+    delta_all = torch.full((BH, L), 321.0, dtype=torch.float32, device=DEV)
+    P = 0
+    for T in slices:
+        ops.attn_prefix_fwd(qd[:, P:], kd, vd, B, H, Dh, T, P, 1.0, out=o_all[P:P + T], lse=lse_all[:, P:],
+                            q_bh_rows=L, stat_bh_rows=L)
+        P += T
+    q64 = q[:, :Ltot].double().requires_grad_(True)
+    k64, v64 = kc[:, :Ltot].double().requires_grad_(True), vc[:, :Ltot].double().requires_grad_(True)
+    oref = _attn_ref(q64, k64, v64, B, H, Ltot, 0)
+    assert_close(o_all, oref, dtype, "o, all slices")
+    s = torch.bmm(q64, k64.transpose(1, 2)) + oracle.causal_prefix_mask(Ltot, 0, torch.float64)
+    assert_close(lse_all[:, :Ltot], torch.logsumexp(s, -1), torch.float32, "lse, all slices", 1e3)
+    assert (lse_all[:, Ltot:] == 123).all()
+    oref.backward(d_o.double())
+    dqkv_all = torch.zeros(Ltot * B, 3 * E, dtype=dtype, device=DEV)
+    for i in reversed(range(len(slices))):
+        T, P = slices[i], sum(slices[:i])
+        dqkv = dqkv_all[P * B:(P + T) * B]
+        ops.attn_prefix_bwd(qd[:, P:], kd, vd, o_all[P:P + T], lse_all[:, P:], dod[P:P + T], dqkv, None, None, B, H, Dh,
+                            T, P, 0.5, False, False, False, delta=delta_all[:, P:], q_bh_rows=L, stat_bh_rows=L,
+                            dq_only=True)
+        ops.attn_suffix_dkdv(kd, vd, qd, dod, lse_all, delta_all, dqkv, B, H, Dh, P, T, Ltot)
+    delta_ref = (oref.detach() * d_o.double()).view(Ltot, B, H, Dh).sum(-1).permute(1, 2, 0).reshape(BH, Ltot)
+    assert_close(delta_all[:, :Ltot], delta_ref, torch.float32, "delta", 1e3)
+    assert (delta_all[:, Ltot:] == 321).all()
+    dq, dk, dv = oracle.split_qkv(dqkv_all.view(Ltot, B, 3 * E).double().cpu(), H)
+    assert_close(dq, q64.grad * 0.5, dtype, "dq")
+    assert_close(dk, k64.grad, dtype, "dk over all later queries")
+    assert_close(dv, v64.grad, dtype, "dv over all later queries")
+
+
 def test_error_paths():
     """Bad arguments come back as status codes with a message; nothing is launched."""
     import ctypes

@@ -326,14 +326,15 @@ def test_terapipe_16bit_reduced_shapes(dtype, case):
     g = torch.Generator().manual_seed(17)
     x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
-    for fp32gc in (True, False):
-        runner, y, dx = _run_terapipe(ta, layers, x, dy, B, L, bs, ss, keep_states=True, fp32_grad_cache=fp32gc)
+    # the one-pass dK/dV over all later positions (default), then the gradient caches in fp32 and in dtype
+    for kw in (dict(), dict(suffix_dkdv=False, fp32_grad_cache=True), dict(suffix_dkdv=False, fp32_grad_cache=False)):
+        runner, y, dx = _run_terapipe(ta, layers, x, dy, B, L, bs, ss, keep_states=True, **kw)
         # oracle with the ReLU active set of this run (module docstring)
         leaf = [{k: v.clone().requires_grad_(True) for k, v in p.items()} for p in ps]
         yo, dxo, fco = oracle.terapipe_forward_backward(leaf, x.float(), dy.float(), H, bs, ss,
                                                         relu_masks=_relu_masks_from_states(runner.last_states))
         go = [{k: v.grad for k, v in p.items()} for p in leaf]
-        tag = "%s fp32gc=%s" % (case, fp32gc)
+        tag = "%s %s" % (case, kw)
         assert_close(y, yo, dtype, tag + " y")
         assert_close(dx, dxo, dtype, tag + " dx")
         for b in range(len(bs)):
