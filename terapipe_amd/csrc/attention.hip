@@ -1638,11 +1638,6 @@ struct SuffixArgs {
     long cache_rows, q_bhs, st_bhs;
 };
 
-__device__ __forceinline__ void dma4(const void* gptr, unsigned lds_wave_base) {
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off"
-                 :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)) : "memory");
-}
-
 template <typename T, int DH, int NW>
 __global__ __launch_bounds__(NW * 64) void attn_suffix_dkdv_kernel(SuffixArgs a) {
     typedef Elem<T> E;

@@ -366,6 +366,12 @@ __device__ __forceinline__ void dma16_saddr_lds(unsigned off, const void* sbase,
                  :: "v"(off), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)) : "memory");
 }
 
+// One dword per lane into 256 bytes of LDS at lds_wave_base (wave-uniform byte address).
+__device__ __forceinline__ void dma4(const void* gptr, unsigned lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off"
+                 :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)) : "memory");
+}
+
 template <typename T, int ROWS, int COLS, int NT> struct RowSlideDma {
     static constexpr int CPR = COLS / 8;
     static constexpr int TOTAL = ROWS * CPR;

@@ -483,17 +483,17 @@ static constexpr int kNumCU = 256;  // MI355X
 struct TileCfg { int bm, bn, bk, stages; };
 static const TileCfg kCfgs[] = {
     {64, 64, 64, 2},     // 0: register-staged kernel's 16-bit tile (fp32 uses 64 x 64 x 16)
-    {256, 256, 64, 2},   // 1: 8 waves of 128 x 64
-    {256, 128, 64, 3},   // 2: 8 waves of 64 x 64
+    {64, 64, 64, 2},     // 1: (register-staged kernel)
+    {64, 64, 64, 2},     // 2: (register-staged kernel)
     {128, 256, 64, 3},   // 3: 8 waves of 64 x 64
-    {256, 256, 32, 4},   // 4: 8 waves of 128 x 64
+    {64, 64, 64, 2},     // 4: (register-staged kernel)
     {128, 128, 64, 2},   // 5
-    {256, 128, 64, 3},   // 6: 4 waves of 128 x 64
+    {64, 64, 64, 2},     // 6: (register-staged kernel)
     {64, 64, 64, 2},     // 7: (register-staged kernel)
     {64, 64, 64, 4},     // 8
     {64, 64, 64, 2},     // 9: (register-staged kernel)
     {128, 128, 32, 4},   // 10
-    {64, 64, 64, 2},     // 11: (register-staged kernel)
+    {64, 256, 64, 3},    // 11
     {64, 64, 128, 4},    // 12
     {128, 128, 64, 3},   // 13
 };
@@ -542,19 +542,22 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     const long t128 = (long)((d->M + 127) / 128) * ((d->N + 127) / 128);
     const long t64 = (long)((d->M + 63) / 64) * ((d->N + 63) / 64);
     int cfg, ns = 1;
-    if (d->M > 64 && d->M <= 128 && t128 >= 64 && d->K >= 4096) {
-        // one row of 128-row tiles streaming the weight once
-        if (t128 >= 144) {
-            cfg = 3;            // 128 x 256 x 64, eight waves: half the activation re-reads of 128 x 128
-        } else {
-            // few tiles: three-stage 128 x 128 x 64 with k split so that two to three workgroups' worth of
-            // loads per CU are in flight
-            cfg = 13;
-            ns = (int)((512 + t128 - 1) / t128);
-            int maxs = d->K / 2048;
-            if (ns > maxs) ns = maxs;
-            if (ns > 8) ns = 8;
-        }
+    const long t256n = (d->N + 255) / 256;
+    if (d->M <= 64 && (long)d->N * d->K >= (64L << 20)) {
+        // a short activation against a large weight: 64 x 256 x 64 tiles stream the weight with a quarter
+        // of the activation re-reads of 64-wide tiles; k is split to about 200 workgroups
+        cfg = 11;
+        ns = (int)((208 + t256n / 2) / t256n);
+        int maxs = d->K / 1536;
+        if (ns > maxs) ns = maxs;
+        if (ns > 8) ns = 8;
+    } else if (d->M > 64 && d->M <= 128 && t128 >= 64 && d->K >= 4096) {
+        // one row of 128 x 256 x 64 tiles (eight waves) streaming the weight once
+        cfg = 3;
+        ns = t256n >= 176 ? 1 : (t256n >= 96 ? 3 : (int)((192 + t256n - 1) / t256n));
+        int maxs = d->K / 2048;
+        if (ns > maxs) ns = maxs;
+        if (ns > 8) ns = 8;
     } else if (t128 >= 144) {
         cfg = d->M <= 256 ? 13 : 5;     // short activations: the deeper ring keeps the weight stream going
         if (t128 < 224) {
@@ -588,13 +591,10 @@ static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
         gemm_kernel<T, AKM, BKM, 64, 64, 16, 2, 2><<<grid, 256, 0, s>>>(a);
     } else {
         switch (p.cfg) {
-        case 1: gemm_dma_kernel<T, AKM, BKM, 256, 256, 64, 2, 4, 2><<<grid, 512, 0, s>>>(a); break;
-        case 2: gemm_dma_kernel<T, AKM, BKM, 256, 128, 64, 4, 2, 3><<<grid, 512, 0, s>>>(a); break;
         case 3: gemm_dma_kernel<T, AKM, BKM, 128, 256, 64, 2, 4, 3><<<grid, 512, 0, s>>>(a); break;
-        case 4: gemm_dma_kernel<T, AKM, BKM, 256, 256, 32, 2, 4, 4><<<grid, 512, 0, s>>>(a); break;
         case 5: gemm_dma_kernel<T, AKM, BKM, 128, 128, 64, 2, 2, 2><<<grid, 256, 0, s>>>(a); break;
-        case 6: gemm_dma_kernel<T, AKM, BKM, 256, 128, 64, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
         case 8: gemm_dma_kernel<T, AKM, BKM, 64, 64, 64, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
+        case 11: gemm_dma_kernel<T, AKM, BKM, 64, 256, 64, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
         case 10: gemm_dma_kernel<T, AKM, BKM, 128, 128, 32, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
         case 12: gemm_dma_kernel<T, AKM, BKM, 64, 64, 128, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
         case 13: gemm_dma_kernel<T, AKM, BKM, 128, 128, 64, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
