@@ -7,8 +7,8 @@ One step = every sequence slice of one synthetic batch through the whole layer s
 caches growing slice by slice), then the reverse-order slice backward, with the loss
 ``sum(y * R)`` for a fixed random R (inputs N(0,1), weights N(0,0.02), all resident in HBM before the
 timed region).  Prints ONE JSON line: tokens/s, the MFMA roofline of the GEMM kernels (algorithmic
-flops / HIP-event kernel time, measured live in an extra instrumented step), the HBM figure of the
-prefix-attention kernels, and the CPU oracle timed on this host's cores on a bounded sample.
+flops / kernel time, measured live: the GEMM calls of one recorded step replayed in a HIP graph between
+two HIP events), the HBM figure of the prefix-attention kernels, and the CPU oracle timed on this host's cores on a bounded sample.
 """
 import argparse
 import json
@@ -26,6 +26,10 @@ if ROOT not in sys.path:
 PEAK_MFMA_16BIT = 2.5e15     # dense fp16/bf16 MFMA flop/s
 PEAK_MFMA_FP32 = 157.3e12
 PEAK_HBM = 8.0e12            # bytes/s
+
+# HBM bytes per tp_gemm call (FETCH_SIZE + WRITE_SIZE of the GEMM kernels of one step / calls), from the two
+# rocprofv3 --pmc runs summarised in profiles/bench_C2_gemm_hbm_traffic.pmc.txt; only measured for C2
+PMC_GEMM_TRAFFIC_BYTES = {"C2": 31.46e6}
 
 WORKLOADS = {
     # name: layers, hidden, heads, ffn, seq, batch, dtype, slices, weight std
@@ -95,7 +99,7 @@ def cpu_baseline(w, budget_layers=None):
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
     flops_layer = gemm_flops_per_step(w) / w["n_layers"]
-    sample_layers = budget_layers or max(1, min(w["n_layers"], int(4e12 // flops_layer)))
+    sample_layers = budget_layers or max(1, min(w["n_layers"], int(1.5e13 // flops_layer)))
     ps = oracle.init_stack_params(sample_layers, w["E"], w["F"], w["std"], torch.float32, seed=0)
     for p in ps:
         for v in p.values():
@@ -121,6 +125,9 @@ def main():
     ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 256 MiB device copy (torch copy_ kernel) before the steps: the "
+                         "known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     ap.add_argument("--eager", action="store_true",
                     help="launch every kernel from the host each step instead of replaying the runner's HIP graphs")
     args = ap.parse_args()
@@ -138,6 +145,12 @@ def main():
 
     layers, runner, x, R = build_model(w, device)
     runner.use_hip_graph = not args.eager
+    if args.copy_calibration:
+        src = torch.ones(64 << 20, dtype=torch.int32, device=device)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         one_step(layers, runner, x, R)
     torch.cuda.synchronize()
@@ -205,7 +218,7 @@ def main():
         out["roofline"] = {
             "kernel": "tp::gemm_dma_kernel / tp::gemm_kernel (all NT/NN/TN launches of one step, split-K reduce included)",
             "bound": "mfma", "achieved": achieved / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
-            "frac": achieved / peak, "traffic": None,
+            "frac": achieved / peak, "traffic": PMC_GEMM_TRAFFIC_BYTES.get(args.workload),
             "launches": g_calls, "avg_launch_us": g_ms * 1e3 / max(g_calls, 1),
             "algorithmic_flops_per_step": flops, "kernel_ms_per_step": g_ms,
             "method": "graph replay of the step's GEMM calls between two HIP events",
