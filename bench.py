@@ -128,6 +128,8 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy (torch copy_ kernel) before the steps: the "
                          "known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--slice-streams", type=int, default=1,
+                    help="streams the runner spreads consecutive slices over (1 = one chain of kernels)")
     ap.add_argument("--eager", action="store_true",
                     help="launch every kernel from the host each step instead of replaying the runner's HIP graphs")
     args = ap.parse_args()
@@ -145,6 +147,7 @@ def main():
 
     layers, runner, x, R = build_model(w, device)
     runner.use_hip_graph = not args.eager
+    runner.slice_streams = args.slice_streams
     if args.copy_calibration:
         src = torch.ones(64 << 20, dtype=torch.int32, device=device)
         dst = torch.empty_like(src)
@@ -170,7 +173,8 @@ def main():
         "dtype": w["dtype"], "data": "synthetic",
         "config": {"workload": "%s: %s" % (args.workload, w["desc"]),
                    "loss": "sum(y * R), R ~ N(0,1) fixed", "optimizer_step": "not part of the path",
-                   "launch": "eager" if args.eager else "HIP-graph replay of forward and of backward"},
+                   "launch": "eager" if args.eager else "HIP-graph replay of forward and of backward",
+                   "slice_streams": args.slice_streams},
     }
 
     if not args.no_roofline:

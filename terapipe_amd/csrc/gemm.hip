@@ -559,7 +559,9 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
         if (ns > maxs) ns = maxs;
         if (ns > 8) ns = 8;
     } else if (t128 >= 144) {
-        cfg = d->M <= 256 ? 13 : 5;     // short activations: the deeper ring keeps the weight stream going
+        // short activations: the deeper ring keeps the weight stream going; parameter gradients (both
+        // operands fetched with transpose reads): 128 x 128 x 32, four stages, two workgroups per CU
+        cfg = d->op == TP_GEMM_TN ? 10 : (d->M <= 256 ? 13 : 5);
         if (t128 < 224) {
             ns = (int)(448 / t128);
             int maxs = d->K / 1024;

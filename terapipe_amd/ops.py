@@ -107,12 +107,13 @@ class _timed:
 
 
 class Workspace:
-    """A grow-only scratch tensor per device (torch-owned), handed to calls that need workspace."""
+    """A grow-only scratch tensor per device and stream (torch-owned), handed to calls that need
+    workspace: kernels of different streams may run at the same time and must not share partial sums."""
     _bufs = {}
 
     @classmethod
     def get(cls, nbytes, device):
-        key = (device.type, device.index)
+        key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
         buf = cls._bufs.get(key)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)

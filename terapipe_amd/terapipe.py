@@ -123,37 +123,62 @@ class _StackBuffers:
         self.param_ptrs = [t.data_ptr() for w in ws for t in w.values()]
         self.fwd_graph = self.bwd_graph = None
         self.states = None
+        # streams for the slice lanes (see TeraPipe's slice_streams); the gradient-cache mode shares per-slice
+        # scratch between layers and stays on one stream
+        n = runner.slice_streams if self.position_indexed else 1
+        self.lanes = [torch.cuda.Stream(device=device) for _ in range(n)] if n > 1 else []
 
 
 def _forward_body(runner, ws, act, bufs, states):
     """Every (batch slice, sequence slice) through the whole layer stack, slice-major, reading the batch
     slices from bufs x[0] and leaving the outputs in bufs x[n_layers].  Launches kernels only (no
-    allocation, no host synchronisation), so it can be recorded into a HIP graph."""
+    allocation, no host synchronisation), so it can be recorded into a HIP graph.
+
+    With slice lanes (bufs.lanes) slice i runs on stream i mod n and its layer l waits for layer l of
+    slice i-1 (the K/V rows it attends to): consecutive slices then overlap one layer apart, which keeps
+    the chip busier than one chain of short kernels can."""
     layers = runner.layers
     nl, H, E = layers.n_layers, layers.num_attention_heads, layers.embedding_dim
+    lanes = bufs.lanes
+    main = torch.cuda.current_stream()
+    for st in lanes:
+        st.wait_stream(main)
     for b, Bs in enumerate(runner.batch_slices):
         pb = bufs.per_batch[b]
         cache = pb["cache"]
         P = 0
+        prev_done = None
         for i, T in enumerate(runner.seq_slices):
             r0, r1 = P * Bs, (P + T) * Bs
-            sts = []
-            for l in range(nl):
-                if bufs.position_indexed:
-                    qv, lv, rows = pb["q"][l][:, P:], pb["lse"][l][:, P:], runner.seq_len
-                else:
-                    qv, lv, rows = pb["q"][l][r0:r1].view(Bs * H, T, E // H), pb["lse"][l][r0 * H:r1 * H].view(Bs * H, T), 0
-                bf = core.Bufs(xn=pb["xn"][l][r0:r1], mean1=pb["mean1"][l][r0:r1], rstd1=pb["rstd1"][l][r0:r1],
-                               q=qv, o=pb["o"][l][r0:r1].view(T, Bs, E), lse=lv, q_bh_rows=rows, stat_bh_rows=rows,
-                               h=pb["h"][l][r0:r1],
-                               mean2=pb["mean2"][l][r0:r1], rstd2=pb["rstd2"][l][r0:r1], hn=pb["hn"][l][r0:r1],
-                               a=pb["a"][l][r0:r1], z=None if pb["z"][l] is None else pb["z"][l][r0:r1],
-                               out=pb["x"][l + 1][r0:r1])
-                _, st = core.layer_fwd(ws[l], pb["x"][l][r0:r1].view(T, Bs, E), H, cache[2 * l], cache[2 * l + 1],
-                                       P, act[l], need_state=True, buf=bf)
-                sts.append(st)
+            sts, done = [], []
+            st_i = lanes[i % len(lanes)] if lanes else main
+            with torch.cuda.stream(st_i):
+                for l in range(nl):
+                    if lanes and prev_done is not None:
+                        st_i.wait_event(prev_done[l])
+                    if bufs.position_indexed:
+                        qv, lv, rows = pb["q"][l][:, P:], pb["lse"][l][:, P:], runner.seq_len
+                    else:
+                        qv, lv, rows = (pb["q"][l][r0:r1].view(Bs * H, T, E // H),
+                                        pb["lse"][l][r0 * H:r1 * H].view(Bs * H, T), 0)
+                    bf = core.Bufs(xn=pb["xn"][l][r0:r1], mean1=pb["mean1"][l][r0:r1], rstd1=pb["rstd1"][l][r0:r1],
+                                   q=qv, o=pb["o"][l][r0:r1].view(T, Bs, E), lse=lv, q_bh_rows=rows,
+                                   stat_bh_rows=rows, h=pb["h"][l][r0:r1],
+                                   mean2=pb["mean2"][l][r0:r1], rstd2=pb["rstd2"][l][r0:r1], hn=pb["hn"][l][r0:r1],
+                                   a=pb["a"][l][r0:r1], z=None if pb["z"][l] is None else pb["z"][l][r0:r1],
+                                   out=pb["x"][l + 1][r0:r1])
+                    _, st = core.layer_fwd(ws[l], pb["x"][l][r0:r1].view(T, Bs, E), H, cache[2 * l], cache[2 * l + 1],
+                                           P, act[l], need_state=True, buf=bf)
+                    sts.append(st)
+                    if lanes:
+                        ev = torch.cuda.Event()
+                        ev.record(st_i)
+                        done.append(ev)
+            prev_done = done
             states[b, i] = sts
             P += T                                                               # terapipe.py:264
+    for st in lanes:
+        main.wait_stream(st)
 
 
 def _backward_body(runner, ws, act, bufs, states):
@@ -166,26 +191,43 @@ def _backward_body(runner, ws, act, bufs, states):
     nb, ns = len(runner.batch_slices), len(runner.seq_slices)
     L = runner.seq_len
     ops.zero_(bufs.small)
+    lanes = bufs.lanes
+    main = torch.cuda.current_stream()
+    for st in lanes:
+        st.wait_stream(main)
     for b in reversed(range(nb)):
         Bs = runner.batch_slices[b]
         pb = bufs.per_batch[b]
         gc = pb["gcache"]
         P = L
+        later_done = None
         for i in reversed(range(ns)):
             T = runner.seq_slices[i]
             P -= T
             r0, r1 = P * Bs, (P + T) * Bs
             last = i == ns - 1
+            if bufs.position_indexed:
+                # slice lanes: layer l of slice i waits for layer l of slice i+1 (whose dO and delta the
+                # one-pass dK/dV reads, and through it for every later slice)
+                st_i = lanes[i % len(lanes)] if lanes else main
+                done = [None] * nl
+                with torch.cuda.stream(st_i):
+                    for l in reversed(range(nl)):
+                        if lanes and later_done is not None:
+                            st_i.wait_event(later_done[l])
+                        bf = core.Bufs(dz1=pb["dz1"][l][r0:r1], dhn=pb["dhn"][l][r0:r1], dh=pb["dh"][l][r0:r1],
+                                       d_o=pb["d_o"][l][r0:r1], dqkv=pb["dqkv"][l][r0:r1], dxn=pb["dxn"][l][r0:r1],
+                                       dx=pb["dx"][l][r0:r1], delta=pb["delta"][l][:, P:])
+                        core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), H, None, None,
+                                       None, False, None, False, False, False, activation=act[l], buf=bf,
+                                       suffix=dict(q_all=pb["q"][l], d_o_all=pb["d_o"][l], lse_all=pb["lse"][l],
+                                                   delta_all=pb["delta"][l], q_end=L))
+                        if lanes:
+                            done[l] = torch.cuda.Event()
+                            done[l].record(st_i)
+                later_done = done
+                continue
             for l in reversed(range(nl)):
-                if bufs.position_indexed:
-                    bf = core.Bufs(dz1=pb["dz1"][l][r0:r1], dhn=pb["dhn"][l][r0:r1], dh=pb["dh"][l][r0:r1],
-                                   d_o=pb["d_o"][l][r0:r1], dqkv=pb["dqkv"][l][r0:r1], dxn=pb["dxn"][l][r0:r1],
-                                   dx=pb["dx"][l][r0:r1], delta=pb["delta"][l][:, P:])
-                    core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), H, None, None,
-                                   None, False, None, False, False, False, activation=act[l], buf=bf,
-                                   suffix=dict(q_all=pb["q"][l], d_o_all=pb["d_o"][l], lse_all=pb["lse"][l],
-                                               delta_all=pb["delta"][l], q_end=L))
-                    continue
                 bf = core.Bufs(dz1=pb["dz1"][l][r0:r1], dhn=pb["dhn"][l][r0:r1], dh=pb["dh"][l][r0:r1],
                                d_o=pb["d_o"][:T * Bs], dqkv=pb["dqkv"][l][r0:r1], dxn=pb["dxn"][l][r0:r1],
                                dx=pb["dx"][l][r0:r1], delta=pb["delta"][:T * Bs * H].view(Bs * H, T))
@@ -194,6 +236,8 @@ def _backward_body(runner, ws, act, bufs, states):
                 core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), H,
                                gc[2 * l], gc[2 * l + 1], None, False, None, accumulate_prefix=not last,
                                has_incoming=not last, zero_slice_rows=False, activation=act[l], buf=bf)
+    for st in lanes:
+        main.wait_stream(st)
     # parameter gradients over all tokens: dW = dY_all^T X_all (one GEMM per weight and batch slice),
     # bias gradients = column sums of dY_all, LayerNorm gradients from (dy, x, mean, rstd) of all rows
     for l in range(nl):
@@ -314,6 +358,10 @@ class TeraPipe(nn.Module):
     positions (every later slice has run its backward by then) -- the same sum that the reference builds
     up through the cache gradients, without gradient caches and their read-modify-write per slice.  With
     False (and always in fp32) the gradient caches are used.
+    slice_streams (with suffix_dkdv, fp16 / bf16): slice i runs on stream i mod slice_streams; layer l of a
+    slice waits (by event) for layer l of the previous slice in forward -- the next slice in backward --
+    so consecutive slices run one layer apart at the same time.  Same kernels, same arguments, same
+    results; the overlap fills the chip where one chain of 256-row kernels cannot.
     use_hip_graph: after the first (eager) step, record the kernel launches of forward and of backward
     into two HIP graphs and replay them on later steps.  The runner's buffers are static and the
     launches depend only on shapes, so the replays compute the same thing without the per-launch host
@@ -321,7 +369,7 @@ class TeraPipe(nn.Module):
     """
 
     def __init__(self, layers, batch_size, seq_len, batch_slices, seq_slices, batch_dim=1, sequence_dim=0,
-                 fp32_grad_cache=True, use_hip_graph=False, suffix_dkdv=True):
+                 fp32_grad_cache=True, use_hip_graph=False, suffix_dkdv=True, slice_streams=1):
         super().__init__()
         assert sum(batch_slices) == batch_size and sum(seq_slices) == seq_len
         assert batch_dim == 1 and sequence_dim == 0, "layers take [seq, batch, embed] inputs"
@@ -332,6 +380,7 @@ class TeraPipe(nn.Module):
         self.fp32_grad_cache = fp32_grad_cache
         self.use_hip_graph = use_hip_graph
         self.suffix_dkdv = suffix_dkdv
+        self.slice_streams = int(slice_streams)
         self._sbufs = None
         self.last_caches = None
         self.keep_states = False   # debugging / tests: keep the per-slice saved activations of the last forward

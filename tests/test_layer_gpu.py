@@ -430,7 +430,8 @@ def test_hip_graph_replays_match_eager(dtype):
     bs, ss = [1, 1], [32, 48, 16]
     ps = make_params(n_layers, E, Fd, dtype, seed=6)
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps, "gelu")
-    graph_runner = ta.TeraPipe(layers, B, L, bs, ss, use_hip_graph=True)
+    # three slice lanes as well (16 bit): the recorded graphs then hold the cross-stream dependencies
+    graph_runner = ta.TeraPipe(layers, B, L, bs, ss, use_hip_graph=True, slice_streams=3)
     eager_runner = ta.TeraPipe(layers, B, L, bs, ss)
 
     def step(runner, x, dy):
@@ -457,3 +458,27 @@ def test_hip_graph_replays_match_eager(dtype):
             # the vector-parameter gradients are summed with atomics: compare to rounding, not bitwise
             assert_close(a, b, dtype, "replay %d: parameter gradient" % seed, 0.05 if dtype == torch.float32 else 1.0)
     assert graph_runner._sbufs.fwd_graph is not None and graph_runner._sbufs.bwd_graph is not None
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_slice_streams_match_single_stream(dtype):
+    """slice_streams > 1 runs consecutive slices on different streams, one layer apart: same kernels and
+    arguments, so outputs and input gradients are bit-identical to the single-stream run (the vector-
+    parameter gradients are summed with atomics and compared to rounding)."""
+    ta = _mods()
+    n_layers, E, H, Fd, L, B = 3, 512, 4, 2048, 512, 2
+    ss = [128, 32, 96, 64, 64, 128]
+    ps = make_params(n_layers, E, Fd, dtype, seed=9)
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    g = torch.Generator().manual_seed(5)
+    x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
+    _, y1, dx1 = _run_terapipe(ta, layers, x, dy, B, L, [B], ss)
+    g1 = [p.grad.clone() for p in layers.parameters()]
+    for n in (2, 4):
+        for rep in range(2):
+            _, y2, dx2 = _run_terapipe(ta, layers, x, dy, B, L, [B], ss, slice_streams=n)
+            torch.cuda.synchronize()
+            assert torch.equal(y2, y1), "y with %d lanes" % n
+            assert torch.equal(dx2, dx1), "dx with %d lanes" % n
+            for a, b in zip([p.grad for p in layers.parameters()], g1):
+                assert_close(a, b, dtype, "parameter gradient with %d lanes" % n, 1.0)
