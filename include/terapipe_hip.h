@@ -58,6 +58,18 @@ int tp_layernorm_bwd(const void* dy, const void* x, const float* mean, const flo
                      float* dbeta_acc, float* colsum_dres_acc, float* colsum_dx_acc, int M, int E,
                      int dtype, void* stream);
 
+/* The same two kernels fed from the partial sums a k-split tp_gemm with defer_reduce left in its workspace
+ * (partials[z][m][e], z < nsplit, fp32): the input row is sum_z partials (+ bias[e]) (+ residual[m][e]),
+ * rounded to dtype exactly as the GEMM's own reduce would have, written to x_out / dy_out (the tensor the
+ * GEMM was asked for) and normalised from there.  Saves the reduce launch and one pass over the tensor. */
+int tp_layernorm_fwd_partials(const float* partials, int nsplit, const void* bias, const void* residual,
+                              void* x_out, const void* gamma, const void* beta, void* y, float* mean,
+                              float* rstd, int M, int E, float eps, int dtype, void* stream);
+int tp_layernorm_bwd_partials(const float* partials, int nsplit, void* dy_out, const void* x,
+                              const float* mean, const float* rstd, const void* gamma, const void* dres,
+                              void* dx, float* dgamma_acc, float* dbeta_acc, float* colsum_dres_acc,
+                              float* colsum_dx_acc, int M, int E, int dtype, void* stream);
+
 /* LayerNorm parameter gradients over a block of rows (used once per layer over ALL tokens of a step
  * when the per-slice tp_layernorm_bwd calls pass NULL accumulators):
  *   dgamma_acc[E] += sum_m dy[m] * (x[m] - mean[m]) * rstd[m],   dbeta_acc[E] += sum_m dy[m].
@@ -114,8 +126,16 @@ typedef struct tp_gemm_desc {
     int32_t reserved;                   /* 0 = automatic; bits 0-7: tile configuration + 1, bits 8-15: k splits (tuning, tests) */
     int64_t q_bh_rows;                  /* rows per (b,h) block of q: 0 = T (compact [B*H,T,Dh]); a runner that
                                            keeps the queries of every slice passes L_max and q offset to row P */
+    int32_t defer_reduce;               /* 1 (STORE / BIAS_RESIDUAL epilogues only): when the plan splits k
+                                           (tp_gemm_splits > 1) leave the fp32 partial sums [splits][M][N] in the
+                                           workspace and write nothing else; the LayerNorm that consumes C sums them,
+                                           applies bias / residual and writes C (tp_layernorm_fwd/bwd_partials).
+                                           Without a split the GEMM completes as usual. */
+    int32_t reserved4;
 } tp_gemm_desc;
 
+/* number of k splits the plan uses for this product (1 = none; 0 = invalid descriptor) */
+int tp_gemm_splits(const tp_gemm_desc* d);
 size_t tp_gemm_workspace_bytes(const tp_gemm_desc* d);
 int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_bytes, void* stream);
 

@@ -48,9 +48,12 @@ class Bufs:
     """Optional preallocated outputs for one layer-slice call (views into the runner's per-layer
     buffers).  Any attribute left at None is allocated by the call.  q_bh_rows / stat_bh_rows: q and
     lse / delta are views, starting at the slice's position, into position-indexed buffers with that many
-    rows per (batch, head) -- 0 means compact [B*H, T, ...] tensors."""
+    rows per (batch, head) -- 0 means compact [B*H, T, ...] tensors.  x_pending: the layer input is still the
+    partial sums of the previous layer's k-split fc2 GEMM (ops.PendingReduce) and the first LayerNorm
+    finishes it; defer_out: leave this layer's fc2 output in that state, returned in out_pending."""
     __slots__ = ("xn", "mean1", "rstd1", "q", "o", "lse", "h", "mean2", "rstd2", "hn", "a", "z", "out",
-                 "dz1", "dhn", "dh", "d_o", "dqkv", "dxn", "dx", "delta", "q_bh_rows", "stat_bh_rows")
+                 "dz1", "dhn", "dh", "d_o", "dqkv", "dxn", "dx", "delta", "q_bh_rows", "stat_bh_rows",
+                 "x_pending", "defer_out", "out_pending")
 
     def __init__(self, **kw):
         for n in self.__slots__:
@@ -90,14 +93,15 @@ def layer_fwd(w, x, heads, k_cache, v_cache, cache_len, activation="relu", need_
     F = w["fc1.weight"].shape[0]
     dt, dev = x.dtype, x.device
     x2d = x.view(M, E)
-    xn, mean1, rstd1 = ops.layernorm_fwd(x2d, w["attn_ln.weight"], w["attn_ln.bias"], out=buf.xn, mean=buf.mean1,
-                                         rstd=buf.rstd1)
+    xn, mean1, rstd1 = ops.layernorm_fwd(buf.x_pending if buf.x_pending is not None else x2d, w["attn_ln.weight"],
+                                         w["attn_ln.bias"], out=buf.xn, mean=buf.mean1, rstd=buf.rstd1)
     q, o, lse = attention_fwd(w, xn, T, B, heads, k_cache, v_cache, cache_len, buf)
     o2d = o.view(M, E)
     h = _buf(buf.h, (M, E), dt, dev)
-    ops.gemm(TP_GEMM_NT, o2d, w["attn.out_proj.weight"], M, E, E, C=h, epilogue=TP_EPI_BIAS_RESIDUAL,
-             bias=w["attn.out_proj.bias"], residual=x2d)
-    hn, mean2, rstd2 = ops.layernorm_fwd(h, w["fc_ln.weight"], w["fc_ln.bias"], out=buf.hn, mean=buf.mean2,
+    # a k-split out_proj leaves its partial sums to the LayerNorm that follows directly (which then writes h)
+    h_in = ops.gemm(TP_GEMM_NT, o2d, w["attn.out_proj.weight"], M, E, E, C=h, epilogue=TP_EPI_BIAS_RESIDUAL,
+                    bias=w["attn.out_proj.bias"], residual=x2d, defer_reduce=True)
+    hn, mean2, rstd2 = ops.layernorm_fwd(h_in, w["fc_ln.weight"], w["fc_ln.bias"], out=buf.hn, mean=buf.mean2,
                                          rstd=buf.rstd2)
     a = _buf(buf.a, (M, F), dt, dev)
     z = None
@@ -110,8 +114,10 @@ def layer_fwd(w, x, heads, k_cache, v_cache, cache_len, activation="relu", need_
     else:
         raise ValueError("activation must be 'relu' or 'gelu'")
     out = _buf(buf.out, (M, E), dt, dev)
-    ops.gemm(TP_GEMM_NT, a, w["fc2.weight"], M, E, F, C=out, epilogue=TP_EPI_BIAS_RESIDUAL,
-             bias=w["fc2.bias"], residual=h)
+    res = ops.gemm(TP_GEMM_NT, a, w["fc2.weight"], M, E, F, C=out, epilogue=TP_EPI_BIAS_RESIDUAL,
+                   bias=w["fc2.bias"], residual=h, defer_reduce=bool(buf.defer_out))
+    if buf.defer_out:
+        buf.out_pending = res if isinstance(res, ops.PendingReduce) else None
     st = None
     if need_state:
         st = SliceState()
@@ -162,10 +168,11 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
     if wgrad is not None:
         _wgrad(wgrad["fc2.weight"], accumulate_wgrad, dout2d, st.a, E, F, M)
     dhn = _buf(buf.dhn, (M, E), dt, dev)
-    ops.gemm(TP_GEMM_NN, dz1, w["fc1.weight"], M, E, F, C=dhn)
     if wgrad is not None:
         _wgrad(wgrad["fc1.weight"], accumulate_wgrad, dz1, st.hn, F, E, M)
-    dh = ops.layernorm_bwd(dhn, st.h, st.mean2, st.rstd2, w["fc_ln.weight"], dout2d, sa.get("fc_ln.weight"),
+    # a k-split data-gradient GEMM leaves its partial sums to the LayerNorm backward that follows directly
+    dhn_in = ops.gemm(TP_GEMM_NN, dz1, w["fc1.weight"], M, E, F, C=dhn, defer_reduce=True)
+    dh = ops.layernorm_bwd(dhn_in, st.h, st.mean2, st.rstd2, w["fc_ln.weight"], dout2d, sa.get("fc_ln.weight"),
                            sa.get("fc_ln.bias"), sa.get("fc2.bias"), sa.get("attn.out_proj.bias"), out=buf.dh)
     # attention
     d_o = _buf(buf.d_o, (M, E), dt, dev)
@@ -187,9 +194,9 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
         if "attn.in_proj.bias" in sa:
             ops.colsum_acc(dqkv, sa["attn.in_proj.bias"])
     dxn = _buf(buf.dxn, (M, E), dt, dev)
-    ops.gemm(TP_GEMM_NN, dqkv, w["attn.in_proj.weight"], M, E, 3 * E, C=dxn)
     if wgrad is not None:
         _wgrad(wgrad["attn.in_proj.weight"], accumulate_wgrad, dqkv, st.xn, 3 * E, E, M)
-    dx = ops.layernorm_bwd(dxn, st.x, st.mean1, st.rstd1, w["attn_ln.weight"], dh, sa.get("attn_ln.weight"),
+    dxn_in = ops.gemm(TP_GEMM_NN, dqkv, w["attn.in_proj.weight"], M, E, 3 * E, C=dxn, defer_reduce=True)
+    dx = ops.layernorm_bwd(dxn_in, st.x, st.mean1, st.rstd1, w["attn_ln.weight"], dh, sa.get("attn_ln.weight"),
                            sa.get("attn_ln.bias"), None, None, out=buf.dx)
     return dx.view(T, B, E)

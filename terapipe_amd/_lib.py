@@ -36,6 +36,7 @@ class GemmDesc(ctypes.Structure):
         ("cache_rows", c_int64),
         ("q_scale", c_float), ("reserved", c_int32),
         ("q_bh_rows", c_int64),
+        ("defer_reduce", c_int32), ("reserved4", c_int32),
     ]
 
 
@@ -79,6 +80,9 @@ SYMBOLS = {
     "tp_layernorm_fwd": (c_int, [c_void_p] * 6 + [c_int, c_int, c_float, c_int, c_void_p]),
     "tp_layernorm_bwd": (c_int, [c_void_p] * 11 + [c_int, c_int, c_int, c_void_p]),
     "tp_ln_param_grads": (c_int, [c_void_p] * 6 + [c_int, c_int, c_int, c_void_p]),
+    "tp_layernorm_fwd_partials": (c_int, [c_void_p, c_int] + [c_void_p] * 8 + [c_int, c_int, c_float, c_int, c_void_p]),
+    "tp_layernorm_bwd_partials": (c_int, [c_void_p, c_int] + [c_void_p] * 11 + [c_int, c_int, c_int, c_void_p]),
+    "tp_gemm_splits": (c_int, [ctypes.POINTER(GemmDesc)]),
     "tp_gemm_workspace_bytes": (c_size_t, [ctypes.POINTER(GemmDesc)]),
     "tp_gemm": (c_int, [ctypes.POINTER(GemmDesc), c_void_p, c_size_t, c_void_p]),
     "tp_attn_fwd_workspace_bytes": (c_size_t, [ctypes.POINTER(AttnDesc)]),

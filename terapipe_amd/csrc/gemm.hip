@@ -612,7 +612,7 @@ static void launch_gemm(const tp_gemm_desc* d, const GemmPlan& p, const GemmArgs
     case TP_GEMM_NN: launch_cfg<T, true, false>(p, a, s); break;
     default: launch_cfg<T, false, false>(p, a, s); break;
     }
-    if (p.nsplit > 1) {
+    if (p.nsplit > 1 && !d->defer_reduce) {
         dim3 grid((d->N + 255) / 256, (d->M + 31) / 32);
         gemm_splitk_reduce_kernel<T><<<grid, 256, 0, s>>>(a);
     }
@@ -637,6 +637,10 @@ static int validate_gemm(const tp_gemm_desc* d) {
     if (d->lda < a_cols || d->ldb < b_cols) { set_error("tp_gemm: leading dimension smaller than row"); return TP_ERR_ARG; }
     if (((uintptr_t)d->A | (uintptr_t)d->B) & 15) { set_error("tp_gemm: operands must be 16-byte aligned"); return TP_ERR_ARG; }
     if (d->N % 8) { set_error("tp_gemm: N=%d must be a multiple of 8", d->N); return TP_ERR_UNSUPPORTED; }
+    if (d->defer_reduce && ((d->epilogue != TP_EPI_STORE && d->epilogue != TP_EPI_BIAS_RESIDUAL) || d->colsum_acc)) {
+        set_error("tp_gemm: defer_reduce needs the STORE or BIAS_RESIDUAL epilogue and no colsum_acc");
+        return TP_ERR_ARG;
+    }
     if (d->epilogue != TP_EPI_QKV_SCATTER) {
         if (!d->C || d->ldc < d->N || d->ldc % ch || ((uintptr_t)d->C & 15)) { set_error("tp_gemm: bad C / ldc / alignment"); return TP_ERR_ARG; }
     }
@@ -674,6 +678,11 @@ static int validate_gemm(const tp_gemm_desc* d) {
 }
 
 }  // namespace tp
+
+extern "C" int tp_gemm_splits(const tp_gemm_desc* d) {
+    if (tp::validate_gemm(d) != TP_OK) return 0;
+    return tp::plan_gemm(d).nsplit;
+}
 
 extern "C" size_t tp_gemm_workspace_bytes(const tp_gemm_desc* d) {
     if (tp::validate_gemm(d) != TP_OK) return 0;

@@ -52,8 +52,54 @@ template <typename T> __device__ __forceinline__ void store_chunk(T* p, const fl
     *reinterpret_cast<uint4*>(p) = raw;
 }
 
+// Where the kernels take their input row from when it is still the fp32 partial sums of a k-split GEMM:
+// value = sum_z partial[z][row][col] (+ bias[col]) (+ resid[row][col]), rounded to T, written to out16 (the
+// tensor the split-K reduce kernel would have produced) and used from there on.  partial == nullptr: the
+// row is read from the kernel's ordinary input pointer.
+struct LnPartialSrc {
+    const float* partial; int nsplit; long zstride;
+    const void* bias; const void* resid; void* out16;
+};
+
+template <typename T>
+__device__ __forceinline__ void load_input_chunk(const LnPartialSrc& ps, const T* direct, long row, int c, int E,
+                                                 float* out) {
+    constexpr int CH = 16 / sizeof(T);
+    const long off = row * E + (long)c * CH;
+    if (ps.partial == nullptr) {
+        load_chunk<T>(direct + off, out);
+        return;
+    }
+#pragma unroll
+    for (int e = 0; e < CH; ++e) out[e] = 0.f;
+    for (int z = 0; z < ps.nsplit; ++z) {
+        const float* pp = ps.partial + (long)z * ps.zstride + off;
+#pragma unroll
+        for (int q = 0; q < CH / 4; ++q) {
+            const float4 v = *reinterpret_cast<const float4*>(pp + 4 * q);
+            out[4 * q] += v.x; out[4 * q + 1] += v.y; out[4 * q + 2] += v.z; out[4 * q + 3] += v.w;
+        }
+    }
+    if (ps.bias) {
+        float b[CH];
+        load_chunk<T>(reinterpret_cast<const T*>(ps.bias) + (long)c * CH, b);
+#pragma unroll
+        for (int e = 0; e < CH; ++e) out[e] += b[e];
+    }
+    if (ps.resid) {
+        float r[CH];
+        load_chunk<T>(reinterpret_cast<const T*>(ps.resid) + off, r);
+#pragma unroll
+        for (int e = 0; e < CH; ++e) out[e] += r[e];
+    }
+    // round through T exactly as the stand-alone reduce kernel does, and keep the rounded tensor
+#pragma unroll
+    for (int e = 0; e < CH; ++e) out[e] = Elem<T>::to_float(Elem<T>::from_float(out[e]));
+    store_chunk<T>(reinterpret_cast<T*>(ps.out16) + off, out);
+}
+
 template <typename T, int MAXC>
-__global__ __launch_bounds__(1024) void ln_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
+__global__ __launch_bounds__(1024) void ln_fwd_kernel(LnPartialSrc ps, const T* __restrict__ x, const T* __restrict__ gamma,
                                                       const T* __restrict__ beta, T* __restrict__ y,
                                                       float* __restrict__ mean, float* __restrict__ rstd,
                                                       int M, int E, float eps) {
@@ -61,14 +107,13 @@ __global__ __launch_bounds__(1024) void ln_fwd_kernel(const T* __restrict__ x, c
     __shared__ float scratch[16];
     const int row = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
     const int nch = E / CH;
-    const T* xr = x + (long)row * E;
     float v[MAXC][CH];
     float s[1] = {0.f};
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
         int c = tid + i * nt;
         if (c < nch) {
-            load_chunk<T>(xr + (long)c * CH, v[i]);
+            load_input_chunk<T>(ps, x, row, c, E, v[i]);
 #pragma unroll
             for (int e = 0; e < CH; ++e) s[0] += v[i][e];
         }
@@ -102,7 +147,7 @@ __global__ __launch_bounds__(1024) void ln_fwd_kernel(const T* __restrict__ x, c
 }
 
 template <typename T, int MAXC>
-__global__ __launch_bounds__(1024) void ln_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+__global__ __launch_bounds__(1024) void ln_bwd_kernel(LnPartialSrc ps, const T* __restrict__ dy, const T* __restrict__ x,
                                                       const float* __restrict__ mean, const float* __restrict__ rstd,
                                                       const T* __restrict__ gamma, const T* __restrict__ dres,
                                                       T* __restrict__ dx, float* dgamma, float* dbeta,
@@ -128,7 +173,7 @@ __global__ __launch_bounds__(1024) void ln_bwd_kernel(const T* __restrict__ dy, 
             int c = tid + i * nt;
             if (c < nch) {
                 float d[CH], xv[CH];
-                load_chunk<T>(dy + (long)row * E + (long)c * CH, d);
+                load_input_chunk<T>(ps, dy, row, c, E, d);
                 load_chunk<T>(x + (long)row * E + (long)c * CH, xv);
 #pragma unroll
                 for (int e = 0; e < CH; ++e) {
@@ -241,23 +286,23 @@ static int ln_geometry(int E, int dtype, int* threads, int* maxc) {
 }
 
 template <typename T>
-static void launch_ln_fwd(int maxc, int nt, const void* x, const void* gamma, const void* beta, void* y,
-                          float* mean, float* rstd, int M, int E, float eps, hipStream_t s) {
+static void launch_ln_fwd(int maxc, int nt, const LnPartialSrc& ps, const void* x, const void* gamma,
+                          const void* beta, void* y, float* mean, float* rstd, int M, int E, float eps, hipStream_t s) {
     const T* xp = (const T*)x; const T* gp = (const T*)gamma; const T* bp = (const T*)beta; T* yp = (T*)y;
-    if (maxc == 1) ln_fwd_kernel<T, 1><<<M, nt, 0, s>>>(xp, gp, bp, yp, mean, rstd, M, E, eps);
-    else if (maxc == 2) ln_fwd_kernel<T, 2><<<M, nt, 0, s>>>(xp, gp, bp, yp, mean, rstd, M, E, eps);
-    else ln_fwd_kernel<T, 4><<<M, nt, 0, s>>>(xp, gp, bp, yp, mean, rstd, M, E, eps);
+    if (maxc == 1) ln_fwd_kernel<T, 1><<<M, nt, 0, s>>>(ps, xp, gp, bp, yp, mean, rstd, M, E, eps);
+    else if (maxc == 2) ln_fwd_kernel<T, 2><<<M, nt, 0, s>>>(ps, xp, gp, bp, yp, mean, rstd, M, E, eps);
+    else ln_fwd_kernel<T, 4><<<M, nt, 0, s>>>(ps, xp, gp, bp, yp, mean, rstd, M, E, eps);
 }
 
 template <typename T>
-static void launch_ln_bwd(int maxc, int nt, int grid, const void* dy, const void* x, const float* mean,
+static void launch_ln_bwd(int maxc, int nt, int grid, const LnPartialSrc& ps, const void* dy, const void* x, const float* mean,
                           const float* rstd, const void* gamma, const void* dres, void* dx, float* dg,
                           float* db, float* cr, float* cx, int M, int E, hipStream_t s) {
     const T* dyp = (const T*)dy; const T* xp = (const T*)x; const T* gp = (const T*)gamma;
     const T* rp = (const T*)dres; T* dxp = (T*)dx;
-    if (maxc == 1) ln_bwd_kernel<T, 1><<<grid, nt, 0, s>>>(dyp, xp, mean, rstd, gp, rp, dxp, dg, db, cr, cx, M, E);
-    else if (maxc == 2) ln_bwd_kernel<T, 2><<<grid, nt, 0, s>>>(dyp, xp, mean, rstd, gp, rp, dxp, dg, db, cr, cx, M, E);
-    else ln_bwd_kernel<T, 4><<<grid, nt, 0, s>>>(dyp, xp, mean, rstd, gp, rp, dxp, dg, db, cr, cx, M, E);
+    if (maxc == 1) ln_bwd_kernel<T, 1><<<grid, nt, 0, s>>>(ps, dyp, xp, mean, rstd, gp, rp, dxp, dg, db, cr, cx, M, E);
+    else if (maxc == 2) ln_bwd_kernel<T, 2><<<grid, nt, 0, s>>>(ps, dyp, xp, mean, rstd, gp, rp, dxp, dg, db, cr, cx, M, E);
+    else ln_bwd_kernel<T, 4><<<grid, nt, 0, s>>>(ps, dyp, xp, mean, rstd, gp, rp, dxp, dg, db, cr, cx, M, E);
 }
 
 static int check_launch(const char* what) {
@@ -268,8 +313,8 @@ static int check_launch(const char* what) {
 
 }  // namespace tp
 
-extern "C" int tp_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
-                                float* rstd, int M, int E, float eps, int dtype, void* stream) {
+static int ln_fwd_impl(const tp::LnPartialSrc& ps, const void* x, const void* gamma, const void* beta, void* y,
+                       float* mean, float* rstd, int M, int E, float eps, int dtype, void* stream) {
     using namespace tp;
     if (!x || !gamma || !beta || !y || !mean || !rstd) { set_error("tp_layernorm_fwd: null pointer"); return TP_ERR_ARG; }
     if (M <= 0) { set_error("tp_layernorm_fwd: M=%d", M); return TP_ERR_ARG; }
@@ -280,17 +325,39 @@ extern "C" int tp_layernorm_fwd(const void* x, const void* gamma, const void* be
     if (rc != TP_OK) return rc;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     switch (dtype) {
-    case TP_F32: launch_ln_fwd<float>(maxc, nt, x, gamma, beta, y, mean, rstd, M, E, eps, s); break;
-    case TP_F16: launch_ln_fwd<f16>(maxc, nt, x, gamma, beta, y, mean, rstd, M, E, eps, s); break;
-    default: launch_ln_fwd<bf16>(maxc, nt, x, gamma, beta, y, mean, rstd, M, E, eps, s); break;
+    case TP_F32: launch_ln_fwd<float>(maxc, nt, ps, x, gamma, beta, y, mean, rstd, M, E, eps, s); break;
+    case TP_F16: launch_ln_fwd<f16>(maxc, nt, ps, x, gamma, beta, y, mean, rstd, M, E, eps, s); break;
+    default: launch_ln_fwd<bf16>(maxc, nt, ps, x, gamma, beta, y, mean, rstd, M, E, eps, s); break;
     }
     return check_launch("tp_layernorm_fwd");
 }
 
-extern "C" int tp_layernorm_bwd(const void* dy, const void* x, const float* mean, const float* rstd,
-                                const void* gamma, const void* dres, void* dx, float* dgamma_acc,
-                                float* dbeta_acc, float* colsum_dres_acc, float* colsum_dx_acc, int M, int E,
-                                int dtype, void* stream) {
+extern "C" int tp_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
+                                float* rstd, int M, int E, float eps, int dtype, void* stream) {
+    tp::LnPartialSrc ps = {nullptr, 0, 0, nullptr, nullptr, nullptr};
+    return ln_fwd_impl(ps, x, gamma, beta, y, mean, rstd, M, E, eps, dtype, stream);
+}
+
+static int check_partials(const char* who, const float* partials, int nsplit, const void* out16) {
+    if (!partials || nsplit < 1 || !out16) { tp::set_error("%s: partials, nsplit >= 1 and the output tensor are required", who); return TP_ERR_ARG; }
+    if (((uintptr_t)partials | (uintptr_t)out16) & 15) { tp::set_error("%s: pointers must be 16-byte aligned", who); return TP_ERR_ARG; }
+    return TP_OK;
+}
+
+extern "C" int tp_layernorm_fwd_partials(const float* partials, int nsplit, const void* bias, const void* residual,
+                                         void* x_out, const void* gamma, const void* beta, void* y, float* mean,
+                                         float* rstd, int M, int E, float eps, int dtype, void* stream) {
+    int rc = check_partials("tp_layernorm_fwd_partials", partials, nsplit, x_out);
+    if (rc != TP_OK) return rc;
+    if (((uintptr_t)bias | (uintptr_t)residual) & 15) { tp::set_error("tp_layernorm_fwd_partials: pointers must be 16-byte aligned"); return TP_ERR_ARG; }
+    tp::LnPartialSrc ps = {partials, nsplit, (long)M * E, bias, residual, x_out};
+    return ln_fwd_impl(ps, x_out, gamma, beta, y, mean, rstd, M, E, eps, dtype, stream);
+}
+
+static int ln_bwd_impl(const tp::LnPartialSrc& ps, const void* dy, const void* x, const float* mean, const float* rstd,
+                       const void* gamma, const void* dres, void* dx, float* dgamma_acc,
+                       float* dbeta_acc, float* colsum_dres_acc, float* colsum_dx_acc, int M, int E,
+                       int dtype, void* stream) {
     using namespace tp;
     if (!dy || !x || !mean || !rstd || !gamma || !dx) { set_error("tp_layernorm_bwd: null pointer"); return TP_ERR_ARG; }
     if ((dgamma_acc == nullptr) != (dbeta_acc == nullptr)) { set_error("tp_layernorm_bwd: dgamma_acc and dbeta_acc must both be given or both be NULL"); return TP_ERR_ARG; }
@@ -305,11 +372,31 @@ extern "C" int tp_layernorm_bwd(const void* dy, const void* x, const float* mean
     int grid = (dgamma_acc || colsum_dres_acc || colsum_dx_acc) ? (M < 128 ? M : 128) : M;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     switch (dtype) {
-    case TP_F32: launch_ln_bwd<float>(maxc, nt, grid, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc, M, E, s); break;
-    case TP_F16: launch_ln_bwd<f16>(maxc, nt, grid, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc, M, E, s); break;
-    default: launch_ln_bwd<bf16>(maxc, nt, grid, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc, M, E, s); break;
+    case TP_F32: launch_ln_bwd<float>(maxc, nt, grid, ps, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc, M, E, s); break;
+    case TP_F16: launch_ln_bwd<f16>(maxc, nt, grid, ps, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc, M, E, s); break;
+    default: launch_ln_bwd<bf16>(maxc, nt, grid, ps, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc, M, E, s); break;
     }
     return check_launch("tp_layernorm_bwd");
+}
+
+extern "C" int tp_layernorm_bwd(const void* dy, const void* x, const float* mean, const float* rstd,
+                                const void* gamma, const void* dres, void* dx, float* dgamma_acc,
+                                float* dbeta_acc, float* colsum_dres_acc, float* colsum_dx_acc, int M, int E,
+                                int dtype, void* stream) {
+    tp::LnPartialSrc ps = {nullptr, 0, 0, nullptr, nullptr, nullptr};
+    return ln_bwd_impl(ps, dy, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc, colsum_dx_acc,
+                       M, E, dtype, stream);
+}
+
+extern "C" int tp_layernorm_bwd_partials(const float* partials, int nsplit, void* dy_out, const void* x,
+                                         const float* mean, const float* rstd, const void* gamma, const void* dres,
+                                         void* dx, float* dgamma_acc, float* dbeta_acc, float* colsum_dres_acc,
+                                         float* colsum_dx_acc, int M, int E, int dtype, void* stream) {
+    int rc = check_partials("tp_layernorm_bwd_partials", partials, nsplit, dy_out);
+    if (rc != TP_OK) return rc;
+    tp::LnPartialSrc ps = {partials, nsplit, (long)M * E, nullptr, nullptr, dy_out};
+    return ln_bwd_impl(ps, dy_out, x, mean, rstd, gamma, dres, dx, dgamma_acc, dbeta_acc, colsum_dres_acc,
+                       colsum_dx_acc, M, E, dtype, stream);
 }
 
 extern "C" int tp_ln_param_grads(const void* dy, const void* x, const float* mean, const float* rstd,

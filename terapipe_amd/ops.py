@@ -121,13 +121,35 @@ class Workspace:
         return buf
 
 
+class PendingReduce:
+    """What gemm(..., defer_reduce=True) returns when the plan splits k: the fp32 partial sums are in `ws`
+    and the tensor `out` is NOT written yet.  layernorm_fwd / layernorm_bwd accept it in place of their input
+    tensor and then also produce `out` (sum of the partials + bias + residual, rounded to out's dtype).  It
+    must be consumed before the next split-k GEMM of the same stream reuses the workspace."""
+    __slots__ = ("ws", "nsplit", "bias", "residual", "out")
+
+    def __init__(self, ws, nsplit, bias, residual, out):
+        self.ws, self.nsplit, self.bias, self.residual, self.out = ws, nsplit, bias, residual, out
+
+
 def layernorm_fwd(x2d, gamma, beta, eps=1e-5, out=None, mean=None, rstd=None):
+    """x2d: the input rows, or a PendingReduce (then x2d.out is written as well)."""
+    pend = x2d if isinstance(x2d, PendingReduce) else None
+    if pend is not None:
+        x2d = pend.out
     _require_cuda(x2d, gamma, beta)
     M, E = x2d.shape
     y = torch.empty_like(x2d) if out is None else out
     mean = torch.empty(M, dtype=torch.float32, device=x2d.device) if mean is None else mean
     rstd = torch.empty(M, dtype=torch.float32, device=x2d.device) if rstd is None else rstd
     lib = _lib.load()
+    if pend is not None:
+        a = (_p(pend.ws), pend.nsplit, _p(pend.bias), _p(pend.residual), _p(x2d), _p(gamma), _p(beta), _p(y), _p(mean),
+             _p(rstd), M, E, eps, tp_dtype(x2d.dtype))
+        with _timed("layernorm_fwd", (M, E)):
+            _lib.check(lib.tp_layernorm_fwd_partials(*a, _stream()), "tp_layernorm_fwd_partials")
+        _record("layernorm_fwd", (M, E), lambda: lib.tp_layernorm_fwd_partials(*a, _stream()))
+        return y, mean, rstd
     with _timed("layernorm_fwd", (M, E)):
         _lib.check(lib.tp_layernorm_fwd(_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps,
                                         tp_dtype(x2d.dtype), _stream()), "tp_layernorm_fwd")
@@ -140,11 +162,21 @@ def layernorm_fwd(x2d, gamma, beta, eps=1e-5, out=None, mean=None, rstd=None):
 def layernorm_bwd(dy, x2d, mean, rstd, gamma, dres, dgamma_acc, dbeta_acc, colsum_dres_acc=None,
                   colsum_dx_acc=None, out=None):
     """dgamma_acc / dbeta_acc may be None: then only dx is computed (the parameter gradients are left
-    to ln_param_grads over all rows)."""
+    to ln_param_grads over all rows).  dy: the gradient rows, or a PendingReduce (then dy.out is written)."""
+    pend = dy if isinstance(dy, PendingReduce) else None
+    if pend is not None:
+        dy = pend.out
     _require_cuda(dy, x2d, gamma)
     M, E = x2d.shape
     dx = torch.empty_like(x2d) if out is None else out
     lib = _lib.load()
+    if pend is not None:
+        a = (_p(pend.ws), pend.nsplit, _p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx), _p(dgamma_acc),
+             _p(dbeta_acc), _p(colsum_dres_acc), _p(colsum_dx_acc), M, E, tp_dtype(x2d.dtype))
+        with _timed("layernorm_bwd", (M, E)):
+            _lib.check(lib.tp_layernorm_bwd_partials(*a, _stream()), "tp_layernorm_bwd_partials")
+        _record("layernorm_bwd", (M, E), lambda: lib.tp_layernorm_bwd_partials(*a, _stream()))
+        return dx
     with _timed("layernorm_bwd", (M, E)):
         _lib.check(lib.tp_layernorm_bwd(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx),
                                         _p(dgamma_acc), _p(dbeta_acc), _p(colsum_dres_acc), _p(colsum_dx_acc),
@@ -157,10 +189,12 @@ def layernorm_bwd(dy, x2d, mean, rstd, gamma, dres, dgamma_acc, dbeta_acc, colsu
 
 
 def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=None, aux=None, aux_out=None,
-         colsum_acc=None, qkv=None, tile_cfg=None, ksplit=None):
+         colsum_acc=None, qkv=None, tile_cfg=None, ksplit=None, defer_reduce=False):
     """Runs one GEMM.  A, B, C, residual, aux are 2-D row-major tensors (stride(1) == 1).
     qkv = dict(q, k_cache, v_cache, batch, heads, head_dim, cache_len, cache_rows, q_scale).
-    tile_cfg / ksplit force a tile configuration / k-split count (tuning and tests); default automatic."""
+    tile_cfg / ksplit force a tile configuration / k-split count (tuning and tests); default automatic.
+    defer_reduce (STORE / BIAS_RESIDUAL epilogues): if the plan splits k, C is left unwritten and a
+    PendingReduce is returned for the LayerNorm call that consumes C; otherwise C as usual."""
     _require_cuda(A, B, C)
     d = GemmDesc()
     d.op, d.dtype, d.epilogue = op, tp_dtype(A.dtype), epilogue
@@ -185,6 +219,11 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
     if tile_cfg is not None or ksplit is not None:
         d.reserved = ((tile_cfg + 1) if tile_cfg is not None else 0) | ((ksplit or 0) << 8)
     lib = _lib.load()
+    nsplit = 1
+    if defer_reduce:
+        nsplit = lib.tp_gemm_splits(ctypes.byref(d))
+        if nsplit > 1:
+            d.defer_reduce = 1
     need = lib.tp_gemm_workspace_bytes(ctypes.byref(d))
     ws = Workspace.get(need, A.device) if need else None
     with _timed("gemm", (op, M, N, K)):
@@ -192,6 +231,8 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
     if CallRecorder.active is not None:
         wsp, wsn = _p(ws), (ws.numel() if ws is not None else 0)
         _record("gemm", (op, M, N, K), lambda: lib.tp_gemm(ctypes.byref(d), wsp, wsn, _stream()))
+    if nsplit > 1:
+        return PendingReduce(ws, nsplit, bias, residual, C)
     return C
 
 

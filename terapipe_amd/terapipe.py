@@ -152,6 +152,7 @@ def _forward_body(runner, ws, act, bufs, states):
             r0, r1 = P * Bs, (P + T) * Bs
             sts, done = [], []
             st_i = lanes[i % len(lanes)] if lanes else main
+            pending = None
             with torch.cuda.stream(st_i):
                 for l in range(nl):
                     if lanes and prev_done is not None:
@@ -161,15 +162,18 @@ def _forward_body(runner, ws, act, bufs, states):
                     else:
                         qv, lv, rows = (pb["q"][l][r0:r1].view(Bs * H, T, E // H),
                                         pb["lse"][l][r0 * H:r1 * H].view(Bs * H, T), 0)
+                    # a k-split fc2 leaves its partial sums to the next layer's first LayerNorm (same stream,
+                    # nothing in between); the last layer finishes its own output
                     bf = core.Bufs(xn=pb["xn"][l][r0:r1], mean1=pb["mean1"][l][r0:r1], rstd1=pb["rstd1"][l][r0:r1],
                                    q=qv, o=pb["o"][l][r0:r1].view(T, Bs, E), lse=lv, q_bh_rows=rows,
-                                   stat_bh_rows=rows, h=pb["h"][l][r0:r1],
+                                   stat_bh_rows=rows, h=pb["h"][l][r0:r1], x_pending=pending, defer_out=l + 1 < nl,
                                    mean2=pb["mean2"][l][r0:r1], rstd2=pb["rstd2"][l][r0:r1], hn=pb["hn"][l][r0:r1],
                                    a=pb["a"][l][r0:r1], z=None if pb["z"][l] is None else pb["z"][l][r0:r1],
                                    out=pb["x"][l + 1][r0:r1])
                     _, st = core.layer_fwd(ws[l], pb["x"][l][r0:r1].view(T, Bs, E), H, cache[2 * l], cache[2 * l + 1],
                                            P, act[l], need_state=True, buf=bf)
                     sts.append(st)
+                    pending = bf.out_pending
                     if lanes:
                         ev = torch.cuda.Event()
                         ev.record(st_i)

@@ -42,6 +42,9 @@ int main(void) {
   printf("%zu %zu %zu %zu %zu %zu\n", sizeof(tp_gemm_desc), offsetof(tp_gemm_desc, colsum_acc),
          offsetof(tp_gemm_desc, q_scale), sizeof(tp_attn_desc), offsetof(tp_attn_desc, q_scale),
          offsetof(tp_attn_desc, colsum_dqkv_acc));
+  printf("%zu %zu %zu %zu %zu %zu\n", offsetof(tp_gemm_desc, defer_reduce), offsetof(tp_attn_desc, dq_only),
+         offsetof(tp_attn_desc, stat_bh_rows), sizeof(tp_attn_suffix_desc), offsetof(tp_attn_suffix_desc, q_all),
+         offsetof(tp_attn_suffix_desc, dqkv));
   return 0;
 }'''
     with tempfile.TemporaryDirectory() as d:
@@ -50,9 +53,10 @@ int main(void) {
         exe = os.path.join(d, "t")
         subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), c, "-o", exe])
         got = [int(v) for v in subprocess.check_output([exe]).split()]
-    G, A = _lib.GemmDesc, _lib.AttnDesc
+    G, A, S = _lib.GemmDesc, _lib.AttnDesc, _lib.AttnSuffixDesc
     assert got == [ctypes.sizeof(G), G.colsum_acc.offset, G.q_scale.offset, ctypes.sizeof(A), A.q_scale.offset,
-                   A.colsum_dqkv_acc.offset]
+                   A.colsum_dqkv_acc.offset, G.defer_reduce.offset, A.dq_only.offset, A.stat_bh_rows.offset,
+                   ctypes.sizeof(S), S.q_all.offset, S.dqkv.offset]
 
 
 def test_argument_errors_without_gpu(lib):

@@ -307,6 +307,49 @@ def test_attn_position_indexed_and_suffix_dkdv(dtype, B, H, Dh, L, slices):
     assert_close(dv, v64.grad, dtype, "dv over all later queries")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("M,E,K,ks", [(64, 256, 1024, 2), (37, 512, 4096, 4), (256, 2048, 8192, 2), (5, 64, 512, 1)])
+def test_layernorm_consumes_deferred_split_k(dtype, M, E, K, ks):
+    """A k-split GEMM with defer_reduce leaves fp32 partial sums; the LayerNorm forward / backward that
+    consumes the GEMM's result sums them (+ bias + residual), writes the result tensor and normalises it.
+    Bit-identical to GEMM (own reduce) followed by the plain LayerNorm call; without a split (ks = 1) the
+    GEMM completes normally and returns the tensor."""
+    ops = _ops()
+    from terapipe_amd import _lib as Lb
+    g = torch.Generator().manual_seed(M + E)
+    A, W = _rnd((M, K), dtype, g).to(DEV), _rnd((E, K), dtype, g, K ** -0.5).to(DEV)
+    b, r = _rnd((E,), dtype, g, 0.3).to(DEV), _rnd((M, E), dtype, g).to(DEV)
+    gm, bt = (_rnd((E,), dtype, g, 0.2) + 1).to(DEV), _rnd((E,), dtype, g, 0.2).to(DEV)
+    force = dict(ksplit=ks) if dtype != torch.float32 else {}
+    C1 = torch.empty(M, E, dtype=dtype, device=DEV)
+    ops.gemm(Lb.TP_GEMM_NT, A, W, M, E, K, C=C1, epilogue=Lb.TP_EPI_BIAS_RESIDUAL, bias=b, residual=r, **force)
+    y1, m1, s1 = ops.layernorm_fwd(C1, gm, bt)
+    C2 = torch.full((M, E), 9.0, dtype=dtype, device=DEV)
+    res = ops.gemm(Lb.TP_GEMM_NT, A, W, M, E, K, C=C2, epilogue=Lb.TP_EPI_BIAS_RESIDUAL, bias=b, residual=r,
+                   defer_reduce=True, **force)
+    if dtype != torch.float32 and ks > 1:
+        assert isinstance(res, ops.PendingReduce) and res.nsplit == ks
+        assert (C2 == 9).all(), "the deferred GEMM must not write its result tensor"
+    y2, m2, s2 = ops.layernorm_fwd(res, gm, bt)
+    assert torch.equal(C1, C2) and torch.equal(y1, y2) and torch.equal(m1, m2) and torch.equal(s1, s2)
+    # backward: dy = A W^T as the (deferred) gradient GEMM, x = r
+    D1 = torch.empty(M, E, dtype=dtype, device=DEV)
+    ops.gemm(Lb.TP_GEMM_NT, A, W, M, E, K, C=D1, **force)
+    xm, xs = ops.layernorm_fwd(r, gm, bt)[1:]
+    acc1 = [torch.zeros(E, dtype=torch.float32, device=DEV) for _ in range(4)]
+    dx1 = ops.layernorm_bwd(D1, r, xm, xs, gm, C1, *acc1)
+    D2 = torch.full((M, E), 9.0, dtype=dtype, device=DEV)
+    res = ops.gemm(Lb.TP_GEMM_NT, A, W, M, E, K, C=D2, defer_reduce=True, **force)
+    acc2 = [torch.zeros(E, dtype=torch.float32, device=DEV) for _ in range(4)]
+    dx2 = ops.layernorm_bwd(res, r, xm, xs, gm, C1, *acc2)
+    assert torch.equal(D1, D2) and torch.equal(dx1, dx2)
+    for a1, a2 in zip(acc1, acc2):
+        assert_close(a2, a1, torch.float32, "accumulators", 100)     # atomics: order differs
+    dx3 = ops.layernorm_bwd(ops.gemm(Lb.TP_GEMM_NT, A, W, M, E, K, C=D2, defer_reduce=True, **force), r, xm, xs, gm,
+                            None, None, None)
+    assert torch.equal(dx3, ops.layernorm_bwd(D1, r, xm, xs, gm, None, None, None))
+
+
 def test_error_paths():
     """Bad arguments come back as status codes with a message; nothing is launched."""
     import ctypes
