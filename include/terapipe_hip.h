@@ -207,6 +207,25 @@ typedef struct tp_attn_suffix_desc {
 int tp_attn_suffix_dkdv(const tp_attn_suffix_desc* d, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * The two ends of the layer stack in the reference's end-to-end configuration (token ids in, next-token
+ * cross-entropy out), at tensor-parallel size 1.
+ */
+/* out[m, :] = weight[ids[m], :]   (F.embedding inside VocabParallelEmbedding.forward, mpu/layers.py:126-141;
+ * ids outside [0, V) give a zero row, as the reference's masked rows do). */
+int tp_embedding_fwd(const int64_t* ids, const void* weight, void* out, int M, int E, int V, int dtype, void* stream);
+/* dweight_acc[ids[m], :] += dout[m, :]   (fp32 accumulators; autograd's embedding backward) */
+int tp_embedding_bwd(const int64_t* ids, const void* dout, float* dweight_acc, int M, int E, int V, int dtype, void* stream);
+/* _VocabParallelCrossEntropy (mpu/cross_entropy.py:25-104) forward and backward in one pass over logits
+ * [M, ld] whose first V columns are the vocabulary (columns [V, Vpad) are alignment padding of the LM-head
+ * GEMM): loss[m] = logsumexp(logits[m, :V]) - logits[m, target[m]], and logits is overwritten IN PLACE with
+ * its gradient (softmax - onehot(target)) * grad_scale (padding columns 0), the way the reference overwrites
+ * its input with the softmax (:65-74) and returns it scaled as grad_input (:79-99). */
+int tp_cross_entropy(void* logits, int64_t ld, const int64_t* target, float* loss, int M, int V, int Vpad,
+                     float grad_scale, int dtype, void* stream);
+/* x[m, :N] *= scale[m] in place: the per-token grad_output factor of the cross-entropy backward (:97) */
+int tp_scale_rows(void* x, int64_t ld, const float* scale, int M, int N, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * Small helpers around the kernels above.
  */
 /* dst[n] (dtype) = (accumulate ? dst[n] : 0) + src[n] (fp32): folds the fp32 accumulators of the

@@ -36,7 +36,7 @@ __all__ = [
     "assign_cache", "attention_core", "attention_forward", "layer_forward", "stack_forward",
     "create_cache", "init_layer_params", "init_stack_params", "uniform_slice",
     "grid_slice_batch_and_sequence", "terapipe_forward_backward", "unsliced_forward_backward",
-    "gelu_erf", "LAYER_PARAM_NAMES",
+    "gelu_erf", "LAYER_PARAM_NAMES", "embedding", "vocab_cross_entropy",
 ]
 
 # transformer_models.py:16 -- fp16 lowest, used as the additive mask value.
@@ -226,6 +226,28 @@ def init_layer_params(E: int, Fdim: int, std: float = 0.02, dtype=torch.float32,
 def init_stack_params(n_layers, E, Fdim, std=0.02, dtype=torch.float32, seed=0):
     g = torch.Generator().manual_seed(seed)
     return [init_layer_params(E, Fdim, std, dtype, g) for _ in range(n_layers)]
+
+
+def embedding(ids, weight):
+    """VocabParallelEmbedding.forward at tensor-parallel size 1 (mpu/layers.py:126-141): ids outside the
+    partition's vocabulary range [0, V) are looked up as row 0 and their output rows zeroed; the all-reduce
+    is the identity.  Pinned by F.embedding and a Python loop (tests/test_oracle_pins.py)."""
+    V = weight.shape[0]
+    mask = (ids < 0) | (ids >= V)
+    masked = ids.clone()
+    masked[mask] = 0
+    out = weight[masked]                                                             # F.embedding, :134-137
+    out = torch.where(mask.unsqueeze(-1), torch.zeros((), dtype=out.dtype), out)     # :139
+    return out
+
+
+def vocab_cross_entropy(logits, target):
+    """_VocabParallelCrossEntropy.forward at tensor-parallel size 1 (mpu/cross_entropy.py:25-77), without
+    the in-place overwrites: per-token loss = log(sum exp(logits - max)) - (logits - max)[target].
+    Pinned by F.cross_entropy(reduction='none') and a Python loop."""
+    z = logits - logits.max(dim=-1, keepdim=True)[0]                                 # :28-33
+    predicted = z.gather(-1, target.unsqueeze(-1)).squeeze(-1)                       # :48-57
+    return torch.log(torch.exp(z).sum(dim=-1)) - predicted                           # :63-71
 
 
 def uniform_slice(length: int, n_slices: int) -> List[int]:

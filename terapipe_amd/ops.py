@@ -353,3 +353,44 @@ def zero_(t):
     lib = _lib.load()
     _lib.check(lib.tp_zero_words(_p(t), nbytes // 4, _stream()), "tp_zero_words")
     return t
+
+
+def embedding_fwd(ids, weight, out=None):
+    """ids int64 [M] -> out [M, E] = weight[ids]."""
+    _require_cuda(ids, weight)
+    M, (V, E) = ids.numel(), weight.shape
+    out = torch.empty(M, E, dtype=weight.dtype, device=weight.device) if out is None else out
+    lib = _lib.load()
+    _lib.check(lib.tp_embedding_fwd(_p(ids), _p(weight), _p(out), M, E, V, tp_dtype(weight.dtype), _stream()),
+               "tp_embedding_fwd")
+    return out
+
+
+def embedding_bwd(ids, dout, dweight_acc):
+    """dweight_acc fp32 [V, E] += scatter of dout [M, E] by ids."""
+    _require_cuda(ids, dout, dweight_acc)
+    V, E = dweight_acc.shape
+    lib = _lib.load()
+    _lib.check(lib.tp_embedding_bwd(_p(ids), _p(dout), _p(dweight_acc), ids.numel(), E, V, tp_dtype(dout.dtype),
+                                    _stream()), "tp_embedding_bwd")
+    return dweight_acc
+
+
+def cross_entropy_(logits, target, V, grad_scale=1.0):
+    """logits [M, Vpad] (row-major, first V columns valid) is overwritten with its gradient
+    (softmax - onehot) * grad_scale; returns the per-row loss (fp32 [M])."""
+    _require_cuda(logits, target)
+    M, Vpad = logits.shape
+    loss = torch.empty(M, dtype=torch.float32, device=logits.device)
+    lib = _lib.load()
+    _lib.check(lib.tp_cross_entropy(_p(logits), logits.stride(0), _p(target), _p(loss), M, V, Vpad, float(grad_scale),
+                                    tp_dtype(logits.dtype), _stream()), "tp_cross_entropy")
+    return loss
+
+
+def scale_rows_(x2d, scale_f32):
+    _require_cuda(x2d, scale_f32)
+    lib = _lib.load()
+    _lib.check(lib.tp_scale_rows(_p(x2d), x2d.stride(0), _p(scale_f32), x2d.shape[0], x2d.shape[1], tp_dtype(x2d.dtype),
+                                 _stream()), "tp_scale_rows")
+    return x2d

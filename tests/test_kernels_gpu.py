@@ -350,6 +350,40 @@ def test_layernorm_consumes_deferred_split_k(dtype, M, E, K, ks):
     assert torch.equal(dx3, ops.layernorm_bwd(D1, r, xm, xs, gm, None, None, None))
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("M,E,V", [(24, 64, 50257), (7, 256, 1003), (130, 128, 512)])
+def test_embedding_lm_head_cross_entropy(dtype, M, E, V):
+    """Token ids -> embedding -> (tied) LM head -> per-token cross-entropy -> mean, forward and backward,
+    against the oracle's restatements of mpu.VocabParallelEmbedding and mpu.vocab_parallel_cross_entropy."""
+    import terapipe_amd as ta
+    g = torch.Generator().manual_seed(V + M)
+    W = _rnd((V, E), dtype, g, 0.05)
+    ids = torch.randint(0, V, (M,), generator=g)
+    tgt = torch.randint(0, V, (M,), generator=g)
+    ids[0], tgt[-1] = V - 1, V - 1                        # last vocabulary row on both ends
+    ids[1] = ids[2]                                       # a repeated id (gradient rows add up)
+    emb = ta.VocabParallelEmbedding(V, E, device=DEV, dtype=dtype)
+    with torch.no_grad():
+        emb.weight.copy_(W.to(DEV))
+    x = emb(ids.to(DEV))
+    logits = ta.lm_head_logits(x.view(M, E), emb.weight)
+    assert logits.shape == (M, (V + 7) // 8 * 8)
+    loss = ta.vocab_parallel_cross_entropy(logits, tgt.to(DEV), vocab_size=V)
+    scale = _rnd((M,), torch.float32, g).abs() + 0.5
+    (loss * scale.to(DEV)).sum().backward()
+    W64 = W.double().requires_grad_(True)
+    x64 = oracle.embedding(ids, W64)
+    loss64 = oracle.vocab_cross_entropy(x64 @ W64.t(), tgt)
+    (loss64 * scale.double()).sum().backward()
+    assert_close(x, x64, dtype, "embedding")
+    assert_close(loss, loss64, torch.float32 if dtype == torch.float32 else dtype, "per-token loss",
+                 10 if dtype == torch.float32 else 1)
+    assert_close(emb.weight.grad, W64.grad, dtype, "d weight (embedding + LM head)", 3)
+    # out-of-range ids give zero rows
+    bad = ids.clone(); bad[3] = V + 5
+    assert (emb(bad.to(DEV))[3] == 0).all()
+
+
 def test_error_paths():
     """Bad arguments come back as status codes with a message; nothing is launched."""
     import ctypes

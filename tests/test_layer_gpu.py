@@ -302,6 +302,52 @@ def test_terapipe_c1_tokens_and_cross_entropy():
     _check_param_grads(_param_grads(layers), [{k: v.grad for k, v in p.items()} for p in leaf], torch.float32, "C1 CE")
 
 
+def test_terapipe_c1_end_to_end_native_embedding_and_loss():
+    """BASELINE config 1 end to end with nothing but the HIP path between the token ids and the loss:
+    VocabParallelEmbedding -> sliced stack -> tied LM head -> vocab_parallel_cross_entropy -> mean, against
+    the oracle (embedding, stack, cross-entropy restatements) in fp32 at 1e-5."""
+    ta = _mods()
+    n_layers, E, H, Fd, L, B, V = 4, 256, 4, 1024, 128, 2, 50257
+    ss = oracle.uniform_slice(L, 8)
+    ps = make_params(n_layers, E, Fd, torch.float32, seed=0, rand_small=False)
+    g = torch.Generator().manual_seed(321)
+    emb = torch.randn(V, E, generator=g) * 0.02
+    ids = torch.randint(0, V, (L, B), generator=g)
+    tgt = torch.randint(0, V, (L, B), generator=g)
+    # oracle: forward without grad for y, the loss gradient dy, then the sliced backward, then the embedding
+    emb_o = emb.clone().requires_grad_(True)
+    x_o = oracle.embedding(ids, emb_o)
+    x_leaf = x_o.detach().clone()
+    leaf = [{k: v.clone().requires_grad_(True) for k, v in p.items()} for p in ps]
+    with torch.no_grad():
+        cache = oracle.create_cache(n_layers, B, H, L, E // H)
+        outs, cl = [], 0
+        for sl in ss:
+            yi, cache = oracle.stack_forward(leaf, x_leaf[cl:cl + sl], H, cache, cl)
+            outs.append(yi)
+            cl += sl
+        y_full = torch.cat(outs, 0)
+    y_req = y_full.clone().requires_grad_(True)
+    loss_o = oracle.vocab_cross_entropy(y_req.view(L * B, E) @ emb_o.t(), tgt.view(-1)).mean()
+    loss_o.backward()
+    yo, dxo, _ = oracle.terapipe_forward_backward(leaf, x_leaf, y_req.grad, H, [B], ss)
+    x_o.backward(dxo)
+
+    layers = _build_layers(ta, n_layers, E, Fd, H, torch.float32, ps)
+    embd = ta.VocabParallelEmbedding(V, E, device=DEV, dtype=torch.float32)
+    with torch.no_grad():
+        embd.weight.copy_(emb.to(DEV))
+    runner = ta.TeraPipe(layers, B, L, [B], ss)
+    y = runner(embd(ids.to(DEV)))
+    logits = ta.lm_head_logits(y.reshape(L * B, E), embd.weight)
+    loss = ta.vocab_parallel_cross_entropy(logits, tgt.to(DEV).view(-1), vocab_size=V).mean()
+    loss.backward()
+    assert abs(loss.item() - loss_o.item()) <= 1e-5 * abs(loss_o.item())
+    assert_close(y, yo, torch.float32, "y")
+    assert_close(embd.weight.grad, emb_o.grad, torch.float32, "d embedding (lookup + tied head)", 2)
+    _check_param_grads(_param_grads(layers), [{k: v.grad for k, v in p.items()} for p in leaf], torch.float32, "C1 native")
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
 @pytest.mark.parametrize("case", ["uniform", "nonuniform", "fine", "batch_sliced"])
 def test_terapipe_16bit_reduced_shapes(dtype, case):

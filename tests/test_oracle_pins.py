@@ -179,6 +179,31 @@ def test_gelu_erf_is_library_gelu():
     assert torch.allclose(oracle.gelu_erf(x), F.gelu(x), atol=1e-12)
 
 
+def test_embedding_and_vocab_cross_entropy_match_library_and_loops():
+    g = torch.Generator().manual_seed(4)
+    V, E = 11, 6
+    W = _rnd(V, E, seed=5)
+    ids = torch.randint(0, V, (4, 3), generator=g)
+    assert torch.equal(oracle.embedding(ids, W), F.embedding(ids, W))
+    bad = ids.clone(); bad[1, 2] = V + 3; bad[0, 0] = -1          # outside the vocabulary: zero rows
+    e = oracle.embedding(bad, W)
+    for t in range(4):
+        for b in range(3):
+            ref = W[bad[t, b]] if 0 <= bad[t, b] < V else torch.zeros(E, dtype=W.dtype)
+            assert torch.equal(e[t, b], ref)
+    z, tgt = _rnd(4, 3, V, seed=6) * 3, torch.randint(0, V, (4, 3), generator=g)
+    loss = oracle.vocab_cross_entropy(z, tgt)
+    assert torch.allclose(loss, F.cross_entropy(z.view(-1, V), tgt.view(-1), reduction="none").view(4, 3), atol=1e-12)
+    for t in range(4):
+        for b in range(3):
+            s = sum(math.exp(z[t, b, v].item()) for v in range(V))
+            assert abs(loss[t, b].item() - (math.log(s) - z[t, b, tgt[t, b]].item())) < 1e-10
+    # gradient of the summed loss: softmax - onehot (what the reference returns as grad_input, :79-99)
+    zr = z.clone().requires_grad_(True)
+    oracle.vocab_cross_entropy(zr, tgt).sum().backward()
+    assert torch.allclose(zr.grad, torch.softmax(z, -1) - F.one_hot(tgt, V).to(z.dtype), atol=1e-12)
+
+
 def test_slicers():
     assert oracle.uniform_slice(10, 4) == [3, 3, 2, 2]          # first len % n slices get one more
     assert oracle.uniform_slice(128, 8) == [16] * 8
