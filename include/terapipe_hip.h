@@ -226,6 +226,19 @@ int tp_cross_entropy(void* logits, int64_t ld, const int64_t* target, float* los
 int tp_scale_rows(void* x, int64_t ld, const float* scale, int M, int N, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * Slice planner (host code, no GPU work): `planning` of latency_model.py:97-152.
+ * latency_grid[bs][step][ctx], bs <= total_batch_size, step, ctx <= n_steps (row-major doubles): latency of
+ * one slice of `step` sequence steps after `ctx` steps of context at batch size bs.  Minimises the sum of
+ * slice latencies + (pipeline_len - 1) * the largest one with every slice latency <= max_latency.
+ * Output: *final_time (infinity and *n_groups = 0 when no plan is feasible), the batch groups in the order the
+ * reference emits them, and for each group its slices in steps, LAST slice of the sequence first (as the
+ * reference's list before analysis_model reverses it, :172-173).  group_batch, group_nslices hold up to
+ * total_batch_size entries, slice_steps up to total_batch_size * n_steps. */
+int tp_plan_slices(const double* latency_grid, int total_batch_size, int n_steps, int pipeline_len,
+                   double max_latency, double* final_time, int* n_groups, int* group_batch, int* group_nslices,
+                   int* slice_steps);
+
+/* ------------------------------------------------------------------------------------------------
  * Small helpers around the kernels above.
  */
 /* dst[n] (dtype) = (accumulate ? dst[n] : 0) + src[n] (fp32): folds the fp32 accumulators of the

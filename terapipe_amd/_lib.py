@@ -94,6 +94,7 @@ SYMBOLS = {
     "tp_embedding_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "tp_cross_entropy": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "tp_scale_rows": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "tp_plan_slices": (c_int, [c_void_p, c_int, c_int, c_int, ctypes.c_double] + [c_void_p] * 5),
     "tp_accum_cast": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "tp_colsum_acc": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_void_p]),
     "tp_zero_words": (c_int, [c_void_p, c_int64, c_void_p]),

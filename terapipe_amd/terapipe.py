@@ -153,6 +153,8 @@ def _forward_body(runner, ws, act, bufs, states):
             sts, done = [], []
             st_i = lanes[i % len(lanes)] if lanes else main
             pending = None
+            if runner.slice_timing is not None:
+                runner.slice_timing["fwd"].append(_timing_event(main))
             with torch.cuda.stream(st_i):
                 for l in range(nl):
                     if lanes and prev_done is not None:
@@ -180,6 +182,8 @@ def _forward_body(runner, ws, act, bufs, states):
                         done.append(ev)
             prev_done = done
             states[b, i] = sts
+            if runner.slice_timing is not None:
+                runner.slice_timing["fwd"].append(_timing_event(main))
             P += T                                                               # terapipe.py:264
     for st in lanes:
         main.wait_stream(st)
@@ -210,6 +214,8 @@ def _backward_body(runner, ws, act, bufs, states):
             P -= T
             r0, r1 = P * Bs, (P + T) * Bs
             last = i == ns - 1
+            if runner.slice_timing is not None:
+                runner.slice_timing["bwd"].append(_timing_event(main))
             if bufs.position_indexed:
                 # slice lanes: layer l of slice i waits for layer l of slice i+1 (whose dO and delta the
                 # one-pass dK/dV reads, and through it for every later slice)
@@ -230,6 +236,8 @@ def _backward_body(runner, ws, act, bufs, states):
                             done[l] = torch.cuda.Event()
                             done[l].record(st_i)
                 later_done = done
+                if runner.slice_timing is not None:
+                    runner.slice_timing["bwd"].append(_timing_event(main))
                 continue
             for l in reversed(range(nl)):
                 bf = core.Bufs(dz1=pb["dz1"][l][r0:r1], dhn=pb["dhn"][l][r0:r1], dh=pb["dh"][l][r0:r1],
@@ -240,8 +248,12 @@ def _backward_body(runner, ws, act, bufs, states):
                 core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), H,
                                gc[2 * l], gc[2 * l + 1], None, False, None, accumulate_prefix=not last,
                                has_incoming=not last, zero_slice_rows=False, activation=act[l], buf=bf)
+            if runner.slice_timing is not None:
+                runner.slice_timing["bwd"].append(_timing_event(main))
     for st in lanes:
         main.wait_stream(st)
+    if runner.slice_timing is not None:
+        runner.slice_timing["param"].append(_timing_event(main))
     # parameter gradients over all tokens: dW = dY_all^T X_all (one GEMM per weight and batch slice),
     # bias gradients = column sums of dY_all, LayerNorm gradients from (dy, x, mean, rstd) of all rows
     for l in range(nl):
@@ -265,6 +277,14 @@ def _backward_body(runner, ws, act, bufs, states):
                                sv["fc_ln.bias"])
         for n in core.SMALL_PARAMS:
             ops.accum_cast(bufs.sgrads[l][n], sv[n], False)
+    if runner.slice_timing is not None:
+        runner.slice_timing["param"].append(_timing_event(main))
+
+
+def _timing_event(stream):
+    ev = torch.cuda.Event(enable_timing=True)
+    ev.record(stream)
+    return ev
 
 
 def _capture(fn):
@@ -385,6 +405,9 @@ class TeraPipe(nn.Module):
         self.use_hip_graph = use_hip_graph
         self.suffix_dkdv = suffix_dkdv
         self.slice_streams = int(slice_streams)
+        # set to {"fwd": [], "bwd": [], "param": []} to have the (eager, single-stream) step bracket every slice's
+        # forward and backward and the parameter-gradient tail with timing events (latency_model.py uses it)
+        self.slice_timing = None
         self._sbufs = None
         self.last_caches = None
         self.keep_states = False   # debugging / tests: keep the per-slice saved activations of the last forward

@@ -528,3 +528,21 @@ def test_slice_streams_match_single_stream(dtype):
             assert torch.equal(dx2, dx1), "dx with %d lanes" % n
             for a, b in zip([p.grad for p in layers.parameters()], g1):
                 assert_close(a, b, dtype, "parameter gradient with %d lanes" % n, 1.0)
+
+
+def test_latency_measurement_feeds_the_planner():
+    """measure_layer_latency -> fit_latency_grid -> best_plan on a small stack: every requested point is
+    measured, latencies are positive, and the plan covers the sequence (at this size the times are launch
+    bound, so nothing is asserted about their order)."""
+    ta = _mods()
+    from terapipe_amd import latency_model as lm
+    n_layers, E, H, Fd, L = 2, 512, 4, 2048, 256
+    ps = make_params(n_layers, E, Fd, torch.float16, seed=1)
+    layers = _build_layers(ta, n_layers, E, Fd, H, torch.float16, ps)
+    samples = lm.measure_layer_latency(layers, 1, L, [32, 64, 128, 256], reps=2)
+    assert set(samples) == ({(1, 32, c) for c in range(0, L, 32)} | {(1, 64, c) for c in range(0, L, 64)} |
+                            {(1, 128, 0), (1, 128, 128), (1, 256, 0)})
+    assert all(t > 0 and t == t for t in samples.values())
+    grid = lm.fit_latency_grid(samples, 1, L, layers_per_stage=n_layers)
+    scheme, latency = lm.best_plan(grid, 1, L, pipelinelen=4)
+    assert scheme is not None and sum(scheme[0][1]) == L and latency >= 0 and latency == latency
