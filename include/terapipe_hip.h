@@ -239,6 +239,41 @@ int tp_plan_slices(const double* latency_grid, int total_batch_size, int n_steps
                    int* slice_steps);
 
 /* ------------------------------------------------------------------------------------------------
+ * Mixed-precision optimizer step: `update_weights` of test_transformer_terapipe.py:245-266 in one launch
+ * (gradient copy to fp32 with 1/loss-scale :248-252, FusedAdam on the fp32 master weights :255 as constructed
+ * at :92-97, zero_grad :256-260, master -> 16-bit model copy :262-266).  The update follows apex's
+ * multi_tensor_adam (adam_w_mode 1 = decoupled weight decay, 0 = L2), which with weight_decay 0 is
+ * torch.optim.Adam.  All state is fp32; every pointer is 16-byte aligned.
+ */
+typedef struct tp_adam_tensor {
+    void* master;       /* fp32 [n] weights, updated in place */
+    void* grad;         /* [n] gradient of desc.grad_dtype; zeroed when desc.zero_grad */
+    void* exp_avg;      /* fp32 [n] first moment, updated in place */
+    void* exp_avg_sq;   /* fp32 [n] second moment, updated in place */
+    void* model;        /* [n] weights of desc.model_dtype, overwritten with the new master; unused when -1 */
+    int64_t n;
+} tp_adam_tensor;
+
+typedef struct tp_adam_desc {
+    int32_t n_tensors;          /* <= 65535 */
+    int32_t grad_dtype;         /* tp_dtype of every gradient in the table */
+    int32_t model_dtype;        /* TP_F16 / TP_BF16, or -1: no 16-bit copy is written */
+    int32_t adam_w_mode;
+    int32_t bias_correction;
+    int32_t zero_grad;
+    int32_t step;               /* 1 for the first update */
+    int32_t blocks_per_tensor;  /* 0 = default (256) */
+    double lr, beta1, beta2, eps, weight_decay;   /* doubles: 1 - beta and the bias corrections are formed in
+                                                     double and rounded once, as torch.optim does */
+    double grad_scale;          /* gradients are multiplied by this first (1 / loss scale) */
+    const tp_adam_tensor* tensors;  /* DEVICE memory, n_tensors records */
+} tp_adam_desc;
+
+/* validates a HOST copy of the table (null pointers, alignment, lengths) before it is uploaded */
+int tp_adam_check_table(const tp_adam_tensor* host_table, int n_tensors, int model_dtype);
+int tp_adam_step(const tp_adam_desc* desc, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * Small helpers around the kernels above.
  */
 /* dst[n] (dtype) = (accumulate ? dst[n] : 0) + src[n] (fp32): folds the fp32 accumulators of the

@@ -15,3 +15,4 @@ from .transformer_models import (MODEL_CONFIGS, BATCH_CONFIGS, NEG_INF, ColumnPa
 
 __version__ = "0.1.0"
 from .vocab import VocabParallelEmbedding, lm_head_logits, vocab_parallel_cross_entropy  # noqa: F401
+from .optim import FusedAdam  # noqa: F401

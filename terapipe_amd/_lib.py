@@ -73,6 +73,23 @@ class AttnSuffixDesc(ctypes.Structure):
     ]
 
 
+class AdamTensor(ctypes.Structure):
+    """Mirror of ``tp_adam_tensor``."""
+    _fields_ = [("master", c_void_p), ("grad", c_void_p), ("exp_avg", c_void_p), ("exp_avg_sq", c_void_p),
+                ("model", c_void_p), ("n", c_int64)]
+
+
+class AdamDesc(ctypes.Structure):
+    """Mirror of ``tp_adam_desc``."""
+    _fields_ = [
+        ("n_tensors", c_int32), ("grad_dtype", c_int32), ("model_dtype", c_int32), ("adam_w_mode", c_int32),
+        ("bias_correction", c_int32), ("zero_grad", c_int32), ("step", c_int32), ("blocks_per_tensor", c_int32),
+        ("lr", ctypes.c_double), ("beta1", ctypes.c_double), ("beta2", ctypes.c_double), ("eps", ctypes.c_double),
+        ("weight_decay", ctypes.c_double), ("grad_scale", ctypes.c_double),
+        ("tensors", c_void_p),
+    ]
+
+
 # every symbol include/terapipe_hip.h declares: name -> (restype, argtypes)
 SYMBOLS = {
     "tp_version": (c_int, []),
@@ -95,6 +112,8 @@ SYMBOLS = {
     "tp_cross_entropy": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "tp_scale_rows": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_void_p]),
     "tp_plan_slices": (c_int, [c_void_p, c_int, c_int, c_int, ctypes.c_double] + [c_void_p] * 5),
+    "tp_adam_check_table": (c_int, [c_void_p, c_int, c_int]),
+    "tp_adam_step": (c_int, [ctypes.POINTER(AdamDesc), c_void_p]),
     "tp_accum_cast": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "tp_colsum_acc": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_void_p]),
     "tp_zero_words": (c_int, [c_void_p, c_int64, c_void_p]),

@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libterapipe_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["misc.hip", "layernorm.hip", "gemm.hip", "attention.hip", "vocab.hip", "planner.hip"]
+SOURCES = ["misc.hip", "layernorm.hip", "gemm.hip", "attention.hip", "vocab.hip", "planner.hip", "optimizer.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

@@ -45,6 +45,8 @@ int main(void) {
   printf("%zu %zu %zu %zu %zu %zu\n", offsetof(tp_gemm_desc, defer_reduce), offsetof(tp_attn_desc, dq_only),
          offsetof(tp_attn_desc, stat_bh_rows), sizeof(tp_attn_suffix_desc), offsetof(tp_attn_suffix_desc, q_all),
          offsetof(tp_attn_suffix_desc, dqkv));
+  printf("%zu %zu %zu %zu\n", sizeof(tp_adam_tensor), offsetof(tp_adam_tensor, n), sizeof(tp_adam_desc),
+         offsetof(tp_adam_desc, tensors));
   return 0;
 }'''
     with tempfile.TemporaryDirectory() as d:
@@ -56,7 +58,9 @@ int main(void) {
     G, A, S = _lib.GemmDesc, _lib.AttnDesc, _lib.AttnSuffixDesc
     assert got == [ctypes.sizeof(G), G.colsum_acc.offset, G.q_scale.offset, ctypes.sizeof(A), A.q_scale.offset,
                    A.colsum_dqkv_acc.offset, G.defer_reduce.offset, A.dq_only.offset, A.stat_bh_rows.offset,
-                   ctypes.sizeof(S), S.q_all.offset, S.dqkv.offset]
+                   ctypes.sizeof(S), S.q_all.offset, S.dqkv.offset,
+                   ctypes.sizeof(_lib.AdamTensor), _lib.AdamTensor.n.offset, ctypes.sizeof(_lib.AdamDesc),
+                   _lib.AdamDesc.tensors.offset]
 
 
 def test_argument_errors_without_gpu(lib):
@@ -123,3 +127,21 @@ def test_host_side_surface_mirrors_reference_names():
     assert (cfg.n_layers, cfg.embedding_dim, cfg.ffn_embedding_dim, cfg.attention_heads_dim) == (24, 2048, 8192, 128)
     with pytest.raises(AssertionError):
         ta.TeraPipe(None, 2, 16, [2], [8, 4])                 # slices must sum to the sequence length
+
+
+def test_adam_table_validation_without_gpu(lib):
+    from terapipe_amd import _lib
+    t = (_lib.AdamTensor * 2)()
+    for i in range(2):
+        t[i].master, t[i].grad, t[i].exp_avg, t[i].exp_avg_sq, t[i].model, t[i].n = 256, 512, 768, 1024, 1280, 100
+    assert lib.tp_adam_check_table(ctypes.cast(t, ctypes.c_void_p), 2, _lib.TP_F16) == 0
+    t[1].grad = 520                                                   # 8-byte aligned only
+    assert lib.tp_adam_check_table(ctypes.cast(t, ctypes.c_void_p), 2, _lib.TP_F16) == 2      # TP_ERR_UNSUPPORTED
+    assert b"tensor 1" in lib.tp_last_error()
+    t[1].grad, t[0].model = 512, None
+    assert lib.tp_adam_check_table(ctypes.cast(t, ctypes.c_void_p), 2, -1) == 0               # model unused
+    assert lib.tp_adam_check_table(ctypes.cast(t, ctypes.c_void_p), 2, _lib.TP_BF16) == 1
+    d = _lib.AdamDesc()
+    assert lib.tp_adam_step(ctypes.byref(d), None) == 1
+    d.n_tensors, d.tensors, d.model_dtype, d.step = 1, 256, -1, 0
+    assert lib.tp_adam_step(ctypes.byref(d), None) == 1 and b"step" in lib.tp_last_error()

@@ -204,6 +204,41 @@ def test_embedding_and_vocab_cross_entropy_match_library_and_loops():
     assert torch.allclose(zr.grad, torch.softmax(z, -1) - F.one_hot(tgt, V).to(z.dtype), atol=1e-12)
 
 
+@pytest.mark.parametrize("mode,wd", [("l2", 0.0), ("l2", 0.05), ("adamw", 0.05), ("adamw", 0.0)])
+def test_adam_step_matches_library_optimizers(mode, wd):
+    """torch.optim.Adam is the L2 form, torch.optim.AdamW the decoupled form apex's adam_w_mode selects; six
+    steps in float64 so that bias correction and both moments matter."""
+    from oracle import optimizer_oracle as opt
+    rng = np.random.default_rng(11)
+    p0 = rng.standard_normal(257)
+    hyper = dict(lr=3e-3, beta1=0.8, beta2=0.95, eps=1e-6, weight_decay=wd)
+    pt = torch.tensor(p0, dtype=torch.float64, requires_grad=True)
+    cls = torch.optim.Adam if mode == "l2" else torch.optim.AdamW
+    lib = cls([pt], lr=hyper["lr"], betas=(hyper["beta1"], hyper["beta2"]), eps=hyper["eps"], weight_decay=wd)
+    p, m, v = p0.copy(), np.zeros_like(p0), np.zeros_like(p0)
+    for step in range(1, 7):
+        g = rng.standard_normal(257) * (0.1 + step)
+        pt.grad = torch.tensor(g, dtype=torch.float64)
+        lib.step()
+        p, m, v = opt.adam_step(p, g, m, v, step, adam_w_mode=(mode == "adamw"), **hyper)
+        np.testing.assert_allclose(p, pt.detach().numpy(), rtol=1e-12, atol=1e-14)
+    st = lib.state[pt]
+    np.testing.assert_allclose(m, st["exp_avg"].numpy(), rtol=1e-12, atol=0)
+    np.testing.assert_allclose(v, st["exp_avg_sq"].numpy(), rtol=1e-12, atol=0)
+    # without bias correction the first step is lr * (1-b1) g / (sqrt((1-b2) g^2) + eps): closed form
+    g = np.array([2.0, -0.5])
+    p1, _, _ = opt.adam_step(np.zeros(2), g, np.zeros(2), np.zeros(2), 1, lr=1.0, beta1=0.9, beta2=0.99, eps=0.0,
+                             bias_correction=False)
+    np.testing.assert_allclose(p1, -np.sign(g) * 0.1 / math.sqrt(0.01), rtol=1e-12)
+    # loss-scale path: gradients 128 x larger with loss_scale 128 give the same update, and the model copy
+    # is the rounded master
+    ma, m2, v2, model = opt.update_weights(p0, 128.0 * g[0] * np.ones(257), np.zeros(257), np.zeros(257), 1, 128.0,
+                                           np.float16, lr=1e-2)
+    mb, _, _ = opt.adam_step(p0, g[0] * np.ones(257), np.zeros(257), np.zeros(257), 1, lr=1e-2)
+    np.testing.assert_array_equal(ma, mb)
+    np.testing.assert_array_equal(model, mb.astype(np.float32).astype(np.float16))
+
+
 def test_slicers():
     assert oracle.uniform_slice(10, 4) == [3, 3, 2, 2]          # first len % n slices get one more
     assert oracle.uniform_slice(128, 8) == [16] * 8
