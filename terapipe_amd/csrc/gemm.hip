@@ -499,6 +499,28 @@ static const TileCfg kCfgs[] = {
 };
 static constexpr int kNumCfgs = (int)(sizeof(kCfgs) / sizeof(kCfgs[0]));
 
+// Measured plans: for NT / NN the weight extents (N, K) match exactly and M (tokens of the slice) picks the
+// nearest measured M at or above it (at least half of it, so that a much shorter slice falls through to the
+// heuristics); TN (parameter gradients) matches all three extents.
+struct TunedPlan { int op, M, N, K, cfg, nsplit; };
+static const TunedPlan kTuned[] = {
+#include "gemm_tuned.inc"
+    {-1, 0, 0, 0, 0, 0},
+};
+
+static const TunedPlan* find_tuned(const tp_gemm_desc* d) {
+    const TunedPlan* best = nullptr;
+    for (const TunedPlan* t = kTuned; t->op >= 0; ++t) {
+        if (t->op != d->op || t->N != d->N || t->K != d->K) continue;
+        if (d->op == TP_GEMM_TN) {
+            if (t->M == d->M) return t;
+            continue;
+        }
+        if (t->M >= d->M && t->M <= 2 * d->M && (!best || t->M < best->M)) best = t;
+    }
+    return best;
+}
+
 struct GemmPlan {
     int cfg;
     int nsplit;
@@ -575,6 +597,7 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
             if (ns > maxs) ns = maxs;
         }
     }
+    if (const TunedPlan* t = find_tuned(d)) { cfg = t->cfg; ns = t->nsplit; }
     if (ns < 1) ns = 1;
     if (ns > 16) ns = 16;
     if (forced_cfg >= 0 && forced_cfg < kNumCfgs) cfg = forced_cfg;
