@@ -372,6 +372,45 @@ __device__ __forceinline__ void dma4(const void* gptr, unsigned lds_wave_base) {
                  :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)) : "memory");
 }
 
+// Tile loads for full tiles only: the lane's chunk is a loop-invariant 32-bit byte offset from a wave-uniform
+// tile origin that advances by a scalar step, so a tile costs one VGPR per load and no vector ALU work.
+// Coordinates of the fixed axis beyond the matrix are CLAMPED to the last valid row / chunk (the caller never
+// stores results that depend on them); the sliding axis must be a whole number of tiles.
+template <typename T, int ROWS, int COLS, int NT, bool ALONG_COLS> struct ClampTileDma {
+    static constexpr int CPR = COLS / 8;
+    static constexpr int TOTAL = ROWS * CPR;
+    static constexpr int N = TOTAL / NT;
+    static_assert(TOTAL % NT == 0 && NT % 64 == 0, "tile must split evenly over the waves");
+    unsigned off[N];
+    const char* origin;     // wave-uniform
+    long step;              // bytes per tile
+
+    __device__ __forceinline__ void init(const T* __restrict__ base, long ld, int fixed0, int fixed_max,
+                                         int slide0, int tile_step, int tid) {
+        const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int p = (i * (NT / 64) + wave) * 64 + lane;
+            const int row = p / CPR, pc = p % CPR;
+            const int lc = pc ^ swz16<COLS>(row);
+            int fx = ALONG_COLS ? row : lc * 8;
+            const int sl = ALONG_COLS ? lc * 8 : row;
+            const int last = fixed_max - (ALONG_COLS ? 1 : 8) - fixed0;
+            fx = fx < last ? fx : last;
+            off[i] = (unsigned)((ALONG_COLS ? (long)fx * ld + sl : (long)sl * ld + fx) * (long)sizeof(T));
+        }
+        origin = reinterpret_cast<const char*>(base + (ALONG_COLS ? (long)fixed0 * ld + slide0 : (long)slide0 * ld + fixed0));
+        step = (ALONG_COLS ? (long)tile_step : (long)tile_step * ld) * (long)sizeof(T);
+    }
+    __device__ __forceinline__ void issue(T* lds, int tid) {
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const char* o = uniform_ptr(origin);
+#pragma unroll
+        for (int i = 0; i < N; ++i) dma16_saddr_lds(off[i], o, lds_addr(lds + (i * (NT / 64) + wave) * 512));
+        origin += step;
+    }
+};
+
 template <typename T, int ROWS, int COLS, int NT> struct RowSlideDma {
     static constexpr int CPR = COLS / 8;
     static constexpr int TOTAL = ROWS * CPR;

@@ -138,6 +138,16 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& a, int row, int co
 // through its own LDS staging block so that a lane ends up with 8 consecutive columns of a row: 16-byte
 // stores and a vector epilogue.  Lane -> (row = lane / 4 + 16 * pass, columns 8 * (lane % 4) .. + 7).
 // `stage_base` must hold 32 * 36 floats per wave and must no longer be read as tile data by any wave.
+// Compile-time loop: the body sees the index as a constant, so arrays indexed by it stay in registers even
+// when the body is too large for the unroller's budget (a rolled loop over the accumulator blocks would put
+// the whole accumulator array in scratch memory, main loop included).
+template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
 template <typename T, int TM, int TN, int WM, int WN>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, float16v (&acc)[TM][TN], float* stage_base,
                                               int m0, int n0) {
@@ -147,14 +157,14 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, float16v (&acc)
     float* stage = stage_base + wave * 32 * SPITCH;
     const int g = lane >> 5, li = lane & 31;
     const int er = lane >> 2, ec = (lane & 3) * 8;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
+    static_for<TN>([&](auto jc) __attribute__((always_inline)) {
+        constexpr int j = decltype(jc)::value;
         const int col0 = n0 + (wn * TN + j) * 32 + ec;
         float csum[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) csum[e] = 0.f;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
+        static_for<TM>([&](auto ic) __attribute__((always_inline)) {
+            constexpr int i = decltype(ic)::value;
 #pragma unroll
             for (int r = 0; r < 16; ++r) stage[acc_row(r, g) * SPITCH + li] = acc[i][j][r];
             // the block is private to the wave: LDS operations of one wave complete in order
@@ -182,7 +192,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, float16v (&acc)
                 }
             }
             __builtin_amdgcn_wave_barrier();
-        }
+        });
         if (a.nsplit == 1 && a.colsum) {
             // lanes with equal (lane & 3) hold the same columns
 #pragma unroll
@@ -199,7 +209,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, float16v (&acc)
                 for (int e = 0; e < 8; ++e) atomicAdd(a.colsum + col0 + e, csum[e]);
             }
         }
-    }
+    });
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -334,6 +344,143 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_dma_kernel(GemmArgs a) {
         }
     }
     // drain the zero-tile loads still in flight before LDS is reused for the epilogue
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Tall-tile variant for long activations (M >= 256): BM = 256 rows by four waves stacked in M, each
+// holding a 64 x BN block of the output in accumulator registers (BN up to 192 -> 192 AGPRs; one wave per
+// SIMD).  A 256 x 160 x 64 tile moves 52 KB for 5.2 MFLOP, 1.5 times the flops per byte of a 128 x 128 tile:
+// the vector-memory path into LDS (64 B/clk per CU) stops being the limit.  BN is any multiple of 32, so
+// the tile count can be matched to the 256 CUs (N = 20480: BN = 160 gives exactly 256 tiles for M = 512).
+// Tiles are loaded with ClampTileDma (whole k-tiles only) and the operand fetches of k-step s+1 are issued
+// before the MFMAs of k-step s.
+// ---------------------------------------------------------------------------------------------
+template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN, int STAGES>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_tall_kernel(GemmArgs a) {
+    typedef Elem<T> E;
+    static_assert(sizeof(T) == 2, "16-bit only");
+    constexpr int NT = WM * WN * 64;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int AR = AKM ? BM : BK, AC = AKM ? BK : BM;
+    constexpr int BR = BKM ? BN : BK, BC = BKM ? BK : BN;
+    constexpr int A_ELEMS = AR * AC, B_ELEMS = BR * BC;
+    constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
+    typedef ClampTileDma<T, AR, AC, NT, AKM> DA;
+    typedef ClampTileDma<T, BR, BC, NT, BKM> DB;
+    constexpr int NLOAD = DA::N + DB::N;
+    static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
+    constexpr int TILE_BYTES = STAGES * STAGE_ELEMS * 2;
+    constexpr int EPI_BYTES = WM * WN * 32 * 36 * 4;
+    constexpr int SMEM_BYTES = TILE_BYTES > EPI_BYTES ? TILE_BYTES : EPI_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
+    T* tiles = reinterpret_cast<T*>(smem);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WM, wn = wave / WM;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int kbeg = blockIdx.z * a.kper;
+    const int kend = min(a.K, kbeg + a.kper);
+    DA da;
+    DB db;
+    da.init(reinterpret_cast<const T*>(a.A), a.lda, m0, a.M, kbeg, BK, tid);
+    db.init(reinterpret_cast<const T*>(a.B), a.ldb, n0, a.N, kbeg, BK, tid);
+    auto issue = [&](int stage) {
+        T* sA = tiles + stage * STAGE_ELEMS;
+        da.issue(sA, tid);
+        db.issue(sA + A_ELEMS, tid);
+    };
+
+    float16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    constexpr int NKSTEP = BK / E::KSTEP;
+    constexpr int NPA = AKM ? 1 : 2, NPB = BKM ? 1 : 2;
+    // lane's fetch offsets for k-step 0 of stage 0; k-steps and stages are compile-time byte offsets for
+    // k-major operands (a k-step is two chunks further along the row)
+    int oa[NKSTEP][TM][NPA], ob[NKSTEP][TN][NPB];
+#pragma unroll
+    for (int ks = 0; ks < NKSTEP; ++ks) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int mb = (wm * TM + i) * 32;
+            if constexpr (AKM) oa[ks][i][0] = km_offset<T, AC>(mb + (lane & 31), ks * E::KSTEP, lane);
+            else tr_offsets<T, AC, false>(ks * E::KSTEP, mb, lane, oa[ks][i][0], oa[ks][i][NPA - 1]);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int nb = (wn * TN + j) * 32;
+            if constexpr (BKM) ob[ks][j][0] = A_ELEMS + km_offset<T, BC>(nb + (lane & 31), ks * E::KSTEP, lane);
+            else {
+                tr_offsets<T, BC, false>(ks * E::KSTEP, nb, lane, ob[ks][j][0], ob[ks][j][NPB - 1]);
+                ob[ks][j][0] += A_ELEMS;
+                ob[ks][j][NPB - 1] += A_ELEMS;
+            }
+        }
+    }
+
+    const int nk = (kend - kbeg) / BK;          // whole tiles only (the plan guarantees it)
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s)
+        if (s < nk) issue(s);
+
+    typename E::opnd_t fa[2][TM], fb[2][TN];
+    auto fetch = [&](auto ksc, auto sc, int buf) {
+        constexpr int ks = decltype(ksc)::value, s = decltype(sc)::value;
+        const T* st = tiles + s * STAGE_ELEMS;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            if constexpr (AKM) fa[buf][i] = load_km<T>(st + oa[ks][i][0]);
+            else fa[buf][i] = load_tr<T>(st + oa[ks][i][0], st + oa[ks][i][NPA - 1]);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            if constexpr (BKM) fb[buf][j] = load_km<T>(st + ob[ks][j][0]);
+            else fb[buf][j] = load_tr<T>(st + ob[ks][j][0], st + ob[ks][j][NPB - 1]);
+        }
+    };
+    // No tile is loaded past the end of k (ClampTileDma does not bound the sliding axis): the last STAGES - 1
+    // tiles issue nothing and wait for every outstanding load instead of all but the younger tiles'.
+    auto tile = [&](auto sc, int kt) {
+        constexpr int s = decltype(sc)::value;
+        const bool more = kt + STAGES - 1 < nk;      // uniform
+        if (more) wait_vmcnt<NLOAD * (STAGES - 2)>();
+        else wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (more) issue((s + STAGES - 1) % STAGES);
+        fetch(std::integral_constant<int, 0>{}, sc, 0);
+        auto step = [&](auto ksc) {
+            constexpr int ks = decltype(ksc)::value;
+            if constexpr (ks + 1 < NKSTEP) fetch(std::integral_constant<int, ks + 1>{}, sc, (ks + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = E::mfma(fa[ks & 1][i], fb[ks & 1][j], acc[i][j]);
+        };
+        step(std::integral_constant<int, 0>{});
+        if constexpr (NKSTEP > 1) step(std::integral_constant<int, 1>{});
+        if constexpr (NKSTEP > 2) step(std::integral_constant<int, 2>{});
+        if constexpr (NKSTEP > 3) step(std::integral_constant<int, 3>{});
+        static_assert(NKSTEP <= 4, "k-tile of at most four k-steps");
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    for (int kt0 = 0; kt0 < nk; kt0 += STAGES) {
+        if (kt0 + 0 < nk) tile(std::integral_constant<int, 0>{}, kt0);
+        if constexpr (STAGES > 1) { if (kt0 + 1 < nk) tile(std::integral_constant<int, 1>{}, kt0 + 1); }
+        if constexpr (STAGES > 2) { if (kt0 + 2 < nk) tile(std::integral_constant<int, 2>{}, kt0 + 2); }
+        if constexpr (STAGES > 3) { if (kt0 + 3 < nk) tile(std::integral_constant<int, 3>{}, kt0 + 3); }
+        static_assert(STAGES <= 4, "at most four stages");
+    }
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -496,6 +643,13 @@ static const TileCfg kCfgs[] = {
     {64, 256, 64, 3},    // 11
     {64, 64, 128, 4},    // 12
     {128, 128, 64, 3},   // 13
+    {64, 64, 64, 2},     // 14: (register-staged kernel)
+    {64, 64, 64, 2},     // 15: (register-staged kernel)
+    {64, 64, 64, 2},     // 16: (register-staged kernel)
+    {256, 160, 64, 3},   // 17: tall tile, 4 waves stacked in M, 64 x 160 each (NT only)
+    {256, 128, 64, 3},   // 18: tall tile, 64 x 128 each
+    {256, 256, 64, 2},   // 19: tall tile, 8 waves (4 x 2) of 64 x 128
+    {256, 256, 32, 4},   // 20: the same with half the k-tile and twice the stages
 };
 static constexpr int kNumCfgs = (int)(sizeof(kCfgs) / sizeof(kCfgs[0]));
 
@@ -580,6 +734,10 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
         int maxs = d->K / 2048;
         if (ns > maxs) ns = maxs;
         if (ns > 8) ns = 8;
+    } else if (d->op == TP_GEMM_TN && d->K % 64 == 0 && (long)((d->M + 255) / 256) * ((d->N + 255) / 256) >= 192) {
+        // parameter gradients of a whole step: 256 x 256 tiles by eight waves (half the bytes per flop of a
+        // 128 x 128 tile through the 64 B/clk vector-memory path into LDS)
+        cfg = 19;
     } else if (t128 >= 144) {
         // short activations: the deeper ring keeps the weight stream going; parameter gradients (both
         // operands fetched with transpose reads): 128 x 128 x 32, four stages, two workgroups per CU
@@ -602,6 +760,8 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     if (ns > 16) ns = 16;
     if (forced_cfg >= 0 && forced_cfg < kNumCfgs) cfg = forced_cfg;
     if (forced_split) ns = forced_split;
+    // the tall tiles load whole k-tiles only, and the 160 / 192 wide ones exist for the k-major weight (NT)
+    if (cfg >= 17 && (d->K % 64 || (cfg == 17 && d->op != TP_GEMM_NT))) cfg = 5;
     p.cfg = cfg;
     p.gx = (d->N + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn;
     p.gy = (d->M + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm;
@@ -623,6 +783,10 @@ static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
         case 10: gemm_dma_kernel<T, AKM, BKM, 128, 128, 32, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
         case 12: gemm_dma_kernel<T, AKM, BKM, 64, 64, 128, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
         case 13: gemm_dma_kernel<T, AKM, BKM, 128, 128, 64, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
+        case 17: if constexpr (BKM) gemm_tall_kernel<T, AKM, BKM, 256, 160, 64, 4, 1, 3><<<grid, 256, 0, s>>>(a); break;
+        case 18: gemm_tall_kernel<T, AKM, BKM, 256, 128, 64, 4, 1, 3><<<grid, 256, 0, s>>>(a); break;
+        case 19: gemm_tall_kernel<T, AKM, BKM, 256, 256, 64, 4, 2, 2><<<grid, 512, 0, s>>>(a); break;
+        case 20: gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4><<<grid, 512, 0, s>>>(a); break;
         default: gemm_kernel<T, AKM, BKM, 64, 64, 64, 2, 2><<<grid, 256, 0, s>>>(a); break;
         }
     }

@@ -23,7 +23,7 @@ DEFAULT_GEOMETRIES = [
     "12288:49152:128:2048",                                 # 175B shape, 128-token slices
     "6144:24576:64:4096",                                   # 44B shape, 32-token slices x batch 2
 ]
-DMA_CFGS = [3, 5, 8, 10, 11, 12, 13]
+DMA_CFGS = [3, 5, 8, 10, 11, 12, 13, 17, 18, 19, 20]
 SPLITS = [1, 2, 3, 4, 6, 8]
 OPS = {"NT": _lib.TP_GEMM_NT, "NN": _lib.TP_GEMM_NN, "TN": _lib.TP_GEMM_TN}
 
@@ -64,7 +64,7 @@ def sweep(op, M, N, K, dtype, device, log):
     results = []
     for cfg in DMA_CFGS:
         for ns in SPLITS:
-            if K // ns < 512:
+            if K // ns < 512 or (cfg >= 17 and (M < 192 or K % 64)) or (cfg == 17 and op != "NT"):
                 continue
             try:
                 t = _time_us(lambda i: ops.gemm(code, A, Bs[i % nb], M, N, K, C=C, tile_cfg=cfg, ksplit=ns))

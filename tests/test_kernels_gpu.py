@@ -114,6 +114,38 @@ def test_gemm_nt_nn_tn(dtype, M, N, K):
         assert_close(W, 2 * ref, dtype, "TN accumulate")
 
 
+TILE_CFGS = [3, 5, 8, 10, 11, 12, 13, 17, 18, 19, 20]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("cfg", TILE_CFGS)
+def test_gemm_every_tile_configuration(dtype, cfg):
+    """Every tile configuration of the 16-bit kernels forced in turn on ragged shapes (rows and columns that
+    end inside a tile, k split and unsplit), all three operand layouts, plus one epilogue with column sums."""
+    ops = _ops()
+    from terapipe_amd import _lib as L
+    g = torch.Generator().manual_seed(cfg)
+    for (M, N, K) in [(304, 1000, 512), (520, 648, 256), (64, 160, 64)]:
+        sc = 1.0 / math.sqrt(K)
+        A, B, B2 = _rnd((M, K), dtype, g), _rnd((N, K), dtype, g, sc), _rnd((K, N), dtype, g, sc)
+        At = _rnd((K, M), dtype, g)
+        R = _rnd((M, N), dtype, g)
+        for ks in (1, 2):
+            C = torch.zeros(M, N, dtype=dtype, device=DEV)
+            ops.gemm(L.TP_GEMM_NT, A.to(DEV), B.to(DEV), M, N, K, C=C, tile_cfg=cfg, ksplit=ks)
+            assert_close(C, A.double() @ B.double().t(), dtype, "NT cfg %d split %d %s" % (cfg, ks, (M, N, K)))
+            ops.gemm(L.TP_GEMM_NN, A.to(DEV), B2.to(DEV), M, N, K, C=C, tile_cfg=cfg, ksplit=ks)
+            assert_close(C, A.double() @ B2.double(), dtype, "NN cfg %d split %d" % (cfg, ks))
+            ops.gemm(L.TP_GEMM_TN, At.to(DEV), B2.to(DEV), M, N, K, C=C, tile_cfg=cfg, ksplit=ks)
+            assert_close(C, At.double().t() @ B2.double(), dtype, "TN cfg %d split %d" % (cfg, ks))
+            acc = torch.zeros(N, dtype=torch.float32, device=DEV)
+            ops.gemm(L.TP_GEMM_NT, A.to(DEV), B.to(DEV), M, N, K, C=C, epilogue=L.TP_EPI_RELU_GRAD, aux=R.to(DEV),
+                     colsum_acc=acc, tile_cfg=cfg, ksplit=ks)
+            ref = (A.double() @ B.double().t()) * (R.double() > 0)
+            assert_close(C, ref, dtype, "relu grad cfg %d split %d" % (cfg, ks))
+            assert_close(acc, ref.sum(0), dtype, "colsum cfg %d split %d" % (cfg, ks))
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
 @pytest.mark.parametrize("M,N,K", [(32, 1024, 256), (256, 8192, 2048), (48, 264, 136)])
 def test_gemm_epilogues(dtype, M, N, K):
