@@ -156,13 +156,17 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy (torch copy_ kernel) before the steps: the "
                          "known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
-    ap.add_argument("--slice-streams", type=int, default=1,
-                    help="streams the runner spreads consecutive slices over (1 = one chain of kernels)")
+    ap.add_argument("--slice-streams", type=int, default=2,
+                    help="streams the runner spreads consecutive slices over (1 = one chain of kernels); slice "
+                         "i+1 of layer l runs beside slice i of layer l+1, which fills the CUs the short kernels "
+                         "of one slice leave idle")
     ap.add_argument("--optimizer", action="store_true",
                     help="also time the mixed-precision Adam update (fp32 master weights, loss scale 128) that "
                          "follows the step in the reference's training loop; reported beside, never inside, value")
-    ap.add_argument("--eager", action="store_true",
-                    help="launch every kernel from the host each step instead of replaying the runner's HIP graphs")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay the runner's HIP graphs (forward, backward) instead of launching every kernel "
+                         "from the host each step; one stream only")
+    ap.add_argument("--eager", action="store_true", help="launch every kernel from the host (the default)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -177,7 +181,11 @@ def main():
     from terapipe_amd import ops
 
     layers, runner, x, R = build_model(w, device)
-    runner.use_hip_graph = not args.eager
+    if args.graph and (args.eager or args.slice_streams != 1):
+        print("bench.py: --graph replays a single-stream capture; use it with --slice-streams 1 and without --eager",
+              file=sys.stderr)
+        sys.exit(2)
+    runner.use_hip_graph = args.graph
     runner.slice_streams = args.slice_streams
     if args.copy_calibration:
         src = torch.ones(64 << 20, dtype=torch.int32, device=device)
@@ -204,7 +212,7 @@ def main():
         "dtype": w["dtype"], "data": "synthetic",
         "config": {"workload": "%s: %s" % (args.workload, w["desc"]),
                    "loss": "sum(y * R), R ~ N(0,1) fixed", "optimizer_step": "outside the timed step (--optimizer times it separately)",
-                   "launch": "eager" if args.eager else "HIP-graph replay of forward and of backward",
+                   "launch": "HIP-graph replay of forward and of backward" if args.graph else "eager, every kernel launched from the host",
                    "slice_streams": args.slice_streams},
     }
 
