@@ -156,7 +156,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy (torch copy_ kernel) before the steps: the "
                          "known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
-    ap.add_argument("--slice-streams", type=int, default=2,
+    ap.add_argument("--slice-streams", type=int, default=3,
                     help="streams the runner spreads consecutive slices over (1 = one chain of kernels); slice "
                          "i+1 of layer l runs beside slice i of layer l+1, which fills the CUs the short kernels "
                          "of one slice leave idle")
@@ -167,6 +167,9 @@ def main():
                     help="replay the runner's HIP graphs (forward, backward) instead of launching every kernel "
                          "from the host each step; one stream only")
     ap.add_argument("--eager", action="store_true", help="launch every kernel from the host (the default)")
+    ap.add_argument("--no-launch-replay", action="store_true",
+                    help="rebuild every descriptor in Python each step instead of re-issuing the launches recorded "
+                         "on the second step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -187,6 +190,7 @@ def main():
         sys.exit(2)
     runner.use_hip_graph = args.graph
     runner.slice_streams = args.slice_streams
+    runner.launch_replay = not (args.graph or args.no_launch_replay)
     if args.copy_calibration:
         src = torch.ones(64 << 20, dtype=torch.int32, device=device)
         dst = torch.empty_like(src)
@@ -212,7 +216,9 @@ def main():
         "dtype": w["dtype"], "data": "synthetic",
         "config": {"workload": "%s: %s" % (args.workload, w["desc"]),
                    "loss": "sum(y * R), R ~ N(0,1) fixed", "optimizer_step": "outside the timed step (--optimizer times it separately)",
-                   "launch": "HIP-graph replay of forward and of backward" if args.graph else "eager, every kernel launched from the host",
+                   "launch": "HIP-graph replay of forward and of backward" if args.graph else
+                             ("eager, every kernel launched from the host" if args.no_launch_replay else
+                              "eager, recorded launches re-issued from the host"),
                    "slice_streams": args.slice_streams},
     }
 
@@ -223,6 +229,7 @@ def main():
         # graph keeps host launch gaps out of the figure (events around single eager launches would
         # include the time the GPU waits for the host).
         runner.use_hip_graph = False
+        runner.launch_replay = False
         with ops.CallRecorder() as rec:
             one_step(layers, runner, x, R)
         torch.cuda.synchronize()

@@ -63,13 +63,17 @@ class KernelTimer:
 
 
 class CallRecorder:
-    """Records every library call made while active as (tag, meta, replay) where replay() issues the
-    same call again on the then-current stream with the same descriptor and buffers.  bench.py replays
-    all calls of one kind back to back inside a HIP graph to time that kind of kernel without host gaps."""
+    """Records every library call made while active as (tag, meta, replay) where replay(stream=None) issues
+    the same call again with the same descriptor and buffers, on the given stream handle or else on the
+    then-current stream.  bench.py replays all calls of one kind back to back inside a HIP graph to time that
+    kind of kernel without host gaps.  With ``program`` set to a list, every call is also appended to it as
+    (replay, stream handle it was issued on): the runner interleaves its stream waits and event records in the
+    same list and re-issues the whole step from it without rebuilding a single descriptor."""
     active = None
 
-    def __init__(self):
+    def __init__(self, program=None):
         self.calls = []
+        self.program = program
 
     def __enter__(self):
         CallRecorder.active = self
@@ -83,8 +87,15 @@ class CallRecorder:
 
 
 def _record(tag, meta, replay):
-    if CallRecorder.active is not None:
-        CallRecorder.active.calls.append((tag, meta, replay))
+    rec = CallRecorder.active
+    if rec is not None:
+        rec.calls.append((tag, meta, replay))
+        if rec.program is not None:
+            rec.program.append((replay, _stream()))
+
+
+def _on(stream):
+    return _stream() if stream is None else stream
 
 
 class _timed:
@@ -148,14 +159,14 @@ def layernorm_fwd(x2d, gamma, beta, eps=1e-5, out=None, mean=None, rstd=None):
              _p(rstd), M, E, eps, tp_dtype(x2d.dtype))
         with _timed("layernorm_fwd", (M, E)):
             _lib.check(lib.tp_layernorm_fwd_partials(*a, _stream()), "tp_layernorm_fwd_partials")
-        _record("layernorm_fwd", (M, E), lambda: lib.tp_layernorm_fwd_partials(*a, _stream()))
+        _record("layernorm_fwd", (M, E), lambda s=None: lib.tp_layernorm_fwd_partials(*a, _on(s)))
         return y, mean, rstd
     with _timed("layernorm_fwd", (M, E)):
         _lib.check(lib.tp_layernorm_fwd(_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps,
                                         tp_dtype(x2d.dtype), _stream()), "tp_layernorm_fwd")
     if CallRecorder.active is not None:
         a = (_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps, tp_dtype(x2d.dtype))
-        _record("layernorm_fwd", (M, E), lambda: lib.tp_layernorm_fwd(*a, _stream()))
+        _record("layernorm_fwd", (M, E), lambda s=None: lib.tp_layernorm_fwd(*a, _on(s)))
     return y, mean, rstd
 
 
@@ -175,7 +186,7 @@ def layernorm_bwd(dy, x2d, mean, rstd, gamma, dres, dgamma_acc, dbeta_acc, colsu
              _p(dbeta_acc), _p(colsum_dres_acc), _p(colsum_dx_acc), M, E, tp_dtype(x2d.dtype))
         with _timed("layernorm_bwd", (M, E)):
             _lib.check(lib.tp_layernorm_bwd_partials(*a, _stream()), "tp_layernorm_bwd_partials")
-        _record("layernorm_bwd", (M, E), lambda: lib.tp_layernorm_bwd_partials(*a, _stream()))
+        _record("layernorm_bwd", (M, E), lambda s=None: lib.tp_layernorm_bwd_partials(*a, _on(s)))
         return dx
     with _timed("layernorm_bwd", (M, E)):
         _lib.check(lib.tp_layernorm_bwd(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx),
@@ -184,7 +195,7 @@ def layernorm_bwd(dy, x2d, mean, rstd, gamma, dres, dgamma_acc, dbeta_acc, colsu
     if CallRecorder.active is not None:
         a = (_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx), _p(dgamma_acc), _p(dbeta_acc),
              _p(colsum_dres_acc), _p(colsum_dx_acc), M, E, tp_dtype(x2d.dtype))
-        _record("layernorm_bwd", (M, E), lambda: lib.tp_layernorm_bwd(*a, _stream()))
+        _record("layernorm_bwd", (M, E), lambda s=None: lib.tp_layernorm_bwd(*a, _on(s)))
     return dx
 
 
@@ -230,7 +241,7 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
         _lib.check(lib.tp_gemm(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()), "tp_gemm")
     if CallRecorder.active is not None:
         wsp, wsn = _p(ws), (ws.numel() if ws is not None else 0)
-        _record("gemm", (op, M, N, K), lambda: lib.tp_gemm(ctypes.byref(d), wsp, wsn, _stream()))
+        _record("gemm", (op, M, N, K), lambda s=None: lib.tp_gemm(ctypes.byref(d), wsp, wsn, _on(s)))
     if nsplit > 1:
         return PendingReduce(ws, nsplit, bias, residual, C)
     return C
@@ -270,7 +281,7 @@ def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q
     if CallRecorder.active is not None:
         wsp, wsn = _p(ws), (ws.numel() if ws is not None else 0)
         _record("attn_fwd", (batch, heads, head_dim, T, cache_len),
-                lambda: lib.tp_attn_prefix_fwd(ctypes.byref(d), wsp, wsn, _stream()))
+                lambda s=None: lib.tp_attn_prefix_fwd(ctypes.byref(d), wsp, wsn, _on(s)))
     return o, lse
 
 
@@ -293,7 +304,7 @@ def attn_prefix_bwd(q, k_cache, v_cache, o, lse, d_o, dqkv, dk_cache, dv_cache, 
     with _timed("attn_bwd", (batch, heads, head_dim, T, cache_len)):
         _lib.check(lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()), "tp_attn_prefix_bwd")
     _record("attn_bwd", (batch, heads, head_dim, T, cache_len),
-            lambda: lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()))
+            lambda s=None: lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _on(s)))
     return dqkv
 
 
@@ -315,7 +326,7 @@ def attn_suffix_dkdv(k_cache, v_cache, q_all, d_o_all, lse_all, delta_all, dqkv,
     with _timed("attn_bwd", (batch, heads, head_dim, key_count, key_begin)):
         _lib.check(lib.tp_attn_suffix_dkdv(ctypes.byref(d), _stream()), "tp_attn_suffix_dkdv")
     _record("attn_bwd_dkdv", (batch, heads, head_dim, key_count, key_begin),
-            lambda: lib.tp_attn_suffix_dkdv(ctypes.byref(d), _stream()))
+            lambda s=None: lib.tp_attn_suffix_dkdv(ctypes.byref(d), _on(s)))
     return dqkv
 
 
@@ -327,21 +338,26 @@ def ln_param_grads(dy, x2d, mean, rstd, dgamma_acc, dbeta_acc):
     with _timed("ln_param_grads", (M, E)):
         _lib.check(lib.tp_ln_param_grads(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(dgamma_acc), _p(dbeta_acc), M, E,
                                          tp_dtype(x2d.dtype), _stream()), "tp_ln_param_grads")
+    if CallRecorder.active is not None:
+        a = (_p(dy), _p(x2d), _p(mean), _p(rstd), _p(dgamma_acc), _p(dbeta_acc), M, E, tp_dtype(x2d.dtype))
+        _record("ln_param_grads", (M, E), lambda s=None: lib.tp_ln_param_grads(*a, _on(s)))
 
 
 def accum_cast(dst, src_f32, accumulate):
     _require_cuda(dst, src_f32)
     lib = _lib.load()
-    _lib.check(lib.tp_accum_cast(_p(dst), _p(src_f32), dst.numel(), int(accumulate), tp_dtype(dst.dtype), _stream()),
-               "tp_accum_cast")
+    a = (_p(dst), _p(src_f32), dst.numel(), int(accumulate), tp_dtype(dst.dtype))
+    _lib.check(lib.tp_accum_cast(*a, _stream()), "tp_accum_cast")
+    _record("accum_cast", dst.numel(), lambda s=None: lib.tp_accum_cast(*a, _on(s)))
     return dst
 
 
 def colsum_acc(x2d, acc_f32):
     _require_cuda(x2d, acc_f32)
     lib = _lib.load()
-    _lib.check(lib.tp_colsum_acc(_p(x2d), x2d.stride(0), _p(acc_f32), x2d.shape[0], x2d.shape[1],
-                                 tp_dtype(x2d.dtype), _stream()), "tp_colsum_acc")
+    a = (_p(x2d), x2d.stride(0), _p(acc_f32), x2d.shape[0], x2d.shape[1], tp_dtype(x2d.dtype))
+    _lib.check(lib.tp_colsum_acc(*a, _stream()), "tp_colsum_acc")
+    _record("colsum_acc", tuple(x2d.shape), lambda s=None: lib.tp_colsum_acc(*a, _on(s)))
     return acc_f32
 
 
@@ -351,7 +367,9 @@ def zero_(t):
     nbytes = t.numel() * t.element_size()
     assert t.is_contiguous() and nbytes % 4 == 0
     lib = _lib.load()
-    _lib.check(lib.tp_zero_words(_p(t), nbytes // 4, _stream()), "tp_zero_words")
+    ptr = _p(t)
+    _lib.check(lib.tp_zero_words(ptr, nbytes // 4, _stream()), "tp_zero_words")
+    _record("zero", nbytes, lambda s=None: lib.tp_zero_words(ptr, nbytes // 4, _on(s)))
     return t
 
 

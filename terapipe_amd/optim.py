@@ -84,8 +84,8 @@ class FusedAdam(torch.optim.Optimizer):
         d.tensors = table.data_ptr()
         elems = sum(r[0].numel() for r in records)
 
-        def run():
-            _lib.check(lib.tp_adam_step(ctypes.byref(d), _stream()), "tp_adam_step")
+        def run(stream=None):
+            _lib.check(lib.tp_adam_step(ctypes.byref(d), _stream() if stream is None else stream), "tp_adam_step")
         _record("adam", dict(elems=elems, grad_bytes=torch.empty(0, dtype=grad_dtype).element_size(),
                              model_bytes=0 if model_dtype is None else 2, zero_grad=bool(zero_grad)), run)
         run()

@@ -123,10 +123,49 @@ class _StackBuffers:
         self.param_ptrs = [t.data_ptr() for w in ws for t in w.values()]
         self.fwd_graph = self.bwd_graph = None
         self.states = None
+        # launch_replay: 0 = nothing run yet, 1 = one eager pass done (workspaces have their final size),
+        # then the recorded program (list) of the pass
+        self.fwd_program = self.bwd_program = 0
+        self.program_stream = None
         # streams for the slice lanes (see TeraPipe's slice_streams); the gradient-cache mode shares per-slice
         # scratch between layers and stays on one stream
         n = runner.slice_streams if self.position_indexed else 1
         self.lanes = [torch.cuda.Stream(device=device) for _ in range(n)] if n > 1 else []
+
+
+def _program():
+    rec = ops.CallRecorder.active
+    return rec.program if rec is not None else None
+
+
+def _wait_stream(waiter, other):
+    """waiter.wait_stream(other), noted in the launch program being recorded (if any)."""
+    waiter.wait_stream(other)
+    prog = _program()
+    if prog is not None:
+        prog.append((waiter.wait_stream, other))
+
+
+def _wait_event(stream, event):
+    stream.wait_event(event)
+    prog = _program()
+    if prog is not None:
+        prog.append((stream.wait_event, event))
+
+
+def _record_event(event, stream):
+    event.record(stream)
+    prog = _program()
+    if prog is not None:
+        prog.append((event.record, stream))
+
+
+def _run_program(program):
+    """Re-issues a recorded step: every entry is (callable, argument) -- a library call bound to its descriptor
+    with the stream handle it was recorded on, or a stream wait / event record."""
+    for fn, arg in program:
+        if fn(arg):
+            raise _lib.TeraPipeHipError("replayed launch failed: %s" % (_lib.load().tp_last_error() or b"").decode())
 
 
 def _forward_body(runner, ws, act, bufs, states):
@@ -142,7 +181,7 @@ def _forward_body(runner, ws, act, bufs, states):
     lanes = bufs.lanes
     main = torch.cuda.current_stream()
     for st in lanes:
-        st.wait_stream(main)
+        _wait_stream(st, main)
     for b, Bs in enumerate(runner.batch_slices):
         pb = bufs.per_batch[b]
         cache = pb["cache"]
@@ -158,7 +197,7 @@ def _forward_body(runner, ws, act, bufs, states):
             with torch.cuda.stream(st_i):
                 for l in range(nl):
                     if lanes and prev_done is not None:
-                        st_i.wait_event(prev_done[l])
+                        _wait_event(st_i, prev_done[l])
                     if bufs.position_indexed:
                         qv, lv, rows = pb["q"][l][:, P:], pb["lse"][l][:, P:], runner.seq_len
                     else:
@@ -178,7 +217,7 @@ def _forward_body(runner, ws, act, bufs, states):
                     pending = bf.out_pending
                     if lanes:
                         ev = torch.cuda.Event()
-                        ev.record(st_i)
+                        _record_event(ev, st_i)
                         done.append(ev)
             prev_done = done
             states[b, i] = sts
@@ -186,7 +225,7 @@ def _forward_body(runner, ws, act, bufs, states):
                 runner.slice_timing["fwd"].append(_timing_event(main))
             P += T                                                               # terapipe.py:264
     for st in lanes:
-        main.wait_stream(st)
+        _wait_stream(main, st)
 
 
 def _backward_body(runner, ws, act, bufs, states):
@@ -202,7 +241,7 @@ def _backward_body(runner, ws, act, bufs, states):
     lanes = bufs.lanes
     main = torch.cuda.current_stream()
     for st in lanes:
-        st.wait_stream(main)
+        _wait_stream(st, main)
     for b in reversed(range(nb)):
         Bs = runner.batch_slices[b]
         pb = bufs.per_batch[b]
@@ -224,7 +263,7 @@ def _backward_body(runner, ws, act, bufs, states):
                 with torch.cuda.stream(st_i):
                     for l in reversed(range(nl)):
                         if lanes and later_done is not None:
-                            st_i.wait_event(later_done[l])
+                            _wait_event(st_i, later_done[l])
                         bf = core.Bufs(dz1=pb["dz1"][l][r0:r1], dhn=pb["dhn"][l][r0:r1], dh=pb["dh"][l][r0:r1],
                                        d_o=pb["d_o"][l][r0:r1], dqkv=pb["dqkv"][l][r0:r1], dxn=pb["dxn"][l][r0:r1],
                                        dx=pb["dx"][l][r0:r1], delta=pb["delta"][l][:, P:])
@@ -234,7 +273,7 @@ def _backward_body(runner, ws, act, bufs, states):
                                                    delta_all=pb["delta"][l], q_end=L))
                         if lanes:
                             done[l] = torch.cuda.Event()
-                            done[l].record(st_i)
+                            _record_event(done[l], st_i)
                 later_done = done
                 if runner.slice_timing is not None:
                     runner.slice_timing["bwd"].append(_timing_event(main))
@@ -251,7 +290,7 @@ def _backward_body(runner, ws, act, bufs, states):
             if runner.slice_timing is not None:
                 runner.slice_timing["bwd"].append(_timing_event(main))
     for st in lanes:
-        main.wait_stream(st)
+        _wait_stream(main, st)
     if runner.slice_timing is not None:
         runner.slice_timing["param"].append(_timing_event(main))
     # parameter gradients over all tokens: dW = dY_all^T X_all (one GEMM per weight and batch slice),
@@ -313,10 +352,24 @@ class _TeraPipeFunction(torch.autograd.Function):
             # the batch slice as [L*Bs, E] rows (t, b_local): a copy, as grid_slice_batch_and_sequence makes
             bufs.per_batch[b]["x"][0].view(runner.seq_len, Bs, E).copy_(inputs[:, b0:b0 + Bs, :])
             b0 += Bs
+        replayable = runner.launch_replay and ops.CallRecorder.active is None and runner.slice_timing is None
         if runner.use_hip_graph and bufs.fwd_graph is not None:
             bufs.fwd_graph.replay()
             states = bufs.states
+        elif replayable and isinstance(bufs.fwd_program, list) and \
+                bufs.program_stream == torch.cuda.current_stream().cuda_stream:
+            _run_program(bufs.fwd_program)
+            states = bufs.states
+        elif replayable and bufs.fwd_program == 1:
+            # second pass: run it and keep what it launched
+            states = np.empty((nb, ns), dtype="O")
+            with ops.CallRecorder(program=[]) as rec:
+                _forward_body(runner, ws, act, bufs, states)
+            bufs.fwd_program, bufs.states = rec.program, states
+            bufs.program_stream = torch.cuda.current_stream().cuda_stream
         else:
+            if replayable and bufs.fwd_program == 0:
+                bufs.fwd_program = 1
             states = np.empty((nb, ns), dtype="O")
             _forward_body(runner, ws, act, bufs, states)
             if runner.use_hip_graph:
@@ -343,9 +396,19 @@ class _TeraPipeFunction(torch.autograd.Function):
         for b, Bs in enumerate(runner.batch_slices):
             bufs.per_batch[b]["dx"][nl].view(L, Bs, E).copy_(grad_y[:, b0:b0 + Bs, :])
             b0 += Bs
+        replayable = runner.launch_replay and ops.CallRecorder.active is None and runner.slice_timing is None
         if runner.use_hip_graph and bufs.bwd_graph is not None:
             bufs.bwd_graph.replay()
+        elif replayable and isinstance(bufs.bwd_program, list) and states is bufs.states and \
+                bufs.program_stream == torch.cuda.current_stream().cuda_stream:
+            _run_program(bufs.bwd_program)
+        elif replayable and bufs.bwd_program == 1 and states is bufs.states:
+            with ops.CallRecorder(program=[]) as rec:
+                _backward_body(runner, ws, act, bufs, states)
+            bufs.bwd_program = rec.program
         else:
+            if replayable and bufs.bwd_program == 0:
+                bufs.bwd_program = 1
             _backward_body(runner, ws, act, bufs, states)
             if runner.use_hip_graph:
                 bufs.bwd_graph = _capture(lambda: _backward_body(runner, ws, act, bufs, states))
@@ -386,6 +449,11 @@ class TeraPipe(nn.Module):
     slice waits (by event) for layer l of the previous slice in forward -- the next slice in backward --
     so consecutive slices run one layer apart at the same time.  Same kernels, same arguments, same
     results; the overlap fills the chip where one chain of 256-row kernels cannot.
+    launch_replay: the first step runs as written, the second also keeps every library call it makes (bound
+    descriptor + stream handle) and every stream wait / event record in one list, and later steps re-issue
+    that list: the same launches on the same streams without rebuilding descriptors, views and saved state
+    (about 11 us of Python per launch otherwise, which bounds a step of short kernels from the host side).
+    Works with slice_streams; same conditions as use_hip_graph.
     use_hip_graph: after the first (eager) step, record the kernel launches of forward and of backward
     into two HIP graphs and replay them on later steps.  The runner's buffers are static and the
     launches depend only on shapes, so the replays compute the same thing without the per-launch host
@@ -393,7 +461,7 @@ class TeraPipe(nn.Module):
     """
 
     def __init__(self, layers, batch_size, seq_len, batch_slices, seq_slices, batch_dim=1, sequence_dim=0,
-                 fp32_grad_cache=True, use_hip_graph=False, suffix_dkdv=True, slice_streams=1):
+                 fp32_grad_cache=True, use_hip_graph=False, suffix_dkdv=True, slice_streams=1, launch_replay=False):
         super().__init__()
         assert sum(batch_slices) == batch_size and sum(seq_slices) == seq_len
         assert batch_dim == 1 and sequence_dim == 0, "layers take [seq, batch, embed] inputs"
@@ -405,6 +473,7 @@ class TeraPipe(nn.Module):
         self.use_hip_graph = use_hip_graph
         self.suffix_dkdv = suffix_dkdv
         self.slice_streams = int(slice_streams)
+        self.launch_replay = launch_replay
         # set to {"fwd": [], "bwd": [], "param": []} to have the (eager, single-stream) step bracket every slice's
         # forward and backward and the parameter-gradient tail with timing events (latency_model.py uses it)
         self.slice_timing = None

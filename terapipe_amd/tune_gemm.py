@@ -28,6 +28,39 @@ SPLITS = [1, 2, 3, 4, 6, 8]
 OPS = {"NT": _lib.TP_GEMM_NT, "NN": _lib.TP_GEMM_NN, "TN": _lib.TP_GEMM_TN}
 
 
+def _time_pair_us(fn, n=6):
+    """Two chains of the same call on two streams inside one graph: time per call when a neighbour shares the GPU
+    (the runner overlaps consecutive slices on two streams)."""
+    s0, s1 = torch.cuda.Stream(), torch.cuda.Stream()
+    fn(0, 0)
+    fn(1, 1)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s0):
+        fn(0, 0)
+    with torch.cuda.stream(s1):
+        fn(1, 1)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        main = torch.cuda.current_stream()
+        s1.wait_stream(main)
+        with torch.cuda.stream(s1):
+            for i in range(n):
+                fn(2 * i + 1, 1)
+        for i in range(n):
+            fn(2 * i, 0)
+        main.wait_stream(s1)
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    g.replay()
+    g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (4 * n) * 1e3
+
+
 def _time_us(fn, n=6):
     fn(0)
     torch.cuda.synchronize()
@@ -51,7 +84,7 @@ def _time_us(fn, n=6):
     return e0.elapsed_time(e1) / (2 * n) * 1e3
 
 
-def sweep(op, M, N, K, dtype, device, log):
+def sweep(op, M, N, K, dtype, device, log, pair=False):
     """Returns (best_us, cfg, nsplit, automatic_us) for one shape."""
     a_shape = (K, M) if op == "TN" else (M, K)
     b_shape = (N, K) if op == "NT" else (K, N)
@@ -60,14 +93,19 @@ def sweep(op, M, N, K, dtype, device, log):
     Bs = [torch.randn(b_shape, device=device, dtype=dtype) for _ in range(nb)]
     C = torch.empty(M, N, device=device, dtype=dtype)
     code = OPS[op]
-    auto = _time_us(lambda i: ops.gemm(code, A, Bs[i % nb], M, N, K, C=C))
+    if pair:
+        Cs = [C, torch.empty_like(C)]
+        time_it = lambda **kw: _time_pair_us(lambda i, lane: ops.gemm(code, A, Bs[i % nb], M, N, K, C=Cs[lane], **kw))
+    else:
+        time_it = lambda **kw: _time_us(lambda i: ops.gemm(code, A, Bs[i % nb], M, N, K, C=C, **kw))
+    auto = time_it()
     results = []
     for cfg in DMA_CFGS:
         for ns in SPLITS:
             if K // ns < 512 or (cfg >= 17 and (M < 192 or K % 64)) or (cfg == 17 and op != "NT"):
                 continue
             try:
-                t = _time_us(lambda i: ops.gemm(code, A, Bs[i % nb], M, N, K, C=C, tile_cfg=cfg, ksplit=ns))
+                t = time_it(tile_cfg=cfg, ksplit=ns)
             except _lib.TeraPipeHipError:
                 continue
             results.append((t, cfg, ns))
@@ -94,6 +132,9 @@ def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--geometry", action="append")
     ap.add_argument("--out", default=os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "gemm_tuned.inc"))
+    ap.add_argument("--pair", action="store_true",
+                    help="time two concurrent chains of each GEMM on two streams (per-call time with a neighbour) "
+                         "instead of one chain alone")
     ap.add_argument("--min-gain", type=float, default=0.03,
                     help="shapes whose best time is within this fraction of the heuristic plan's get no entry")
     args = ap.parse_args()
@@ -107,7 +148,7 @@ def main():
                 continue
             seen.add(shape)
             op, M, N, K = shape
-            t, cfg, ns, auto = sweep(op, M, N, K, torch.float16, device, sys.stderr)
+            t, cfg, ns, auto = sweep(op, M, N, K, torch.float16, device, sys.stderr, pair=args.pair and op != "TN")
             rows.append((op, M, N, K, cfg, ns, t, auto))
     with open(args.out, "w") as f:
         f.write("// Measured best tile configuration and k-split per shape on MI355X (fp16; written by\n"
