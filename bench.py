@@ -29,7 +29,7 @@ PEAK_HBM = 8.0e12            # bytes/s
 
 # HBM bytes per tp_gemm call (FETCH_SIZE + WRITE_SIZE of the GEMM kernels of one step / calls), from the two
 # rocprofv3 --pmc runs summarised in profiles/bench_C2_gemm_hbm_traffic.pmc.txt; only measured for C2
-PMC_GEMM_TRAFFIC_BYTES = {"C2": 31.46e6}
+PMC_GEMM_TRAFFIC_BYTES = {"C2": 29.96e6}
 
 WORKLOADS = {
     # name: layers, hidden, heads, ffn, seq, batch, dtype, slices, weight std
@@ -273,6 +273,35 @@ def main():
             "algorithmic_flops_per_step": flops, "kernel_ms_per_step": g_ms,
             "method": "graph replay of the step's GEMM calls between two HIP events",
         }
+        if args.slice_streams > 1:
+            # the same GEMM calls as the step issues them: spread over the slice streams, so that a launch
+            # which fills part of the chip runs beside its neighbours'.  Launched from the host (closures
+            # bound to their descriptors), bracketed by two events on the current stream.
+            chains = [torch.cuda.Stream() for _ in range(args.slice_streams)]
+            calls = [c for c in rec.calls if c[0] == "gemm"]
+            main = torch.cuda.current_stream()
+
+            def spread():
+                for st in chains:
+                    st.wait_stream(main)
+                for i, (_, _, fn) in enumerate(calls):
+                    if fn(chains[i % len(chains)].cuda_stream):
+                        raise RuntimeError("replayed GEMM failed")
+                for st in chains:
+                    main.wait_stream(st)
+            spread()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(3):
+                spread()
+            e1.record()
+            torch.cuda.synchronize()
+            c_ms = e0.elapsed_time(e1) / 3
+            out["roofline"]["shared_chip"] = {
+                "chains": len(chains), "kernel_ms_per_step": c_ms, "achieved": flops / (c_ms * 1e-3) / 1e12,
+                "frac": flops / (c_ms * 1e-3) / peak,
+                "method": "the step's GEMM calls issued round-robin over the slice streams, as the step overlaps them"}
         attn = {}
         kt = {"gemm": round(g_ms, 3)}
         for tag in ("attn_fwd", "attn_bwd"):
