@@ -131,6 +131,9 @@ class _StackBuffers:
         # scratch between layers and stays on one stream
         n = runner.slice_streams if self.position_indexed else 1
         self.lanes = [torch.cuda.Stream(device=device) for _ in range(n)] if n > 1 else []
+        # with lanes, the parameter gradients of a layer run on a stream of their own as soon as the first
+        # slice's backward has passed that layer
+        self.dw_stream = torch.cuda.Stream(device=device) if n > 1 else None
 
 
 def _program():
@@ -240,8 +243,11 @@ def _backward_body(runner, ws, act, bufs, states):
     ops.zero_(bufs.small)
     lanes = bufs.lanes
     main = torch.cuda.current_stream()
+    early_dw = bool(lanes) and bufs.position_indexed
     for st in lanes:
         _wait_stream(st, main)
+    if early_dw:
+        _wait_stream(bufs.dw_stream, main)
     for b in reversed(range(nb)):
         Bs = runner.batch_slices[b]
         pb = bufs.per_batch[b]
@@ -274,6 +280,14 @@ def _backward_body(runner, ws, act, bufs, states):
                         if lanes:
                             done[l] = torch.cuda.Event()
                             _record_event(done[l], st_i)
+                            if early_dw and b == 0 and i == 0:
+                                # the first slice's layer l was the last consumer of layer l: every slice's
+                                # dY and saved input of that layer are final (the event chain of a layer
+                                # runs through all later slices), so its parameter gradients start now,
+                                # beside the lower layers of this slice
+                                _wait_event(bufs.dw_stream, done[l])
+                                with torch.cuda.stream(bufs.dw_stream):
+                                    _param_grads_layer(runner, bufs, l)
                 later_done = done
                 if runner.slice_timing is not None:
                     runner.slice_timing["bwd"].append(_timing_event(main))
@@ -291,33 +305,42 @@ def _backward_body(runner, ws, act, bufs, states):
                 runner.slice_timing["bwd"].append(_timing_event(main))
     for st in lanes:
         _wait_stream(main, st)
+    if early_dw:
+        _wait_stream(main, bufs.dw_stream)
     if runner.slice_timing is not None:
         runner.slice_timing["param"].append(_timing_event(main))
     # parameter gradients over all tokens: dW = dY_all^T X_all (one GEMM per weight and batch slice),
     # bias gradients = column sums of dY_all, LayerNorm gradients from (dy, x, mean, rstd) of all rows
-    for l in range(nl):
-        sv = bufs.small_views[l]
-        g = bufs.wgrads[l]
-        for bi, pb in enumerate(bufs.per_batch):
-            R = L * runner.batch_slices[bi]
-            epi = TP_EPI_STORE if bi == 0 else TP_EPI_ACCUMULATE
-            dy_out = pb["dx"][l + 1]
-            ops.gemm(TP_GEMM_TN, pb["dqkv"][l], pb["xn"][l], 3 * E, E, R, C=g["attn.in_proj.weight"], epilogue=epi)
-            ops.gemm(TP_GEMM_TN, pb["dh"][l], pb["o"][l], E, E, R, C=g["attn.out_proj.weight"], epilogue=epi)
-            ops.gemm(TP_GEMM_TN, pb["dz1"][l], pb["hn"][l], F, E, R, C=g["fc1.weight"], epilogue=epi)
-            ops.gemm(TP_GEMM_TN, dy_out, pb["a"][l], E, F, R, C=g["fc2.weight"], epilogue=epi)
-            ops.colsum_acc(pb["dqkv"][l], sv["attn.in_proj.bias"])
-            ops.colsum_acc(pb["dh"][l], sv["attn.out_proj.bias"])
-            ops.colsum_acc(pb["dz1"][l], sv["fc1.bias"])
-            ops.colsum_acc(dy_out, sv["fc2.bias"])
-            ops.ln_param_grads(pb["dxn"][l], pb["x"][l], pb["mean1"][l], pb["rstd1"][l], sv["attn_ln.weight"],
-                               sv["attn_ln.bias"])
-            ops.ln_param_grads(pb["dhn"][l], pb["h"][l], pb["mean2"][l], pb["rstd2"][l], sv["fc_ln.weight"],
-                               sv["fc_ln.bias"])
-        for n in core.SMALL_PARAMS:
-            ops.accum_cast(bufs.sgrads[l][n], sv[n], False)
+    if not early_dw:
+        for l in range(nl):
+            _param_grads_layer(runner, bufs, l)
     if runner.slice_timing is not None:
         runner.slice_timing["param"].append(_timing_event(main))
+
+
+def _param_grads_layer(runner, bufs, l):
+    layers = runner.layers
+    E, F, L = layers.embedding_dim, layers.ffn_embedding_dim, runner.seq_len
+    sv = bufs.small_views[l]
+    g = bufs.wgrads[l]
+    for bi, pb in enumerate(bufs.per_batch):
+        R = L * runner.batch_slices[bi]
+        epi = TP_EPI_STORE if bi == 0 else TP_EPI_ACCUMULATE
+        dy_out = pb["dx"][l + 1]
+        ops.gemm(TP_GEMM_TN, pb["dqkv"][l], pb["xn"][l], 3 * E, E, R, C=g["attn.in_proj.weight"], epilogue=epi)
+        ops.gemm(TP_GEMM_TN, pb["dh"][l], pb["o"][l], E, E, R, C=g["attn.out_proj.weight"], epilogue=epi)
+        ops.gemm(TP_GEMM_TN, pb["dz1"][l], pb["hn"][l], F, E, R, C=g["fc1.weight"], epilogue=epi)
+        ops.gemm(TP_GEMM_TN, dy_out, pb["a"][l], E, F, R, C=g["fc2.weight"], epilogue=epi)
+        ops.colsum_acc(pb["dqkv"][l], sv["attn.in_proj.bias"])
+        ops.colsum_acc(pb["dh"][l], sv["attn.out_proj.bias"])
+        ops.colsum_acc(pb["dz1"][l], sv["fc1.bias"])
+        ops.colsum_acc(dy_out, sv["fc2.bias"])
+        ops.ln_param_grads(pb["dxn"][l], pb["x"][l], pb["mean1"][l], pb["rstd1"][l], sv["attn_ln.weight"],
+                           sv["attn_ln.bias"])
+        ops.ln_param_grads(pb["dhn"][l], pb["h"][l], pb["mean2"][l], pb["rstd2"][l], sv["fc_ln.weight"],
+                           sv["fc_ln.bias"])
+    for n in core.SMALL_PARAMS:
+        ops.accum_cast(bufs.sgrads[l][n], sv[n], False)
 
 
 def _timing_event(stream):
