@@ -233,6 +233,9 @@ def main():
         with ops.CallRecorder() as rec:
             one_step(layers, runner, x, R)
         torch.cuda.synchronize()
+        # the recorded weight-gradient GEMMs write into this step's gradient tensors: keep them alive while
+        # the calls are replayed
+        recorded_grads = [p.grad for p in layers.parameters()]
 
         def replay_ms(tag, reps=3):
             # "attn_bwd" covers both launches of the attention backward of a slice: delta + dQ, and the
@@ -318,6 +321,8 @@ def main():
             kt[tag] = round(replay_ms(tag)[1], 3)
         out["roofline_attention"] = {"bound": "hbm", "peak": PEAK_HBM / 1e9, "unit": "GB/s", **attn}
         out["kernel_time_ms_per_step"] = kt
+
+        del recorded_grads
 
     if args.optimizer and w["dtype"] != "f32":
         out["optimizer_step"] = optimizer_step(layers, runner, x, R)

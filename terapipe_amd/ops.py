@@ -200,12 +200,14 @@ def layernorm_bwd(dy, x2d, mean, rstd, gamma, dres, dgamma_acc, dbeta_acc, colsu
 
 
 def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=None, aux=None, aux_out=None,
-         colsum_acc=None, qkv=None, tile_cfg=None, ksplit=None, defer_reduce=False):
+         colsum_acc=None, qkv=None, tile_cfg=None, ksplit=None, defer_reduce=False, desc_sink=None):
     """Runs one GEMM.  A, B, C, residual, aux are 2-D row-major tensors (stride(1) == 1).
     qkv = dict(q, k_cache, v_cache, batch, heads, head_dim, cache_len, cache_rows, q_scale).
     tile_cfg / ksplit force a tile configuration / k-split count (tuning and tests); default automatic.
     defer_reduce (STORE / BIAS_RESIDUAL epilogues): if the plan splits k, C is left unwritten and a
-    PendingReduce is returned for the LayerNorm call that consumes C; otherwise C as usual."""
+    PendingReduce is returned for the LayerNorm call that consumes C; otherwise C as usual.
+    desc_sink: a list that receives the call's descriptor (the one a recorded replay re-issues), for callers
+    that re-point C before a replay."""
     _require_cuda(A, B, C)
     d = GemmDesc()
     d.op, d.dtype, d.epilogue = op, tp_dtype(A.dtype), epilogue
@@ -229,6 +231,8 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
         d.q_bh_rows = qkv.get("q_bh_rows", 0)
     if tile_cfg is not None or ksplit is not None:
         d.reserved = ((tile_cfg + 1) if tile_cfg is not None else 0) | ((ksplit or 0) << 8)
+    if desc_sink is not None:
+        desc_sink.append(d)
     lib = _lib.load()
     nsplit = 1
     if defer_reduce:

@@ -117,9 +117,17 @@ class _StackBuffers:
             self.per_batch.append(b)
         self.small = torch.zeros(nl, core.small_acc_numel(E, F), **f32)
         self.small_views = [core.small_acc_views(self.small[l], E, F) for l in range(nl)]
-        # parameter-gradient results (copied out to autograd after every backward)
-        self.wgrads = [{n: torch.empty_like(ws[l][n]) for n in core.BIG_PARAMS} for l in range(nl)]
-        self.sgrads = [{n: torch.empty_like(ws[l][n]) for n in core.SMALL_PARAMS} for l in range(nl)]
+        # parameter-gradient results.  Vector parameters: views of one flat tensor, copied out to autograd
+        # with one clone per backward.  Weights: views of one flat tensor that is allocated anew for every
+        # backward and handed to autograd as it is (under HIP-graph replay: static, and cloned).
+        self.sgrad_layout, n_small = _flat_layout([[(n, ws[l][n].shape) for n in core.SMALL_PARAMS] for l in range(nl)])
+        self.wgrad_layout, self.n_big = _flat_layout([[(n, ws[l][n].shape) for n in core.BIG_PARAMS] for l in range(nl)])
+        self.sgrad_flat = torch.empty(n_small, **kw)
+        self.sgrads = _flat_views(self.sgrad_flat, self.sgrad_layout)
+        self.wgrad_flat = None
+        self.wgrads = None
+        self.wgrad_descs = {}       # (layer, name) -> descriptors of the recorded weight-gradient GEMMs
+        self.recording = False
         self.param_ptrs = [t.data_ptr() for w in ws for t in w.values()]
         self.fwd_graph = self.bwd_graph = None
         self.states = None
@@ -134,6 +142,23 @@ class _StackBuffers:
         # with lanes, the parameter gradients of a layer run on a stream of their own as soon as the first
         # slice's backward has passed that layer
         self.dw_stream = torch.cuda.Stream(device=device) if n > 1 else None
+
+
+def _flat_layout(per_layer):
+    """[[(name, shape), ...] per layer] -> ([{name: (offset, shape)} per layer], total elements); offsets are
+    multiples of 128 elements (256-byte alignment for 16-bit tensors)."""
+    out, off = [], 0
+    for entries in per_layer:
+        d = {}
+        for name, shape in entries:
+            d[name] = (off, tuple(shape))
+            off += (int(np.prod(shape)) + 127) // 128 * 128
+        out.append(d)
+    return out, off
+
+
+def _flat_views(flat, layout):
+    return [{n: flat[o:o + int(np.prod(s))].view(s) for n, (o, s) in d.items()} for d in layout]
 
 
 def _program():
@@ -327,10 +352,12 @@ def _param_grads_layer(runner, bufs, l):
         R = L * runner.batch_slices[bi]
         epi = TP_EPI_STORE if bi == 0 else TP_EPI_ACCUMULATE
         dy_out = pb["dx"][l + 1]
-        ops.gemm(TP_GEMM_TN, pb["dqkv"][l], pb["xn"][l], 3 * E, E, R, C=g["attn.in_proj.weight"], epilogue=epi)
-        ops.gemm(TP_GEMM_TN, pb["dh"][l], pb["o"][l], E, E, R, C=g["attn.out_proj.weight"], epilogue=epi)
-        ops.gemm(TP_GEMM_TN, pb["dz1"][l], pb["hn"][l], F, E, R, C=g["fc1.weight"], epilogue=epi)
-        ops.gemm(TP_GEMM_TN, dy_out, pb["a"][l], E, F, R, C=g["fc2.weight"], epilogue=epi)
+        for name, dy, xin, n_out, n_in in (("attn.in_proj.weight", pb["dqkv"][l], pb["xn"][l], 3 * E, E),
+                                           ("attn.out_proj.weight", pb["dh"][l], pb["o"][l], E, E),
+                                           ("fc1.weight", pb["dz1"][l], pb["hn"][l], F, E),
+                                           ("fc2.weight", dy_out, pb["a"][l], E, F)):
+            sink = bufs.wgrad_descs.setdefault((l, name), []) if bufs.recording else None
+            ops.gemm(TP_GEMM_TN, dy, xin, n_out, n_in, R, C=g[name], epilogue=epi, desc_sink=sink)
         ops.colsum_acc(pb["dqkv"][l], sv["attn.in_proj.bias"])
         ops.colsum_acc(pb["dh"][l], sv["attn.out_proj.bias"])
         ops.colsum_acc(pb["dz1"][l], sv["fc1.bias"])
@@ -420,14 +447,30 @@ class _TeraPipeFunction(torch.autograd.Function):
             bufs.per_batch[b]["dx"][nl].view(L, Bs, E).copy_(grad_y[:, b0:b0 + Bs, :])
             b0 += Bs
         replayable = runner.launch_replay and ops.CallRecorder.active is None and runner.slice_timing is None
+        if runner.use_hip_graph:
+            if bufs.wgrad_flat is None:      # static storage for the graph
+                bufs.wgrad_flat = torch.empty(bufs.n_big, dtype=grad_y.dtype, device=grad_y.device)
+                bufs.wgrads = _flat_views(bufs.wgrad_flat, bufs.wgrad_layout)
+        else:
+            # fresh storage per backward: autograd takes these tensors as the gradients, no copy
+            bufs.wgrad_flat = torch.empty(bufs.n_big, dtype=grad_y.dtype, device=grad_y.device)
+            bufs.wgrads = _flat_views(bufs.wgrad_flat, bufs.wgrad_layout)
         if runner.use_hip_graph and bufs.bwd_graph is not None:
             bufs.bwd_graph.replay()
         elif replayable and isinstance(bufs.bwd_program, list) and states is bufs.states and \
                 bufs.program_stream == torch.cuda.current_stream().cuda_stream:
+            for (l, name), descs in bufs.wgrad_descs.items():
+                ptr = bufs.wgrads[l][name].data_ptr()
+                for d in descs:
+                    d.C = ptr
             _run_program(bufs.bwd_program)
         elif replayable and bufs.bwd_program == 1 and states is bufs.states:
-            with ops.CallRecorder(program=[]) as rec:
-                _backward_body(runner, ws, act, bufs, states)
+            bufs.wgrad_descs, bufs.recording = {}, True
+            try:
+                with ops.CallRecorder(program=[]) as rec:
+                    _backward_body(runner, ws, act, bufs, states)
+            finally:
+                bufs.recording = False
             bufs.bwd_program = rec.program
         else:
             if replayable and bufs.bwd_program == 0:
@@ -435,12 +478,16 @@ class _TeraPipeFunction(torch.autograd.Function):
             _backward_body(runner, ws, act, bufs, states)
             if runner.use_hip_graph:
                 bufs.bwd_graph = _capture(lambda: _backward_body(runner, ws, act, bufs, states))
-        # the gradient buffers are reused by the next step: hand autograd copies
+        # vector-parameter gradients: one clone of the flat buffer (it is reused by the next step); weight
+        # gradients: this backward's own storage, or a clone of the graph's static one
+        sviews = _flat_views(bufs.sgrad_flat.clone(), bufs.sgrad_layout)
+        wviews = _flat_views(bufs.wgrad_flat.clone(), bufs.wgrad_layout) if runner.use_hip_graph else bufs.wgrads
         grads = []
         for l in range(nl):
             for n in core.PARAM_NAMES:
-                src = bufs.wgrads[l][n] if n in bufs.wgrads[l] else bufs.sgrads[l][n]
-                grads.append(src.clone())
+                grads.append(wviews[l][n] if n in wviews[l] else sviews[l][n])
+        if not runner.use_hip_graph:
+            bufs.wgrad_flat = bufs.wgrads = None
         dinputs = None
         if ctx.needs_input_grad[1]:
             if len(runner.batch_slices) == 1:
