@@ -138,7 +138,9 @@ class _StackBuffers:
         # streams for the slice lanes (see TeraPipe's slice_streams); the gradient-cache mode shares per-slice
         # scratch between layers and stays on one stream
         n = runner.slice_streams if self.position_indexed else 1
-        self.lanes = [torch.cuda.Stream(device=device) for _ in range(n)] if n > 1 else []
+        # (lane 0 is the stream the runner is called on: the GPU has few hardware queues per process and two
+        # lanes on one queue would run in turn)
+        self.lanes = [torch.cuda.Stream(device=device) for _ in range(n - 1)] if n > 1 else []
         # with lanes, the parameter gradients of a layer run on a stream of their own as soon as the first
         # slice's backward has passed that layer
         self.dw_stream = torch.cuda.Stream(device=device) if n > 1 else None
@@ -206,9 +208,10 @@ def _forward_body(runner, ws, act, bufs, states):
     the chip busier than one chain of short kernels can."""
     layers = runner.layers
     nl, H, E = layers.n_layers, layers.num_attention_heads, layers.embedding_dim
-    lanes = bufs.lanes
+    side = bufs.lanes
     main = torch.cuda.current_stream()
-    for st in lanes:
+    lanes = [main] + side if side else []
+    for st in side:
         _wait_stream(st, main)
     for b, Bs in enumerate(runner.batch_slices):
         pb = bufs.per_batch[b]
@@ -252,7 +255,7 @@ def _forward_body(runner, ws, act, bufs, states):
             if runner.slice_timing is not None:
                 runner.slice_timing["fwd"].append(_timing_event(main))
             P += T                                                               # terapipe.py:264
-    for st in lanes:
+    for st in side:
         _wait_stream(main, st)
 
 
@@ -266,10 +269,11 @@ def _backward_body(runner, ws, act, bufs, states):
     nb, ns = len(runner.batch_slices), len(runner.seq_slices)
     L = runner.seq_len
     ops.zero_(bufs.small)
-    lanes = bufs.lanes
+    side = bufs.lanes
     main = torch.cuda.current_stream()
+    lanes = [main] + side if side else []
     early_dw = bool(lanes) and bufs.position_indexed
-    for st in lanes:
+    for st in side:
         _wait_stream(st, main)
     if early_dw:
         _wait_stream(bufs.dw_stream, main)
@@ -328,7 +332,7 @@ def _backward_body(runner, ws, act, bufs, states):
                                has_incoming=not last, zero_slice_rows=False, activation=act[l], buf=bf)
             if runner.slice_timing is not None:
                 runner.slice_timing["bwd"].append(_timing_event(main))
-    for st in lanes:
+    for st in side:
         _wait_stream(main, st)
     if early_dw:
         _wait_stream(main, bufs.dw_stream)
