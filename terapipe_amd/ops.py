@@ -117,6 +117,11 @@ class _timed:
             KernelTimer.active.records.append((self.tag, self.meta, self.e0, e1))
 
 
+# (op, M, N, K) -> (tile configuration, k splits): overrides the library's plan for that shape.  A tuning hook:
+# terapipe_amd.tune_gemm's in-step search fills it to time whole steps with one shape's plan changed.
+GEMM_PLAN_OVERRIDE = {}
+
+
 class Workspace:
     """A grow-only scratch tensor per device and stream (torch-owned), handed to calls that need
     workspace: kernels of different streams may run at the same time and must not share partial sums."""
@@ -229,6 +234,8 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
         d.batch, d.heads, d.head_dim = qkv["batch"], qkv["heads"], qkv["head_dim"]
         d.cache_len, d.cache_rows, d.q_scale = qkv["cache_len"], qkv["cache_rows"], qkv["q_scale"]
         d.q_bh_rows = qkv.get("q_bh_rows", 0)
+    if tile_cfg is None and ksplit is None and GEMM_PLAN_OVERRIDE:
+        tile_cfg, ksplit = GEMM_PLAN_OVERRIDE.get((op, M, N, K), (None, None))
     if tile_cfg is not None or ksplit is not None:
         d.reserved = ((tile_cfg + 1) if tile_cfg is not None else 0) | ((ksplit or 0) << 8)
     if desc_sink is not None:

@@ -8,6 +8,14 @@ GEMMs (NN) are measured at every ``slice_tokens`` (tokens of a slice x batch), t
 (TN) at ``step_tokens`` (all tokens of a step).  Weights rotate through a set larger than the caches so that
 they stream from HBM as they do in a step.  Needs the GPU, and a library built with an empty table (the
 heuristic plan is the yardstick); rebuild the library afterwards.
+
+    python -m terapipe_amd.tune_gemm --in-step 2048:8192:16:24:1:256,256,256,256,256,256,256,256
+
+searches in the step itself instead (``hidden:ffn:heads:layers:batch:slice_tokens,...``): the runner runs whole
+forward + backward steps with three slice streams and launch replay, and one slice GEMM shape at a time is given
+every plan in turn (``ops.GEMM_PLAN_OVERRIDE``); a plan is kept when it shortens the step.  It starts from the
+table that is compiled in and prints the entries to change.  This is the measure that counts when launches
+overlap: the fastest plan for a GEMM alone on the chip is often not the one that shares it best.
 """
 import argparse
 import os
@@ -128,10 +136,87 @@ def shapes_of(geometry):
     return out
 
 
+def in_step(spec, dtype=torch.float16, log=sys.stderr):
+    """Coordinate descent over the plans of the slice GEMMs (NT forward, NN data gradient) of one geometry,
+    timing whole steps.  Returns [(op, M, N, K, cfg, nsplit)] for the shapes whose plan changed."""
+    import time
+    from . import TeraPipe, TransformerLayers
+    E, F, H, n_layers, B, slices = spec.split(":")
+    E, F, H, n_layers, B = int(E), int(F), int(H), int(n_layers), int(B)
+    slices = [int(v) for v in slices.split(",")]
+    L = sum(slices)
+    device = torch.device("cuda:0")
+    layers = TransformerLayers(n_layers, E, F, H, dtype=dtype, device=device)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    with torch.no_grad():
+        for p in layers.parameters():
+            if p.dim() == 2:
+                p.copy_((torch.randn(p.shape, generator=g) * 0.02).to(dtype))
+    runner = TeraPipe(layers, B, L, [B], slices, slice_streams=3, launch_replay=True)
+    x = torch.randn(L, B, E, generator=g).to(dtype).to(device)
+    R = torch.randn(L, B, E, generator=g).to(dtype).to(device)
+
+    def one_step():
+        for p in layers.parameters():
+            p.grad = None
+        (runner(x) * R).sum().backward()
+
+    def step_ms(n):
+        if runner._sbufs is not None:       # record the launches again under the current overrides
+            runner._sbufs.fwd_program = runner._sbufs.bwd_program = 0
+        for _ in range(3):
+            one_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            one_step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e3
+
+    base = min(step_ms(8), step_ms(8))
+    print("step with the compiled-in plans: %.2f ms" % base, file=log, flush=True)
+    shapes = []
+    for N, K in ((3 * E, E), (E, E), (F, E), (E, F)):
+        for M in sorted({t * B for t in slices}):
+            shapes += [("NT", M, N, K), ("NN", M, K, N)]
+    chosen = {}
+    for op, M, N, K in shapes:
+        key = (OPS[op], M, N, K)
+        trials = []
+        for cfg in DMA_CFGS:
+            for ns in (1, 2, 3, 4):
+                if K // ns < 512 or (cfg >= 17 and (M < 192 or K % 64)) or (cfg == 17 and op != "NT"):
+                    continue
+                ops.GEMM_PLAN_OVERRIDE[key] = (cfg, ns)
+                try:
+                    trials.append((step_ms(4), cfg, ns))
+                except _lib.TeraPipeHipError:
+                    pass
+        trials.sort()
+        ops.GEMM_PLAN_OVERRIDE.pop(key, None)
+        pick, pick_ms = None, min(step_ms(8), step_ms(8))
+        for _, cfg, ns in trials[:2]:           # confirm against the incumbent with longer runs
+            ops.GEMM_PLAN_OVERRIDE[key] = (cfg, ns)
+            t = min(step_ms(8), step_ms(8))
+            if t < 0.995 * pick_ms:
+                pick, pick_ms = (cfg, ns), t
+        if pick is None:
+            ops.GEMM_PLAN_OVERRIDE.pop(key, None)
+        else:
+            ops.GEMM_PLAN_OVERRIDE[key] = pick
+            chosen[(op, M, N, K)] = pick + (pick_ms,)
+        print("%s %dx%dx%d: %s -> step %.2f ms" % (op, M, N, K, pick or "unchanged", pick_ms), file=log, flush=True)
+    print("step with the picks: %.2f ms" % min(step_ms(8), step_ms(8)), file=log, flush=True)
+    return [(op, M, N, K, c, ns, ms) for (op, M, N, K), (c, ns, ms) in chosen.items()]
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--geometry", action="append")
     ap.add_argument("--out", default=os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "gemm_tuned.inc"))
+    ap.add_argument("--in-step", metavar="SPEC",
+                    help="hidden:ffn:heads:layers:batch:slice_tokens,... -- search the slice GEMM plans by timing "
+                         "whole steps; prints the table entries to change")
     ap.add_argument("--pair", action="store_true",
                     help="time two concurrent chains of each GEMM on two streams (per-call time with a neighbour) "
                          "instead of one chain alone")
@@ -140,6 +225,10 @@ def main():
     args = ap.parse_args()
     if not torch.cuda.is_available():
         sys.exit("tune_gemm: needs the GPU")
+    if args.in_step:
+        for op, M, N, K, cfg, ns, ms in in_step(args.in_step):
+            print("{TP_GEMM_%s, %d, %d, %d, %d, %d},  // in-step search: step %.2f ms" % (op, M, N, K, cfg, ns, ms))
+        return
     device = torch.device("cuda:0")
     seen, rows = set(), []
     for geo in args.geometry or DEFAULT_GEOMETRIES:
