@@ -29,7 +29,7 @@ PEAK_HBM = 8.0e12            # bytes/s
 
 # HBM bytes per tp_gemm call (FETCH_SIZE + WRITE_SIZE of the GEMM kernels of one step / calls), from the two
 # rocprofv3 --pmc runs summarised in profiles/bench_C2_gemm_hbm_traffic.pmc.txt; only measured for C2
-PMC_GEMM_TRAFFIC_BYTES = {"C2": 29.96e6}
+PMC_GEMM_TRAFFIC_BYTES = {"C2": 31.38e6}
 
 WORKLOADS = {
     # name: layers, hidden, heads, ffn, seq, batch, dtype, slices, weight std
