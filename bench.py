@@ -75,7 +75,7 @@ def build_model(w, device):
         for p in layers.parameters():
             if p.dim() == 2:   # weights N(0, std); biases stay 0, LayerNorm gamma 1 / beta 0
                 p.copy_((torch.randn(p.shape, generator=g) * w["std"]).to(dt))
-    runner = ta.TeraPipe(layers, w["B"], w["L"], [w["B"]], w["slices"])
+    runner = ta.TeraPipe(layers, w["B"], w["L"], [w["B"]], w["slices"], slice_streams=1, launch_replay=False)
     x = torch.randn(w["L"], w["B"], w["E"], generator=g).to(dt).to(device)
     R = torch.randn(w["L"], w["B"], w["E"], generator=g).to(dt).to(device)
     return layers, runner, x, R

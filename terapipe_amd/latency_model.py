@@ -116,7 +116,7 @@ def measure_layer_latency(layers, batch_size, seqlen, slice_lens, reps=3):
     for s in slice_lens:
         n = seqlen // s
         slices = [s] * n + ([seqlen - n * s] if seqlen % s else [])
-        runner = TeraPipe(layers, batch_size, seqlen, [batch_size], slices)
+        runner = TeraPipe(layers, batch_size, seqlen, [batch_size], slices, slice_streams=1, launch_replay=False)
         x = torch.randn(seqlen, batch_size, E, device=dev, dtype=dt)
         r = torch.randn(seqlen, batch_size, E, device=dev, dtype=dt)
         acc = np.zeros((reps, n))

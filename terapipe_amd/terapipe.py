@@ -137,6 +137,7 @@ class _StackBuffers:
         self.program_stream = None
         # streams for the slice lanes (see TeraPipe's slice_streams); the gradient-cache mode shares per-slice
         # scratch between layers and stays on one stream
+        self.slice_streams = runner.slice_streams
         n = runner.slice_streams if self.position_indexed else 1
         # (lane 0 is the stream the runner is called on: the GPU has few hardware queues per process and two
         # lanes on one queue would run in turn)
@@ -535,7 +536,7 @@ class TeraPipe(nn.Module):
     """
 
     def __init__(self, layers, batch_size, seq_len, batch_slices, seq_slices, batch_dim=1, sequence_dim=0,
-                 fp32_grad_cache=True, use_hip_graph=False, suffix_dkdv=True, slice_streams=1, launch_replay=False):
+                 fp32_grad_cache=True, use_hip_graph=False, suffix_dkdv=True, slice_streams=None, launch_replay=None):
         super().__init__()
         assert sum(batch_slices) == batch_size and sum(seq_slices) == seq_len
         assert batch_dim == 1 and sequence_dim == 0, "layers take [seq, batch, embed] inputs"
@@ -546,8 +547,9 @@ class TeraPipe(nn.Module):
         self.fp32_grad_cache = fp32_grad_cache
         self.use_hip_graph = use_hip_graph
         self.suffix_dkdv = suffix_dkdv
-        self.slice_streams = int(slice_streams)
-        self.launch_replay = launch_replay
+        # defaults: three slice streams and launch replay; one stream and no replay under use_hip_graph
+        self.slice_streams = int(slice_streams) if slice_streams is not None else (1 if use_hip_graph else 3)
+        self.launch_replay = bool(launch_replay) if launch_replay is not None else not use_hip_graph
         # set to {"fwd": [], "bwd": [], "param": []} to have the (eager, single-stream) step bracket every slice's
         # forward and backward and the parameter-gradient tail with timing events (latency_model.py uses it)
         self.slice_timing = None
@@ -567,7 +569,8 @@ class TeraPipe(nn.Module):
     def _stack_buffers(self, dtype, device, ws):
         ptrs = [t.data_ptr() for w in ws for t in w.values()]
         if (self._sbufs is None or self._sbufs.dtype != dtype or self._sbufs.device != device
-                or self._sbufs.param_ptrs != ptrs):     # recorded graphs hold the parameter addresses
+                or self._sbufs.slice_streams != self.slice_streams
+                or self._sbufs.param_ptrs != ptrs):     # recorded graphs / launches hold the parameter addresses
             self._sbufs = _StackBuffers(self, dtype, device, ws)
         return self._sbufs
 

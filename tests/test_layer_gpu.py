@@ -224,6 +224,8 @@ def test_reference_style_slice_loop(dtype):
 def _run_terapipe(ta, layers, x, dy, B, L, bs, ss, keep_states=False, **kw):
     for p in layers.parameters():
         p.grad = None
+    kw.setdefault("slice_streams", 1)
+    kw.setdefault("launch_replay", False)
     runner = ta.TeraPipe(layers, B, L, bs, ss, **kw)
     runner.keep_states = keep_states
     xd = x.to(DEV).requires_grad_(True)
@@ -478,7 +480,7 @@ def test_hip_graph_replays_match_eager(dtype):
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps, "gelu")
     # three slice lanes as well (16 bit): the recorded graphs then hold the cross-stream dependencies
     graph_runner = ta.TeraPipe(layers, B, L, bs, ss, use_hip_graph=True, slice_streams=3)
-    eager_runner = ta.TeraPipe(layers, B, L, bs, ss)
+    eager_runner = ta.TeraPipe(layers, B, L, bs, ss, slice_streams=1, launch_replay=False)
 
     def step(runner, x, dy):
         for p in layers.parameters():
@@ -506,8 +508,8 @@ def test_hip_graph_replays_match_eager(dtype):
     assert graph_runner._sbufs.fwd_graph is not None and graph_runner._sbufs.bwd_graph is not None
 
 
-@pytest.mark.parametrize("dtype,streams", [(torch.float32, 1), (torch.float16, 1), (torch.float16, 3), (torch.bfloat16, 2)],
-                         ids=str)
+@pytest.mark.parametrize("dtype,streams", [(torch.float32, 1), (torch.float16, 1), (torch.float16, 3), (torch.bfloat16, 2),
+                                           (torch.bfloat16, None)], ids=str)
 def test_launch_replay_matches_eager(dtype, streams):
     """launch_replay=True: step 1 runs as written, step 2 also records every library call and stream
     operation, later steps re-issue the recorded list.  Six steps on different inputs (an in-place parameter
@@ -517,8 +519,12 @@ def test_launch_replay_matches_eager(dtype, streams):
     bs, ss = [1, 1], [32, 48, 16]
     ps = make_params(n_layers, E, Fd, dtype, seed=16)
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps, "gelu")
-    replay_runner = ta.TeraPipe(layers, B, L, bs, ss, launch_replay=True, slice_streams=streams)
-    eager_runner = ta.TeraPipe(layers, B, L, bs, ss)
+    if streams is None:       # the constructor's defaults: three slice streams, launch replay
+        replay_runner = ta.TeraPipe(layers, B, L, bs, ss)
+        assert replay_runner.slice_streams == 3 and replay_runner.launch_replay
+    else:
+        replay_runner = ta.TeraPipe(layers, B, L, bs, ss, launch_replay=True, slice_streams=streams)
+    eager_runner = ta.TeraPipe(layers, B, L, bs, ss, slice_streams=1, launch_replay=False)
 
     def step(runner, x, dy):
         for p in layers.parameters():
