@@ -50,10 +50,15 @@ class Bufs:
     lse / delta are views, starting at the slice's position, into position-indexed buffers with that many
     rows per (batch, head) -- 0 means compact [B*H, T, ...] tensors.  x_pending: the layer input is still the
     partial sums of the previous layer's k-split fc2 GEMM (ops.PendingReduce) and the first LayerNorm
-    finishes it; defer_out: leave this layer's fc2 output in that state, returned in out_pending."""
+    finishes it; defer_out: leave this layer's fc2 output in that state, returned in out_pending.
+    sync: called (no arguments) at the one point of the layer where a slice depends on other slices: in forward
+    after the in_proj GEMM has been launched and before the attention kernel (which reads the K/V rows the
+    earlier slices' in_proj GEMMs write), in backward between the dQ kernel (which leaves this slice's delta)
+    and the one-pass dK/dV kernel (which reads dO and delta of every later slice).  A runner that spreads
+    slices over streams waits for / records its events there."""
     __slots__ = ("xn", "mean1", "rstd1", "q", "o", "lse", "h", "mean2", "rstd2", "hn", "a", "z", "out",
                  "dz1", "dhn", "dh", "d_o", "dqkv", "dxn", "dx", "delta", "q_bh_rows", "stat_bh_rows",
-                 "x_pending", "defer_out", "out_pending")
+                 "x_pending", "defer_out", "out_pending", "sync")
 
     def __init__(self, **kw):
         for n in self.__slots__:
@@ -81,6 +86,8 @@ def attention_fwd(w, xn2d, T, B, heads, k_cache, v_cache, cache_len, buf=_NOBUF)
              bias=w["attn.in_proj.bias"],
              qkv=dict(q=q, k_cache=k_cache, v_cache=v_cache, batch=B, heads=heads, head_dim=Dh,
                       cache_len=cache_len, cache_rows=k_cache.shape[1], q_scale=scale, q_bh_rows=buf.q_bh_rows))
+    if buf.sync is not None:
+        buf.sync()
     o, lse = ops.attn_prefix_fwd(q, k_cache, v_cache, B, heads, Dh, T, cache_len, scale, out=buf.o, lse=buf.lse,
                                  q_bh_rows=buf.q_bh_rows, stat_bh_rows=buf.stat_bh_rows)
     return q, o, lse
@@ -189,6 +196,8 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
         ops.attn_prefix_bwd(st.q, st.k_cache, st.v_cache, st.o, st.lse, d_o, dqkv, None, None, B, heads, Dh, T,
                             st.cache_len, float(Dh) ** -0.5, False, False, False, delta=buf.delta,
                             q_bh_rows=st.q_bh_rows, stat_bh_rows=st.stat_bh_rows, dq_only=True)
+        if buf.sync is not None:
+            buf.sync()
         ops.attn_suffix_dkdv(st.k_cache, st.v_cache, suffix["q_all"], suffix["d_o_all"], suffix["lse_all"],
                              suffix["delta_all"], dqkv, B, heads, Dh, st.cache_len, T, suffix["q_end"])
         if "attn.in_proj.bias" in sa:

@@ -204,9 +204,10 @@ def _forward_body(runner, ws, act, bufs, states):
     slices from bufs x[0] and leaving the outputs in bufs x[n_layers].  Launches kernels only (no
     allocation, no host synchronisation), so it can be recorded into a HIP graph.
 
-    With slice lanes (bufs.lanes) slice i runs on stream i mod n and its layer l waits for layer l of
-    slice i-1 (the K/V rows it attends to): consecutive slices then overlap one layer apart, which keeps
-    the chip busier than one chain of short kernels can."""
+    With slice lanes (bufs.lanes) slice i runs on stream i mod n; the only cross-slice dependency of a layer
+    (the attention kernel reads the K/V rows of the earlier slices) is enforced by an event at that point, so
+    consecutive slices run through the stack side by side, which keeps the chip busier than one chain of
+    short kernels can and lets GEMMs that use the same weight share its way through the caches."""
     layers = runner.layers
     nl, H, E = layers.n_layers, layers.num_attention_heads, layers.embedding_dim
     side = bufs.lanes
@@ -228,8 +229,20 @@ def _forward_body(runner, ws, act, bufs, states):
                 runner.slice_timing["fwd"].append(_timing_event(main))
             with torch.cuda.stream(st_i):
                 for l in range(nl):
-                    if lanes and prev_done is not None:
-                        _wait_event(st_i, prev_done[l])
+                    sync = None
+                    if lanes:
+                        # the attention of (slice i, layer l) reads the K/V rows that the in_proj GEMMs of the
+                        # earlier slices write at layer l: after its own in_proj GEMM the slice waits for the
+                        # previous slice's event of that layer, then records its own -- so an event stands
+                        # for the in_proj GEMMs of every slice up to its own.  Nothing else ties slices
+                        # together: consecutive slices run through a layer side by side, and the GEMMs that
+                        # stream the same weight at the same time share its way through the caches.
+                        def sync(l=l, st_i=st_i, prev=prev_done, done=done):
+                            if prev is not None:
+                                _wait_event(st_i, prev[l])
+                            ev = torch.cuda.Event()
+                            _record_event(ev, st_i)
+                            done.append(ev)
                     if bufs.position_indexed:
                         qv, lv, rows = pb["q"][l][:, P:], pb["lse"][l][:, P:], runner.seq_len
                     else:
@@ -242,15 +255,11 @@ def _forward_body(runner, ws, act, bufs, states):
                                    stat_bh_rows=rows, h=pb["h"][l][r0:r1], x_pending=pending, defer_out=l + 1 < nl,
                                    mean2=pb["mean2"][l][r0:r1], rstd2=pb["rstd2"][l][r0:r1], hn=pb["hn"][l][r0:r1],
                                    a=pb["a"][l][r0:r1], z=None if pb["z"][l] is None else pb["z"][l][r0:r1],
-                                   out=pb["x"][l + 1][r0:r1])
+                                   out=pb["x"][l + 1][r0:r1], sync=sync)
                     _, st = core.layer_fwd(ws[l], pb["x"][l][r0:r1].view(T, Bs, E), H, cache[2 * l], cache[2 * l + 1],
                                            P, act[l], need_state=True, buf=bf)
                     sts.append(st)
                     pending = bf.out_pending
-                    if lanes:
-                        ev = torch.cuda.Event()
-                        _record_event(ev, st_i)
-                        done.append(ev)
             prev_done = done
             states[b, i] = sts
             if runner.slice_timing is not None:
@@ -274,6 +283,7 @@ def _backward_body(runner, ws, act, bufs, states):
     main = torch.cuda.current_stream()
     lanes = [main] + side if side else []
     early_dw = bool(lanes) and bufs.position_indexed
+    finished = [[] for _ in range(nl)]
     for st in side:
         _wait_stream(st, main)
     if early_dw:
@@ -298,24 +308,34 @@ def _backward_body(runner, ws, act, bufs, states):
                 done = [None] * nl
                 with torch.cuda.stream(st_i):
                     for l in reversed(range(nl)):
-                        if lanes and later_done is not None:
-                            _wait_event(st_i, later_done[l])
+                        sync = None
+                        if lanes:
+                            # the one-pass dK/dV of (slice i, layer l) reads dO and delta of every later
+                            # slice at layer l: after its own dQ kernel (which leaves its delta; its dO is
+                            # older) the slice waits for the next slice's event of that layer, then records
+                            # its own
+                            def sync(l=l, st_i=st_i, later=later_done, done=done):
+                                if later is not None:
+                                    _wait_event(st_i, later[l])
+                                done[l] = torch.cuda.Event()
+                                _record_event(done[l], st_i)
                         bf = core.Bufs(dz1=pb["dz1"][l][r0:r1], dhn=pb["dhn"][l][r0:r1], dh=pb["dh"][l][r0:r1],
                                        d_o=pb["d_o"][l][r0:r1], dqkv=pb["dqkv"][l][r0:r1], dxn=pb["dxn"][l][r0:r1],
-                                       dx=pb["dx"][l][r0:r1], delta=pb["delta"][l][:, P:])
+                                       dx=pb["dx"][l][r0:r1], delta=pb["delta"][l][:, P:], sync=sync)
                         core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), H, None, None,
                                        None, False, None, False, False, False, activation=act[l], buf=bf,
                                        suffix=dict(q_all=pb["q"][l], d_o_all=pb["d_o"][l], lse_all=pb["lse"][l],
                                                    delta_all=pb["delta"][l], q_end=L))
                         if lanes:
-                            done[l] = torch.cuda.Event()
-                            _record_event(done[l], st_i)
+                            # end of (slice, layer): what the parameter gradients of the layer wait for
+                            fin = torch.cuda.Event()
+                            _record_event(fin, st_i)
+                            finished[l].append(fin)
                             if early_dw and b == 0 and i == 0:
-                                # the first slice's layer l was the last consumer of layer l: every slice's
-                                # dY and saved input of that layer are final (the event chain of a layer
-                                # runs through all later slices), so its parameter gradients start now,
-                                # beside the lower layers of this slice
-                                _wait_event(bufs.dw_stream, done[l])
+                                # the first slice is the last to pass layer l: once every slice has, the
+                                # parameter gradients of the layer start, beside the lower layers
+                                for ev in finished[l]:
+                                    _wait_event(bufs.dw_stream, ev)
                                 with torch.cuda.stream(bufs.dw_stream):
                                     _param_grads_layer(runner, bufs, l)
                 later_done = done
