@@ -540,10 +540,12 @@ class TeraPipe(nn.Module):
     positions (every later slice has run its backward by then) -- the same sum that the reference builds
     up through the cache gradients, without gradient caches and their read-modify-write per slice.  With
     False (and always in fp32) the gradient caches are used.
-    slice_streams (with suffix_dkdv, fp16 / bf16): slice i runs on stream i mod slice_streams; layer l of a
-    slice waits (by event) for layer l of the previous slice in forward -- the next slice in backward --
-    so consecutive slices run one layer apart at the same time.  Same kernels, same arguments, same
-    results; the overlap fills the chip where one chain of 256-row kernels cannot.
+    slice_streams (with suffix_dkdv, fp16 / bf16): slice i runs on stream i mod slice_streams.  The attention
+    kernel of a layer waits (by event) for the in_proj GEMMs of the earlier slices at that layer, the one-pass
+    dK/dV kernel for the dQ kernels of the later slices; nothing else orders slices, so consecutive slices
+    run through the stack side by side.  Same kernels, same arguments, same results; the overlap fills the
+    chip where one chain of short kernels cannot, and GEMMs that stream the same weight at the same time
+    share its way through the caches.  Default 3 (1 under use_hip_graph).
     launch_replay: the first step runs as written, the second also keeps every library call it makes (bound
     descriptor + stream handle) and every stream wait / event record in one list, and later steps re-issue
     that list: the same launches on the same streams without rebuilding descriptors, views and saved state
