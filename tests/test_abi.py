@@ -145,3 +145,37 @@ def test_adam_table_validation_without_gpu(lib):
     assert lib.tp_adam_step(ctypes.byref(d), None) == 1
     d.n_tensors, d.tensors, d.model_dtype, d.step = 1, 256, -1, 0
     assert lib.tp_adam_step(ctypes.byref(d), None) == 1 and b"step" in lib.tp_last_error()
+
+
+def test_measured_gemm_plans_are_looked_up_without_gpu(lib):
+    """plan_gemm consults csrc/gemm_tuned.inc before its heuristics: the weight extents match exactly and the
+    nearest measured M at or above the slice's (within a factor of two) is taken.  tp_gemm_splits exposes the
+    planned k-split, which is enough to see which rule fired."""
+    import re
+    from terapipe_amd import _lib
+    root = os.path.join(ROOT, "terapipe_amd", "csrc", "gemm_tuned.inc")
+    entries = [tuple(m.groups()) for m in re.finditer(r"\{TP_GEMM_(NT|NN), (\d+), (\d+), (\d+), (\d+), (\d+)\}", open(root).read())]
+    assert entries, "the table holds measured plans"
+    ops_ = {"NT": _lib.TP_GEMM_NT, "NN": _lib.TP_GEMM_NN}
+    by_weight = {}
+    for op, M, N, K, cfg, ns in entries:
+        by_weight.setdefault((op, int(N), int(K)), []).append((int(M), int(ns)))
+
+    def splits(op, M, N, K):
+        d = _lib.GemmDesc()
+        d.op, d.dtype, d.M, d.N, d.K = ops_[op], _lib.TP_F16, M, N, K
+        d.A = d.B = d.C = 256                              # planning only: nothing is dereferenced
+        d.lda, d.ldb, d.ldc = K, (K if op == "NT" else N), N
+        return lib.tp_gemm_splits(ctypes.byref(d))
+
+    checked = 0
+    for (op, N, K), rows in by_weight.items():
+        rows.sort()
+        for M, ns in rows:
+            assert splits(op, M, N, K) == min(ns, K // 8), (op, M, N, K)          # the entry itself
+            lower = [m for m, _ in rows if m < M]
+            probe = M - 8                                                          # a slightly shorter slice
+            if probe > (lower[-1] if lower else 0) and 2 * probe >= M:
+                assert splits(op, probe, N, K) == ns, (op, probe, N, K)
+                checked += 1
+    assert checked > 10
