@@ -592,3 +592,40 @@ def test_latency_measurement_feeds_the_planner():
     grid = lm.fit_latency_grid(samples, 1, L, layers_per_stage=n_layers)
     scheme, latency = lm.best_plan(grid, 1, L, pipelinelen=4)
     assert scheme is not None and sum(scheme[0][1]) == L and latency >= 0 and latency == latency
+
+
+def test_default_runner_matches_single_stream_at_c2_shape():
+    """BASELINE config 2's geometry (hidden 2048, 16 heads, FFN 8192, sequence 2048 as 8 x 256, fp16) on two
+    layers: the constructor's defaults (three slice streams, launch replay) against one stream launched
+    from Python, five steps -- the first as written, the second recorded, the rest re-issued.  Same kernels
+    on the same data: outputs and input gradients are bit-identical; the parameter gradients (fp32 atomics
+    for the vector parameters) agree to rounding."""
+    ta = _mods()
+    dtype = torch.float16
+    n_layers, E, H, Fd, L, B = 2, 2048, 16, 8192, 2048, 1
+    ss = [256] * 8
+    ps = make_params(n_layers, E, Fd, dtype, seed=21)
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    fast = ta.TeraPipe(layers, B, L, [B], ss)
+    plain = ta.TeraPipe(layers, B, L, [B], ss, slice_streams=1, launch_replay=False)
+    assert fast.slice_streams == 3 and fast.launch_replay
+
+    def step(runner, x, dy):
+        for p in layers.parameters():
+            p.grad = None
+        xd = x.clone().requires_grad_(True)
+        y = runner(xd)
+        (y * dy).sum().backward()
+        return y.detach().clone(), xd.grad.clone(), [p.grad.clone() for p in layers.parameters()]
+
+    for seed in range(5):
+        g = torch.Generator().manual_seed(700 + seed)
+        x = torch.randn(L, B, E, generator=g).to(dtype).to(DEV)
+        dy = (torch.randn(L, B, E, generator=g) * 0.1).to(dtype).to(DEV)
+        y0, dx0, g0 = step(plain, x, dy)
+        y1, dx1, g1 = step(fast, x, dy)
+        torch.cuda.synchronize()
+        assert torch.equal(y1, y0), "step %d: y" % seed
+        assert torch.equal(dx1, dx0), "step %d: dx" % seed
+        for a, b in zip(g1, g0):
+            assert_close(a, b, dtype, "step %d: parameter gradient" % seed, 1.0)
