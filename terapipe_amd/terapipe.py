@@ -115,8 +115,6 @@ class _StackBuffers:
             b["gcache"] = (None if self.position_indexed else
                            [torch.empty(Bs * H, L, Dh, dtype=gdt, device=device) for _ in range(2 * nl)])
             self.per_batch.append(b)
-        self.small = torch.zeros(nl, core.small_acc_numel(E, F), **f32)
-        self.small_views = [core.small_acc_views(self.small[l], E, F) for l in range(nl)]
         # parameter-gradient results.  Vector parameters: views of one flat tensor, copied out to autograd
         # with one clone per backward.  Weights: views of one flat tensor that is allocated anew for every
         # backward and handed to autograd as it is (under HIP-graph replay: static, and cloned).
@@ -124,6 +122,9 @@ class _StackBuffers:
         self.wgrad_layout, self.n_big = _flat_layout([[(n, ws[l][n].shape) for n in core.BIG_PARAMS] for l in range(nl)])
         self.sgrad_flat = torch.empty(n_small, **kw)
         self.sgrads = _flat_views(self.sgrad_flat, self.sgrad_layout)
+        # their fp32 accumulators in the same layout, so that one launch casts all of them out
+        self.small = torch.zeros(n_small, **f32)
+        self.small_views = _flat_views(self.small, self.sgrad_layout)
         self.wgrad_flat = None
         self.wgrads = None
         self.wgrad_descs = {}       # (layer, name) -> descriptors of the recorded weight-gradient GEMMs
@@ -364,6 +365,7 @@ def _backward_body(runner, ws, act, bufs, states):
     if not early_dw:
         for l in range(nl):
             _param_grads_layer(runner, bufs, l)
+    ops.accum_cast(bufs.sgrad_flat, bufs.small, False)     # every vector-parameter gradient of the stack
     if runner.slice_timing is not None:
         runner.slice_timing["param"].append(_timing_event(main))
 
@@ -391,8 +393,6 @@ def _param_grads_layer(runner, bufs, l):
                            sv["attn_ln.bias"])
         ops.ln_param_grads(pb["dhn"][l], pb["h"][l], pb["mean2"][l], pb["rstd2"][l], sv["fc_ln.weight"],
                            sv["fc_ln.bias"])
-    for n in core.SMALL_PARAMS:
-        ops.accum_cast(bufs.sgrads[l][n], sv[n], False)
 
 
 def _timing_event(stream):
