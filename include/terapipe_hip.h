@@ -170,7 +170,8 @@ typedef struct tp_attn_desc {
     float q_scale;
     float* colsum_dqkv_acc;             /* optional [3*H*Dh] fp32: += column sums of dqkv (in_proj bias grad) */
     int32_t reserved;                   /* 0 = automatic; bits 0-7: number of key-range splits of the forward (tuning, tests) */
-    int32_t reserved2;                  /* bit 0: use the tile-sharing forward kernel with a split/merge pass (tuning, tests) */
+    int32_t reserved2;                  /* tuning, tests.  bit 0: the tile-sharing forward kernel with a split/merge pass;
+                                           bit 1 / bit 2: force the eight-wave / the four-wave form of the 16-bit forward kernel */
     int64_t q_bh_rows;                  /* rows per (b,h) block of q: 0 = T; see tp_gemm_desc.q_bh_rows */
     int64_t stat_bh_rows;               /* entries per (b,h) block of lse and delta: 0 = T */
     int32_t dq_only;                    /* backward: 1 = compute delta and the q part of dqkv only; dK/dV of the

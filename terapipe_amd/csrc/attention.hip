@@ -1407,7 +1407,11 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq2_kernel(AttnArgs a) {
 // Forward, second generation.  A workgroup owns 32 queries of one (batch, head); its NW waves split the
 // key range, each streaming its own K / V tiles of 32 keys through a private two-stage LDS ring and
 // keeping its own online-softmax state; the NW partial (m, l, O) are merged through LDS at the end.
-template <typename T, int DH, int NW>
+// STG = 1 gives a wave a single tile buffer (it loads, waits, computes) and is meant for eight waves: two
+// per SIMD take turns, which hides the load latency as the second stage does for four, and the key range
+// of a query block is split eight ways instead of four -- for the cases where (batch, head) x query blocks
+// leave CUs without a workgroup and the length of a wave's key loop is what the call takes.
+template <typename T, int DH, int NW, int STG = 2>
 __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
     typedef Elem<T> E;
     static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
@@ -1417,7 +1421,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
     constexpr int NLD = 32 * CPR / 64;
     constexpr int NLOAD = 2 * NLD;
     static_assert(NLOAD <= 63, "too many loads in flight for vmcnt");
-    constexpr int WAVE_RING = 2 * 2 * TILE * 2;
+    constexpr int WAVE_RING = STG * 2 * TILE * 2;        // bytes: STG stages of K + V
     constexpr int EPI_LD = DH + 4;
     constexpr int STAT_FLOATS = 2 * NW * 32;
     constexpr int EPI_BYTES = (STAT_FLOATS + NW * 32 * EPI_LD) * 4;
@@ -1506,11 +1510,14 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
     float m = -INFINITY, lsum = 0.f;
 
     wait_vmcnt<0>();
-    if (nt > 0) issue(0, t_beg);
+    if (STG == 2 && nt > 0) issue(0, t_beg);
 
     auto step = [&](auto stage_c, int it) {
         constexpr int s = decltype(stage_c)::value;
-        if (it + 1 < nt) {
+        if constexpr (STG == 1) {
+            issue(0, t_beg + it);          // the wave's reads of the previous tile are complete (lgkmcnt below)
+            wait_vmcnt<0>();
+        } else if (it + 1 < nt) {
             issue(s ^ 1, t_beg + it + 1);
             wait_vmcnt<NLOAD>();
         } else {
@@ -1575,7 +1582,9 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
             for (int db = 0; db < NDB; ++db) oacc[db] = E::mfma(av[hs][db], pop[hs], oacc[db]);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
-    {
+    if constexpr (STG == 1) {
+        for (int it = 0; it < nt; ++it) step(std::integral_constant<int, 0>(), it);
+    } else {
         int it = 0;
         for (; it + 1 < nt; it += 2) {
             step(std::integral_constant<int, 0>(), it);
@@ -1893,6 +1902,10 @@ static FwdPlan plan_fwd(const tp_attn_desc* d) {
     if (d->dtype != TP_F32 && !(d->reserved2 & 1)) {
         // 16-bit: one workgroup per 32 queries whose four waves split the key range and merge in LDS
         p.nw = 0; p.bn = 32; p.nsplit = 1; p.qblocks = (d->T + 31) / 32;
+        // bn doubles as the wave count of this kernel: 8 = eight waves with one tile buffer each, faster
+        // from about twenty key tiles on (measured: 19 against 24 us at 2048 keys, 7.9 against 7.6 us at 256);
+        // reserved2 bit 1 forces it, bit 2 forces four waves
+        if (((long)d->cache_len + d->T >= 640 || (d->reserved2 & 2)) && !(d->reserved2 & 4)) p.bn = 8;
         return p;
     }
     p.nw = d->T > 64 ? 4 : (d->T > 32 ? 2 : 1);
@@ -1934,7 +1947,8 @@ static void launch_fwd(const FwdPlan& p, const AttnArgs& a, hipStream_t s) {
     dim3 grid(p.qblocks, a.B * a.H, p.nsplit);
     if constexpr (sizeof(T) == 2) {
         if (p.nw == 0) {
-            attn_fwd2_kernel<T, DH, 4><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 256, 0, s>>>(a);
+            if (p.bn == 8) attn_fwd2_kernel<T, DH, 8, 1><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 512, 0, s>>>(a);
+            else attn_fwd2_kernel<T, DH, 4><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 256, 0, s>>>(a);
             return;
         }
         if (p.nw == 4) attn_fwd_dma_kernel<T, DH, 4, 64, 3><<<grid, 256, 0, s>>>(a);

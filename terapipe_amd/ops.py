@@ -273,7 +273,7 @@ def _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len
 
 
 def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q_scale, out=None, lse=None,
-                    nsplit=None, q_bh_rows=0, stat_bh_rows=0):
+                    nsplit=None, q_bh_rows=0, stat_bh_rows=0, variant=0):
     """q [B*H, T, Dh] (pre-scaled); caches [B*H, L, Dh] with rows [0, cache_len+T) valid.
     Returns o [T, B, H*Dh] and lse [B*H, T]."""
     _require_cuda(q, k_cache, v_cache)
@@ -283,6 +283,8 @@ def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q
     d = _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale, q_bh_rows, stat_bh_rows)
     if nsplit:
         d.reserved = int(nsplit)
+    if variant:
+        d.reserved2 = int(variant)      # tuning / tests: see tp_attn_desc.reserved2
     lib = _lib.load()
     need = lib.tp_attn_fwd_workspace_bytes(ctypes.byref(d))
     ws = Workspace.get(need, q.device) if need else None

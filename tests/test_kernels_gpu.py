@@ -247,6 +247,12 @@ def test_attn_prefix_fwd_bwd(dtype, T, B, H, Dh, P, L):
     assert_close(o, oref, dtype, "attn o")
     s = torch.bmm(q64, k64[:, :S].transpose(1, 2)) + oracle.causal_prefix_mask(T, P, torch.float64)
     assert_close(lse, torch.logsumexp(s, -1), torch.float32, "attn lse", 1e3 if dtype != torch.float32 else 10)
+    # both wave counts of the 16-bit forward, whatever the plan picks for this length
+    for variant in (2, 4):
+        o_v, lse_v = ops.attn_prefix_fwd(qd, kd, vd, B, H, Dh, T, P, 1.0, variant=variant)
+        assert_close(o_v, oref, dtype, "attn o, forward variant %d" % variant)
+        assert_close(lse_v, torch.logsumexp(s, -1), torch.float32, "attn lse, forward variant %d" % variant,
+                     1e3 if dtype != torch.float32 else 10)
     oref.backward(d_o.double())
     # library-routine pin for the no-prefix case
     if P == 0:
