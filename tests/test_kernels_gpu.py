@@ -146,6 +146,50 @@ def test_gemm_every_tile_configuration(dtype, cfg):
             assert_close(acc, ref.sum(0), dtype, "colsum cfg %d split %d" % (cfg, ks))
 
 
+def _tuned_entries():
+    import os
+    import re
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "terapipe_amd", "csrc",
+                        "gemm_tuned.inc")
+    rows = [(m.group(1), int(m.group(2)), int(m.group(3)), int(m.group(4)))
+            for m in re.finditer(r"\{TP_GEMM_(NT|NN|TN), (\d+), (\d+), (\d+), \d+, \d+\}", open(path).read())]
+    by_weight = {}
+    for op, M, N, K in rows:
+        by_weight.setdefault((op, N, K) if op != "TN" else (op, M, N), []).append((op, M, N, K))
+    return sorted(by_weight.items())
+
+
+@pytest.mark.parametrize("key,shapes", _tuned_entries(), ids=lambda v: "-".join(map(str, v)) if isinstance(v, tuple) else "")
+def test_gemm_measured_plans_at_their_shapes(key, shapes):
+    """Every shape of the measured plan table (the benchmark geometries' own GEMMs, with the tile configuration
+    and k-split the table prescribes for them) against the fp32 library product of the same fp16 operands."""
+    ops = _ops()
+    from terapipe_amd import _lib as L
+    dtype = torch.float16
+    g = torch.Generator(device=DEV).manual_seed(sum(v for v in key if isinstance(v, int)) % 65521)
+    op = key[0]
+    if op == "TN":
+        _, M, N = key
+        for (_, _, _, K) in shapes:
+            A = (torch.randn(K, M, generator=g, device=DEV) * 0.05).to(dtype)
+            B = torch.randn(K, N, generator=g, device=DEV).to(dtype)
+            C = torch.empty(M, N, dtype=dtype, device=DEV)
+            ops.gemm(L.TP_GEMM_TN, A, B, M, N, K, C=C)
+            rows = torch.randperm(M, generator=g, device=DEV)[:1024]
+            ref = A[:, rows].float().t() @ B.float()
+            assert_close(C[rows], ref.cpu().double(), dtype, "TN %dx%dx%d" % (M, N, K))
+        return
+    _, N, K = key
+    B = (torch.randn((N, K) if op == "NT" else (K, N), generator=g, device=DEV) * K ** -0.5).to(dtype)
+    Bf = B.float()
+    for (_, M, _, _) in shapes:
+        A = torch.randn(M, K, generator=g, device=DEV).to(dtype)
+        C = torch.empty(M, N, dtype=dtype, device=DEV)
+        ops.gemm(L.TP_GEMM_NT if op == "NT" else L.TP_GEMM_NN, A, B, M, N, K, C=C)
+        ref = A.float() @ (Bf.t() if op == "NT" else Bf)
+        assert_close(C, ref.cpu().double(), dtype, "%s %dx%dx%d" % (op, M, N, K))
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
 @pytest.mark.parametrize("M,N,K", [(32, 1024, 256), (256, 8192, 2048), (48, 264, 136)])
 def test_gemm_epilogues(dtype, M, N, K):
