@@ -129,6 +129,7 @@ class _StackBuffers:
         self.wgrads = None
         self.wgrad_descs = {}       # (layer, name) -> descriptors of the recorded weight-gradient GEMMs
         self.recording = False
+        self.generation = 0         # forward passes run on these buffers
         self.param_ptrs = [t.data_ptr() for w in ws for t in w.values()]
         self.fwd_graph = self.bwd_graph = None
         self.states = None
@@ -458,12 +459,18 @@ class _TeraPipeFunction(torch.autograd.Function):
         else:
             y = torch.cat([pb["x"][nl].view(runner.seq_len, Bs, E)
                            for pb, Bs in zip(bufs.per_batch, runner.batch_slices)], dim=1)
+        # the buffers hold ONE step's activations: a backward must run before the next forward overwrites them
+        bufs.generation += 1
+        ctx.generation = bufs.generation
         ctx.runner, ctx.ws, ctx.act, ctx.states, ctx.bufs = runner, ws, act, states, bufs
         return y
 
     @staticmethod
     def backward(ctx, grad_y):
         runner, ws, act, states, bufs = ctx.runner, ctx.ws, ctx.act, ctx.states, ctx.bufs
+        if ctx.generation != bufs.generation or bufs is not runner._sbufs:
+            raise RuntimeError("TeraPipe keeps the activations of one step in buffers that the next forward "
+                               "reuses: this backward belongs to a forward that a later forward has overwritten")
         layers = runner.layers
         nl, E = layers.n_layers, layers.embedding_dim
         L = runner.seq_len
@@ -551,6 +558,8 @@ class TeraPipe(nn.Module):
     that list: the same launches on the same streams without rebuilding descriptors, views and saved state
     (about 11 us of Python per launch otherwise, which bounds a step of short kernels from the host side).
     Works with slice_streams; same conditions as use_hip_graph.
+    One step at a time: the buffers hold the activations of the latest forward, so its backward has to run
+    before the next forward (a backward of an older forward raises).
     use_hip_graph: after the first (eager) step, record the kernel launches of forward and of backward
     into two HIP graphs and replay them on later steps.  The runner's buffers are static and the
     launches depend only on shapes, so the replays compute the same thing without the per-launch host

@@ -629,3 +629,19 @@ def test_default_runner_matches_single_stream_at_c2_shape():
         assert torch.equal(dx1, dx0), "step %d: dx" % seed
         for a, b in zip(g1, g0):
             assert_close(a, b, dtype, "step %d: parameter gradient" % seed, 1.0)
+
+
+def test_backward_of_an_overwritten_forward_raises():
+    ta = _mods()
+    dtype = torch.float16
+    n_layers, E, H, Fd, L, B = 1, 128, 2, 256, 64, 1
+    ps = make_params(n_layers, E, Fd, dtype, seed=2)
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    runner = ta.TeraPipe(layers, B, L, [B], [32, 32])
+    x = torch.randn(L, B, E).to(dtype).to(DEV).requires_grad_(True)
+    y_old = runner(x)
+    y_new = runner(x)
+    with pytest.raises(RuntimeError, match="overwritten"):
+        y_old.sum().backward()
+    y_new.sum().backward()            # the latest forward is still intact
+    assert x.grad is not None
