@@ -402,11 +402,13 @@ template <typename T, int ROWS, int COLS, int NT, bool ALONG_COLS> struct ClampT
         origin = reinterpret_cast<const char*>(base + (ALONG_COLS ? (long)fixed0 * ld + slide0 : (long)slide0 * ld + fixed0));
         step = (ALONG_COLS ? (long)tile_step : (long)tile_step * ld) * (long)sizeof(T);
     }
-    __device__ __forceinline__ void issue(T* lds, int tid) {
-        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // lds_bytes: LDS byte address of the tile (an integer: no generic-pointer cast and its null check per load);
+    // wave_uniform: the wave's index, already in a scalar register.
+    __device__ __forceinline__ void issue(unsigned lds_bytes, int wave_uniform) {
         const char* o = uniform_ptr(origin);
 #pragma unroll
-        for (int i = 0; i < N; ++i) dma16_saddr_lds(off[i], o, lds_addr(lds + (i * (NT / 64) + wave) * 512));
+        for (int i = 0; i < N; ++i)
+            dma16_saddr_lds(off[i], o, lds_bytes + (unsigned)((i * (NT / 64) + wave_uniform) * 512 * (int)sizeof(T)));
         origin += step;
     }
 };

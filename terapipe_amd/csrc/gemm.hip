@@ -388,10 +388,12 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tall_kernel(GemmArgs a) {
     DB db;
     da.init(reinterpret_cast<const T*>(a.A), a.lda, m0, a.M, kbeg, BK, tid);
     db.init(reinterpret_cast<const T*>(a.B), a.ldb, n0, a.N, kbeg, BK, tid);
+    const unsigned lds0 = lds_addr(smem);
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     auto issue = [&](int stage) {
-        T* sA = tiles + stage * STAGE_ELEMS;
-        da.issue(sA, tid);
-        db.issue(sA + A_ELEMS, tid);
+        const unsigned sA = lds0 + (unsigned)(stage * STAGE_ELEMS * (int)sizeof(T));
+        da.issue(sA, wave_u);
+        db.issue(sA + (unsigned)(A_ELEMS * (int)sizeof(T)), wave_u);
     };
 
     float16v acc[TM][TN];
@@ -456,8 +458,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tall_kernel(GemmArgs a) {
         else wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (more) issue((s + STAGES - 1) % STAGES);
         fetch(std::integral_constant<int, 0>{}, sc, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) issue((s + STAGES - 1) % STAGES);   // issued while the fetch above is in flight
         auto step = [&](auto ksc) {
             constexpr int ks = decltype(ksc)::value;
             if constexpr (ks + 1 < NKSTEP) fetch(std::integral_constant<int, ks + 1>{}, sc, (ks + 1) & 1);
