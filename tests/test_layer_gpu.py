@@ -631,6 +631,77 @@ def test_default_runner_matches_single_stream_at_c2_shape():
             assert_close(a, b, dtype, "step %d: parameter gradient" % seed, 1.0)
 
 
+def test_default_runner_usage_patterns():
+    """The constructor's defaults (three slice streams, launch replay) through what a training script does
+    besides forward + backward: evaluation passes under no_grad between training steps, a forward that is never
+    differentiated, an input that needs no gradient, an optimizer step in place, a parameter whose storage is
+    replaced.  Every result against a single-stream runner launched from Python on the same layers."""
+    ta = _mods()
+    dtype = torch.float16
+    n_layers, E, H, Fd, L, B = 2, 256, 2, 1024, 128, 2
+    bs, ss = [1, 1], [32, 64, 32]
+    ps = make_params(n_layers, E, Fd, dtype, seed=33)
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    fast = ta.TeraPipe(layers, B, L, bs, ss)
+    plain = ta.TeraPipe(layers, B, L, bs, ss, slice_streams=1, launch_replay=False)
+
+    def data(seed):
+        g = torch.Generator().manual_seed(seed)
+        return (torch.randn(L, B, E, generator=g).to(dtype).to(DEV),
+                (torch.randn(L, B, E, generator=g) * 0.1).to(dtype).to(DEV))
+
+    def train(runner, x, dy, input_grad=True):
+        for p in layers.parameters():
+            p.grad = None
+        xd = x.clone().requires_grad_(input_grad)
+        y = runner(xd)
+        (y * dy).sum().backward()
+        return y.detach().clone(), (xd.grad.clone() if input_grad else None), [p.grad.clone() for p in layers.parameters()]
+
+    def same_train(seed, input_grad=True, tag=""):
+        x, dy = data(seed)
+        y0, dx0, g0 = train(plain, x, dy, input_grad)
+        y1, dx1, g1 = train(fast, x, dy, input_grad)
+        torch.cuda.synchronize()
+        assert torch.equal(y1, y0), tag + " y"
+        if input_grad:
+            assert torch.equal(dx1, dx0), tag + " dx"
+        for a, b in zip(g1, g0):
+            assert_close(a, b, dtype, tag + " parameter gradient", 1.0)
+
+    def same_eval(seed, tag=""):
+        x, _ = data(seed)
+        with torch.no_grad():
+            y0 = plain(x).clone()
+            y1 = fast(x).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(y1, y0), tag + " y (no_grad)"
+
+    same_eval(1, "eval before any training step")
+    same_train(2, tag="step 1")
+    same_eval(3, "eval after step 1")
+    same_train(4, tag="step 2 (recorded)")
+    same_eval(5, "eval after the recording")
+    same_train(6, tag="step 3 (re-issued)")
+    # a forward that is never differentiated, then a full step
+    x, _ = data(7)
+    y = fast(x.clone().requires_grad_(True))
+    del y
+    same_train(8, tag="step after an abandoned forward")
+    same_train(9, input_grad=False, tag="input without gradient")
+    same_train(10, tag="input with gradient again")
+    with torch.no_grad():
+        for p in layers.parameters():
+            p.add_(torch.randn_like(p) * 1e-3)
+    same_train(11, tag="after an in-place update")
+    # a parameter that moves to new storage (e.g. a checkpoint load that rebinds .data)
+    p0 = next(iter(layers.parameters()))
+    p0.data = p0.data.clone()
+    same_train(12, tag="after a parameter moved")
+    same_train(13, tag="second step after the move")
+    same_eval(14, "eval at the end")
+
+
 def test_backward_of_an_overwritten_forward_raises():
     ta = _mods()
     dtype = torch.float16
