@@ -138,6 +138,14 @@ typedef struct tp_gemm_desc {
 int tp_gemm_splits(const tp_gemm_desc* d);
 size_t tp_gemm_workspace_bytes(const tp_gemm_desc* d);
 int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_bytes, void* stream);
+/* n independent products as if by n tp_gemm calls in order on the stream (the four weight gradients of a layer,
+   which autograd's backward of the four linears of transformer_models.py:273-285 produces one by one).  Up to four
+   16-bit TP_GEMM_TN products of one dtype, k a multiple of 64, whose largest plans to 256 x 256 tiles with unsplit
+   k share ONE launch, so that together they fill whole rounds of the chip's CUs; any other group runs member by
+   member.  workspace: the largest member's tp_gemm_workspace_bytes. */
+int tp_gemm_grouped(const tp_gemm_desc* descs, int n, void* workspace, size_t workspace_bytes, void* stream);
+/* the tile configuration of the single launch tp_gemm_grouped makes for this group; 0 = member by member */
+int tp_gemm_group_cfg(const tp_gemm_desc* descs, int n);
 
 /* ------------------------------------------------------------------------------------------------
  * Prefix-cached causal attention (attn_helper, transformer_models.py:235-245, with the mask of :220

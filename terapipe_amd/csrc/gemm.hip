@@ -26,6 +26,16 @@ struct GemmArgs {
     float* partial;  // [nsplit][M][N] fp32 when nsplit > 1
 };
 
+// Several GEMMs of one tile configuration in one launch (unsplit k): workgroup w works on tile
+// w - first_tile[p] of problem p, the last p whose first_tile is <= w.
+constexpr int kGroupMax = 4;
+struct GemmGroupArgs {
+    GemmArgs g[kGroupMax];
+    int first_tile[kGroupMax];
+    int tiles_x[kGroupMax];
+    int n;
+};
+
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
 __device__ __forceinline__ float gelu_erf_grad(float z) {
     float cdf = 0.5f * (1.0f + erff(z * 0.70710678118654752f));
@@ -359,8 +369,32 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_dma_kernel(GemmArgs a) {
 // Tiles are loaded with ClampTileDma (whole k-tiles only) and the operand fetches of k-step s+1 are issued
 // before the MFMAs of k-step s.
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN, int STAGES>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_tall_kernel(GemmArgs a) {
+template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN, int STAGES, bool GROUPED = false>
+__global__ __launch_bounds__(WM * WN * 64)
+void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs>::type args) {
+    // which problem and which of its tiles (wave-uniform)
+    int prob = 0, tile_x = blockIdx.x, tile_y = blockIdx.y;
+    if constexpr (GROUPED) {
+        static_assert(kGroupMax == 4, "the selects below are written out for four problems");
+        int first = 0, tx = args.tiles_x[0];
+        if (1 < args.n && (int)blockIdx.x >= args.first_tile[1]) { prob = 1; first = args.first_tile[1]; tx = args.tiles_x[1]; }
+        if (2 < args.n && (int)blockIdx.x >= args.first_tile[2]) { prob = 2; first = args.first_tile[2]; tx = args.tiles_x[2]; }
+        if (3 < args.n && (int)blockIdx.x >= args.first_tile[3]) { prob = 3; first = args.first_tile[3]; tx = args.tiles_x[3]; }
+        const int t = (int)blockIdx.x - first;
+        tile_y = t / tx;
+        tile_x = t % tx;
+    }
+    // (constant indices only: a dynamically indexed kernel argument would be copied to scratch memory)
+    const GemmArgs a = [&]() -> GemmArgs {
+        if constexpr (GROUPED) {
+            if (prob == 1) return args.g[1];
+            if (prob == 2) return args.g[2];
+            if (prob == 3) return args.g[3];
+            return args.g[0];
+        } else {
+            return args;
+        }
+    }();
     typedef Elem<T> E;
     static_assert(sizeof(T) == 2, "16-bit only");
     constexpr int NT = WM * WN * 64;
@@ -381,7 +415,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tall_kernel(GemmArgs a) {
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave % WM, wn = wave / WM;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int m0 = tile_y * BM, n0 = tile_x * BN;
     const int kbeg = blockIdx.z * a.kper;
     const int kend = min(a.K, kbeg + a.kper);
     DA da;
@@ -880,16 +914,9 @@ extern "C" size_t tp_gemm_workspace_bytes(const tp_gemm_desc* d) {
     return p.nsplit > 1 ? (size_t)p.nsplit * d->M * d->N * sizeof(float) : 0;
 }
 
-extern "C" int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_bytes, void* stream) {
-    int rc = tp::validate_gemm(d);
-    if (rc != TP_OK) return rc;
-    tp::GemmPlan p = tp::plan_gemm(d);
-    size_t need = p.nsplit > 1 ? (size_t)p.nsplit * d->M * d->N * sizeof(float) : 0;
-    if (need > 0 && (!workspace || workspace_bytes < need)) {
-        tp::set_error("tp_gemm: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-        return TP_ERR_WORKSPACE;
-    }
-    tp::GemmArgs a;
+namespace tp {
+static GemmArgs fill_args(const tp_gemm_desc* d, const GemmPlan& p, void* workspace) {
+    GemmArgs a;
     a.A = d->A; a.B = d->B; a.C = d->C;
     a.lda = d->lda; a.ldb = d->ldb; a.ldc = d->ldc;
     a.M = d->M; a.N = d->N; a.K = d->K;
@@ -903,6 +930,61 @@ extern "C" int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_
     a.q_rows = d->q_bh_rows > 0 ? d->q_bh_rows : a.T;
     a.P = d->cache_len; a.cache_rows = d->cache_rows; a.qscale = d->q_scale;
     a.kper = p.kper; a.nsplit = p.nsplit; a.partial = reinterpret_cast<float*>(workspace);
+    return a;
+}
+
+// One launch for the whole group when every member is a 16-bit TN product (parameter gradients) of the same dtype
+// whose k is a whole number of 64-wide tiles and the group's largest member plans to a 256 x 256 tile with
+// unsplit k.
+// The tile configuration of the single launch that runs the group, or 0 when it runs member by member.
+static int group_cfg(const tp_gemm_desc* descs, int n) {
+    if (n < 2 || n > kGroupMax) return 0;
+    int big = 0;
+    for (int i = 0; i < n; ++i) {
+        const tp_gemm_desc& d = descs[i];
+        if (d.op != TP_GEMM_TN || d.dtype != descs[0].dtype || d.dtype == TP_F32 || d.K % 64 != 0 || d.reserved != 0 ||
+            d.defer_reduce != 0 || d.epilogue == TP_EPI_QKV_SCATTER)
+            return 0;
+        if ((double)d.M * d.N > (double)descs[big].M * descs[big].N) big = i;
+    }
+    const GemmPlan pb = plan_gemm(&descs[big]);
+    return ((pb.cfg == 19 || pb.cfg == 20) && pb.nsplit == 1) ? pb.cfg : 0;
+}
+
+template <typename T>
+static void launch_group(const tp_gemm_desc* descs, int n, int cfg, hipStream_t s) {
+    constexpr bool AKM = false, BKM = false;     // TN: both operands token-major
+    GemmPlan pb;
+    pb.cfg = cfg;
+    GemmGroupArgs ga;
+    int tiles = 0;
+    for (int i = 0; i < n; ++i) {
+        GemmPlan p = pb;
+        p.gx = (descs[i].N + kCfgs[pb.cfg].bn - 1) / kCfgs[pb.cfg].bn;
+        p.gy = (descs[i].M + kCfgs[pb.cfg].bm - 1) / kCfgs[pb.cfg].bm;
+        p.kper = descs[i].K; p.nsplit = 1;
+        ga.g[i] = fill_args(&descs[i], p, nullptr);
+        ga.first_tile[i] = tiles;
+        ga.tiles_x[i] = p.gx;
+        tiles += p.gx * p.gy;
+    }
+    for (int i = n; i < kGroupMax; ++i) { ga.g[i] = ga.g[0]; ga.first_tile[i] = tiles; ga.tiles_x[i] = 1; }
+    ga.n = n;
+    if (pb.cfg == 19) gemm_tall_kernel<T, AKM, BKM, 256, 256, 64, 4, 2, 2, true><<<dim3(tiles), 512, 0, s>>>(ga);
+    else gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4, true><<<dim3(tiles), 512, 0, s>>>(ga);
+}
+}  // namespace tp
+
+extern "C" int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = tp::validate_gemm(d);
+    if (rc != TP_OK) return rc;
+    tp::GemmPlan p = tp::plan_gemm(d);
+    size_t need = p.nsplit > 1 ? (size_t)p.nsplit * d->M * d->N * sizeof(float) : 0;
+    if (need > 0 && (!workspace || workspace_bytes < need)) {
+        tp::set_error("tp_gemm: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+        return TP_ERR_WORKSPACE;
+    }
+    tp::GemmArgs a = tp::fill_args(d, p, workspace);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     switch (d->dtype) {
     case TP_F32: tp::launch_gemm<float>(d, p, a, s); break;
@@ -911,5 +993,34 @@ extern "C" int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { tp::set_error("tp_gemm: launch failed: %s", hipGetErrorString(e)); return TP_ERR_LAUNCH; }
+    return TP_OK;
+}
+
+extern "C" int tp_gemm_group_cfg(const tp_gemm_desc* descs, int n) {
+    if (!descs || n < 1) return 0;
+    for (int i = 0; i < n; ++i)
+        if (tp::validate_gemm(&descs[i]) != TP_OK) return 0;
+    return tp::group_cfg(descs, n);
+}
+
+extern "C" int tp_gemm_grouped(const tp_gemm_desc* descs, int n, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!descs || n < 1) { tp::set_error("tp_gemm_grouped: bad argument"); return TP_ERR_ARG; }
+    for (int i = 0; i < n; ++i) {
+        int rc = tp::validate_gemm(&descs[i]);
+        if (rc != TP_OK) return rc;
+    }
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (const int cfg = tp::group_cfg(descs, n)) {
+        if (descs[0].dtype == TP_F16) tp::launch_group<tp::f16>(descs, n, cfg, s);
+        else tp::launch_group<tp::bf16>(descs, n, cfg, s);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) { tp::set_error("tp_gemm_grouped: launch failed: %s", hipGetErrorString(e)); return TP_ERR_LAUNCH; }
+        return TP_OK;
+    }
+    // any other group: its members one after the other (they share the workspace: same stream, in order)
+    for (int i = 0; i < n; ++i) {
+        int rc = tp_gemm(&descs[i], workspace, workspace_bytes, stream);
+        if (rc != TP_OK) return rc;
+    }
     return TP_OK;
 }

@@ -258,6 +258,37 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
     return C
 
 
+def gemm_grouped(items, desc_sinks=None):
+    """Plain products (epilogue STORE or ACCUMULATE) as one library call: items is a list of
+    (op, A, B, M, N, K, C, epilogue).  The library runs the group as one launch when its members allow it and
+    one after the other otherwise; the result is that of ``gemm`` on every item in order.
+    desc_sinks: per item a list (or None) that receives the item's descriptor, as ``gemm``'s desc_sink."""
+    n = len(items)
+    descs = (GemmDesc * n)()
+    lib = _lib.load()
+    need = 0
+    for i, (op, A, B, M, N, K, C, epilogue) in enumerate(items):
+        _require_cuda(A, B, C)
+        d = descs[i]                        # a view into the array
+        d.op, d.dtype, d.epilogue = op, tp_dtype(A.dtype), epilogue
+        d.M, d.N, d.K = M, N, K
+        d.A, d.lda = A.data_ptr(), A.stride(0)
+        d.B, d.ldb = B.data_ptr(), B.stride(0)
+        d.C, d.ldc = C.data_ptr(), C.stride(0)
+        if GEMM_PLAN_OVERRIDE and (op, M, N, K) in GEMM_PLAN_OVERRIDE:
+            tile_cfg, ksplit = GEMM_PLAN_OVERRIDE[(op, M, N, K)]
+            d.reserved = ((tile_cfg + 1) if tile_cfg is not None else 0) | ((ksplit or 0) << 8)
+        if desc_sinks is not None and desc_sinks[i] is not None:
+            desc_sinks[i].append(d)
+        need = max(need, lib.tp_gemm_workspace_bytes(ctypes.byref(d)))
+    ws = Workspace.get(need, items[0][1].device) if need else None
+    wsp, wsn = _p(ws), (ws.numel() if ws is not None else 0)
+    meta = tuple((op, M, N, K) for (op, _, _, M, N, K, _, _) in items)
+    with _timed("gemm", meta):
+        _lib.check(lib.tp_gemm_grouped(descs, n, wsp, wsn, _stream()), "tp_gemm_grouped")
+    _record("gemm", meta, lambda s=None: lib.tp_gemm_grouped(descs, n, wsp, wsn, _on(s)))
+
+
 def _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale, q_bh_rows=0,
                stat_bh_rows=0):
     """q_bh_rows / stat_bh_rows: rows per (batch, head) block of q / of lse and delta when these are views

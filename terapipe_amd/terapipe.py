@@ -380,12 +380,15 @@ def _param_grads_layer(runner, bufs, l):
         R = L * runner.batch_slices[bi]
         epi = TP_EPI_STORE if bi == 0 else TP_EPI_ACCUMULATE
         dy_out = pb["dx"][l + 1]
+        # the four weight gradients as one library call: together their tiles fill whole rounds of the CUs
+        items, sinks = [], []
         for name, dy, xin, n_out, n_in in (("attn.in_proj.weight", pb["dqkv"][l], pb["xn"][l], 3 * E, E),
                                            ("attn.out_proj.weight", pb["dh"][l], pb["o"][l], E, E),
                                            ("fc1.weight", pb["dz1"][l], pb["hn"][l], F, E),
                                            ("fc2.weight", dy_out, pb["a"][l], E, F)):
-            sink = bufs.wgrad_descs.setdefault((l, name), []) if bufs.recording else None
-            ops.gemm(TP_GEMM_TN, dy, xin, n_out, n_in, R, C=g[name], epilogue=epi, desc_sink=sink)
+            sinks.append(bufs.wgrad_descs.setdefault((l, name), []) if bufs.recording else None)
+            items.append((TP_GEMM_TN, dy, xin, n_out, n_in, R, g[name], epi))
+        ops.gemm_grouped(items, sinks)
         ops.colsum_acc(pb["dqkv"][l], sv["attn.in_proj.bias"])
         ops.colsum_acc(pb["dh"][l], sv["attn.out_proj.bias"])
         ops.colsum_acc(pb["dz1"][l], sv["fc1.bias"])

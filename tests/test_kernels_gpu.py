@@ -146,6 +146,88 @@ def test_gemm_every_tile_configuration(dtype, cfg):
             assert_close(acc, ref.sum(0), dtype, "colsum cfg %d split %d" % (cfg, ks))
 
 
+def _group(ops, L, items, dtype, force_cfg=None):
+    """Runs items [(op, A, B, M, N, K)] once through gemm_grouped and once one by one; returns both outputs."""
+    Cs_g = [torch.zeros(M, N, dtype=dtype, device=DEV) for (_, _, _, M, N, K) in items]
+    Cs_1 = [torch.zeros(M, N, dtype=dtype, device=DEV) for (_, _, _, M, N, K) in items]
+    ops.gemm_grouped([(op, A, B, M, N, K, C, L.TP_EPI_STORE) for (op, A, B, M, N, K), C in zip(items, Cs_g)])
+    for (op, A, B, M, N, K), C in zip(items, Cs_1):
+        ops.gemm(op, A, B, M, N, K, C=C, tile_cfg=force_cfg, ksplit=1 if force_cfg is not None else None)
+    return Cs_g, Cs_1
+
+
+def _group_cfg(L, items, dtype):
+    import ctypes
+    descs = (L.GemmDesc * len(items))()
+    for d, (op, A, B, M, N, K) in zip(descs, items):
+        d.op, d.dtype, d.epilogue, d.M, d.N, d.K = op, 1 if dtype == torch.float16 else 2, L.TP_EPI_STORE, M, N, K
+        d.A, d.lda, d.B, d.ldb, d.C, d.ldc = A.data_ptr(), A.stride(0), B.data_ptr(), B.stride(0), A.data_ptr(), N
+    return L.load().tp_gemm_group_cfg(descs, len(items))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_gemm_grouped_single_launch_matches_member_by_member(dtype):
+    """A layer's four weight-gradient products (hidden 2048, FFN 8192, 256 tokens), and a ragged group whose
+    extents end inside tiles, through tp_gemm_grouped: the library reports one launch of a 256 x 256 tile
+    configuration for them, and every output equals, bit for bit, the same product launched alone with that
+    tile configuration (same tiles, same k order) -- and the fp64 product to the 16-bit tolerance."""
+    ops = _ops()
+    from terapipe_amd import _lib as L
+    g = torch.Generator(device=DEV).manual_seed(77)
+
+    def rnd(r, c, sc=1.0):
+        return (torch.randn(r, c, generator=g, device=DEV) * sc).to(dtype)
+    E, Fd, R = 2048, 8192, 256
+    dys = [rnd(R, 3 * E, 0.1), rnd(R, E, 0.1), rnd(R, Fd, 0.1), rnd(R, E, 0.1)]
+    xs = [rnd(R, E), rnd(R, E), rnd(R, E), rnd(R, Fd)]
+    layer = [(L.TP_GEMM_TN, dy, x, dy.shape[1], x.shape[1], R) for dy, x in zip(dys, xs)]
+    ragged = [(L.TP_GEMM_TN, rnd(192, 1000, 0.1), rnd(192, 2000), 1000, 2000, 192),
+              (L.TP_GEMM_TN, rnd(192, 304, 0.1), rnd(192, 520), 304, 520, 192),
+              (L.TP_GEMM_TN, rnd(192, 3000, 0.1), rnd(192, 4504), 3000, 4504, 192)]
+    for tag, items in (("layer", layer), ("ragged", ragged)):
+        cfg = _group_cfg(L, items, dtype)
+        assert cfg in (19, 20), "%s: the group should run as one launch (got %d)" % (tag, cfg)
+        got, want = _group(ops, L, items, dtype, force_cfg=cfg)
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), "%s member %d differs from the product launched alone" % (tag, i)
+        op, A, B, M, N, K = items[-1]
+        ref = (A.double().t() @ B.double()) if op == L.TP_GEMM_TN else (A.double() @ B.double().t())
+        assert_close(got[-1], ref, dtype, tag + " against fp64")
+
+
+def test_gemm_grouped_falls_back_member_by_member():
+    """Groups the single launch does not cover (small products, a k that is not a multiple of 64, five members,
+    another operand layout) run member by member with the same results; the accumulate epilogue through the
+    single launch."""
+    ops = _ops()
+    from terapipe_amd import _lib as L
+    dtype = torch.float16
+    g = torch.Generator(device=DEV).manual_seed(78)
+
+    def rnd(r, c, sc=1.0):
+        return (torch.randn(r, c, generator=g, device=DEV) * sc).to(dtype)
+    small = [(L.TP_GEMM_TN, rnd(96, 256, 0.1), rnd(96, 512), 256, 512, 96),
+             (L.TP_GEMM_TN, rnd(96, 128, 0.1), rnd(96, 64), 128, 64, 96)]
+    odd_k = [(L.TP_GEMM_TN, rnd(200, 4096, 0.1), rnd(200, 4096), 4096, 4096, 200),
+             (L.TP_GEMM_TN, rnd(200, 512, 0.1), rnd(200, 512), 512, 512, 200)]
+    five = [(L.TP_GEMM_NT, rnd(64, 256), rnd(128, 256, 0.1), 64, 128, 256) for _ in range(5)]
+    nt = [(L.TP_GEMM_NT, rnd(4096, 128), rnd(4096, 128, 0.1), 4096, 4096, 128),
+          (L.TP_GEMM_NT, rnd(520, 128), rnd(264, 128, 0.1), 520, 264, 128)]
+    for tag, items in (("small", small), ("odd k", odd_k), ("five", five), ("not TN", nt)):
+        assert _group_cfg(L, items, dtype) == 0, tag
+        got, want = _group(ops, L, items, dtype)
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), "%s member %d" % (tag, i)
+    # accumulate epilogue through the grouped launch: C += product
+    items = [(L.TP_GEMM_TN, rnd(128, 4096, 0.1), rnd(128, 4096), 4096, 4096, 128),
+             (L.TP_GEMM_TN, rnd(128, 512, 0.1), rnd(128, 768), 512, 768, 128)]
+    assert _group_cfg(L, items, dtype) in (19, 20)
+    Cs = [torch.ones(M, N, dtype=dtype, device=DEV) for (_, _, _, M, N, K) in items]
+    ops.gemm_grouped([(op, A, B, M, N, K, C, L.TP_EPI_ACCUMULATE) for (op, A, B, M, N, K), C in zip(items, Cs)])
+    for (op, A, B, M, N, K), C in zip(items, Cs):
+        assert_close(C, 1.0 + A.double().t() @ B.double(), dtype, "accumulate")
+
+
 def _tuned_entries():
     import os
     import re
