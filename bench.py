@@ -27,9 +27,9 @@ PEAK_MFMA_16BIT = 2.5e15     # dense fp16/bf16 MFMA flop/s
 PEAK_MFMA_FP32 = 157.3e12
 PEAK_HBM = 8.0e12            # bytes/s
 
-# HBM bytes per tp_gemm call (FETCH_SIZE + WRITE_SIZE of the GEMM kernels of one step / calls), from the two
+# HBM bytes per GEMM call (FETCH_SIZE + WRITE_SIZE of the GEMM kernels of one step / calls), from the two
 # rocprofv3 --pmc runs summarised in profiles/bench_C2_gemm_hbm_traffic.pmc.txt; only measured for C2
-PMC_GEMM_TRAFFIC_BYTES = {"C2": 31.38e6}
+PMC_GEMM_TRAFFIC_BYTES = {"C2": 32.86e6}
 
 WORKLOADS = {
     # name: layers, hidden, heads, ffn, seq, batch, dtype, slices, weight std
@@ -269,7 +269,7 @@ def main():
         peak = PEAK_MFMA_FP32 if w["dtype"] == "f32" else PEAK_MFMA_16BIT
         achieved = flops / (g_ms * 1e-3) if g_ms > 0 else 0.0
         out["roofline"] = {
-            "kernel": "tp::gemm_dma_kernel / tp::gemm_kernel (all NT/NN/TN launches of one step, split-K reduce included)",
+            "kernel": "tp::gemm_dma_kernel / tp::gemm_tall_kernel (all NT/NN/TN launches of one step, split-K reduce included)",
             "bound": "mfma", "achieved": achieved / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
             "frac": achieved / peak, "traffic": PMC_GEMM_TRAFFIC_BYTES.get(args.workload),
             "launches": g_calls, "avg_launch_us": g_ms * 1e3 / max(g_calls, 1),
