@@ -70,6 +70,119 @@ __global__ __launch_bounds__(1024) void cross_entropy_kernel(T* __restrict__ log
     }
 }
 
+// The same with 16-byte accesses (rows 16-byte aligned, Vpad a whole number of chunks): the row is read from
+// HBM once for the maximum, the two later passes find it in the caches, and the gradient goes out in
+// 16-byte stores.
+template <typename T>
+__global__ __launch_bounds__(1024) void cross_entropy_vec_kernel(T* __restrict__ logits, long ld, const int64_t* __restrict__ target,
+                                                                 float* __restrict__ loss, int V, int Vpad, float grad_scale) {
+    constexpr int CH = 16 / sizeof(T);
+    __shared__ float scratch[16];
+    const long m = blockIdx.x;
+    T* z = logits + m * ld;
+    const uint4* zv = reinterpret_cast<const uint4*>(z);
+    const int nch = Vpad / CH;
+    float mx = -INFINITY;
+    for (int c = threadIdx.x; c < nch; c += blockDim.x) {
+        const uint4 raw = zv[c];
+        const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+        for (int i = 0; i < CH; ++i)
+            if (c * CH + i < V) mx = fmaxf(mx, Elem<T>::to_float(e[i]));
+    }
+    mx = block_reduce(mx, scratch, true);
+    float s = 0.f;
+    for (int c = threadIdx.x; c < nch; c += blockDim.x) {
+        const uint4 raw = zv[c];
+        const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+        for (int i = 0; i < CH; ++i)
+            if (c * CH + i < V) s += expf(Elem<T>::to_float(e[i]) - mx);
+    }
+    s = block_reduce(s, scratch, false);
+    const int64_t t = target[m];
+    const bool tok = t >= 0 && t < V;
+    if (threadIdx.x == 0) loss[m] = logf(s) + mx - (tok ? Elem<T>::to_float(z[t]) : 0.f);
+    __syncthreads();        // z[t] is read above before any thread overwrites it
+    const float inv = 1.0f / s;
+    for (int c = threadIdx.x; c < nch; c += blockDim.x) {
+        const uint4 raw = zv[c];
+        const T* e = reinterpret_cast<const T*>(&raw);
+        uint4 outv;
+        T* o = reinterpret_cast<T*>(&outv);
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            const int v = c * CH + i;
+            float g = 0.f;
+            if (v < V) g = (expf(Elem<T>::to_float(e[i]) - mx) * inv - ((tok && v == t) ? 1.f : 0.f)) * grad_scale;
+            o[i] = Elem<T>::from_float(g);
+        }
+        reinterpret_cast<uint4*>(z)[c] = outv;
+    }
+}
+
+// Rows of up to 1024 * NCH chunks (65536 columns): the row is read once into registers (NCH 16-byte chunks per
+// lane), maximum, sum and gradient are taken from there -- one read and one write of the logits in all.
+template <typename T, int NCH>
+__global__ __launch_bounds__(1024) void cross_entropy_reg_kernel(T* __restrict__ logits, long ld, const int64_t* __restrict__ target,
+                                                                 float* __restrict__ loss, int V, int Vpad, float grad_scale) {
+    constexpr int CH = 16 / sizeof(T);
+    __shared__ float scratch[16];
+    const long m = blockIdx.x;
+    T* z = logits + m * ld;
+    const uint4* zv = reinterpret_cast<const uint4*>(z);
+    const int nch = Vpad / CH;
+    const int64_t t = target[m];
+    const bool tok = t >= 0 && t < V;
+    const float zt = tok ? Elem<T>::to_float(z[t]) : 0.f;      // read before anything is overwritten
+    // (the row stays in its 16-bit / fp32 form: 8 chunks are 32 registers, which keeps two workgroups on a CU;
+    // holding exp(z - max) as floats instead costs 64 registers, one workgroup per CU and 1.5x the time)
+    uint4 row[NCH];
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int c = k * 1024 + threadIdx.x;
+        row[k] = c < nch ? zv[c] : make_uint4(0, 0, 0, 0);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const T* e = reinterpret_cast<const T*>(&row[k]);
+        const int v0 = (k * 1024 + threadIdx.x) * CH;
+#pragma unroll
+        for (int i = 0; i < CH; ++i)
+            if (v0 + i < V) mx = fmaxf(mx, Elem<T>::to_float(e[i]));
+    }
+    mx = block_reduce(mx, scratch, true);
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const T* e = reinterpret_cast<const T*>(&row[k]);
+        const int v0 = (k * 1024 + threadIdx.x) * CH;
+#pragma unroll
+        for (int i = 0; i < CH; ++i)
+            if (v0 + i < V) s += expf(Elem<T>::to_float(e[i]) - mx);
+    }
+    s = block_reduce(s, scratch, false);
+    if (threadIdx.x == 0) loss[m] = logf(s) + mx - zt;
+    const float inv = 1.0f / s;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int c = k * 1024 + threadIdx.x;
+        if (c >= nch) continue;
+        const T* e = reinterpret_cast<const T*>(&row[k]);
+        uint4 outv;
+        T* o = reinterpret_cast<T*>(&outv);
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            const int v = c * CH + i;
+            float g = 0.f;
+            if (v < V) g = (expf(Elem<T>::to_float(e[i]) - mx) * inv - ((tok && v == t) ? 1.f : 0.f)) * grad_scale;
+            o[i] = Elem<T>::from_float(g);
+        }
+        reinterpret_cast<uint4*>(z)[c] = outv;
+    }
+}
+
 // x[m, :n] *= scale[m] in place (grad_input.mul_(grad_output.unsqueeze(-1)), mpu/cross_entropy.py:97)
 template <typename T>
 __global__ __launch_bounds__(256) void scale_rows_kernel(T* __restrict__ x, long ld, const float* __restrict__ scale, int n) {
@@ -123,6 +236,27 @@ extern "C" int tp_cross_entropy(void* logits, int64_t ld, const int64_t* target,
     if (!logits || !target || !loss || M <= 0 || V <= 0 || Vpad < V || ld < Vpad) { set_error("tp_cross_entropy: bad argument (M=%d V=%d Vpad=%d ld=%ld)", M, V, Vpad, (long)ld); return TP_ERR_ARG; }
     if (dtype < TP_F32 || dtype > TP_BF16) { set_error("tp_cross_entropy: bad dtype %d", dtype); return TP_ERR_ARG; }
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const int ch = dtype == TP_F32 ? 4 : 8;
+    if (Vpad % ch == 0 && ld % ch == 0 && ((uintptr_t)logits & 15) == 0) {
+        if (Vpad / ch <= 1024 * 8) {
+            switch (dtype) {
+            case TP_F32: cross_entropy_reg_kernel<float, 8><<<M, 1024, 0, s>>>((float*)logits, ld, target, loss, V, Vpad, grad_scale); break;
+            case TP_F16: cross_entropy_reg_kernel<f16, 8><<<M, 1024, 0, s>>>((f16*)logits, ld, target, loss, V, Vpad, grad_scale); break;
+            default: cross_entropy_reg_kernel<bf16, 8><<<M, 1024, 0, s>>>((bf16*)logits, ld, target, loss, V, Vpad, grad_scale); break;
+            }
+            return vocab_status("tp_cross_entropy");
+        }
+        if (dtype == TP_F32 && Vpad / ch <= 1024 * 16) {
+            cross_entropy_reg_kernel<float, 16><<<M, 1024, 0, s>>>((float*)logits, ld, target, loss, V, Vpad, grad_scale);
+            return vocab_status("tp_cross_entropy");
+        }
+        switch (dtype) {
+        case TP_F32: cross_entropy_vec_kernel<float><<<M, 1024, 0, s>>>((float*)logits, ld, target, loss, V, Vpad, grad_scale); break;
+        case TP_F16: cross_entropy_vec_kernel<f16><<<M, 1024, 0, s>>>((f16*)logits, ld, target, loss, V, Vpad, grad_scale); break;
+        default: cross_entropy_vec_kernel<bf16><<<M, 1024, 0, s>>>((bf16*)logits, ld, target, loss, V, Vpad, grad_scale); break;
+        }
+        return vocab_status("tp_cross_entropy");
+    }
     switch (dtype) {
     case TP_F32: cross_entropy_kernel<float><<<M, 1024, 0, s>>>((float*)logits, ld, target, loss, V, Vpad, grad_scale); break;
     case TP_F16: cross_entropy_kernel<f16><<<M, 1024, 0, s>>>((f16*)logits, ld, target, loss, V, Vpad, grad_scale); break;

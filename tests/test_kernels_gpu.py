@@ -548,6 +548,41 @@ def test_embedding_lm_head_cross_entropy(dtype, M, E, V):
     assert (emb(bad.to(DEV))[3] == 0).all()
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_cross_entropy_vector_and_scalar_paths(dtype):
+    """tp_cross_entropy on rows that allow 16-byte accesses (short enough to be held in registers, and longer
+    ones) and on rows that do not (odd leading dimension, a padded width that is not a whole number of
+    chunks): loss, in-place gradient (softmax - onehot) * scale,
+    zeroed padding columns, and a target outside the vocabulary (no onehot, loss without the target term)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(5)
+    for (M, V, Vpad, ld) in [(9, 50257, 50264, 50264), (9, 50257, 50264, 50265), (5, 1003, 1003, 1003),
+                             (6, 1000, 1008, 1024), (3, 7, 8, 8), (3, 70001, 70008, 70008)]:
+        z = _rnd((M, V), dtype, g, 3.0)
+        tgt = torch.randint(0, V, (M,), generator=g)
+        tgt[0] = V - 1
+        tgt[1] = V + 3                                   # outside: as a masked target
+        buf = torch.full((M, ld), 7.0, dtype=dtype, device=DEV)
+        buf[:, :V] = z.to(DEV)
+        view = buf[:, :Vpad]
+        loss = ops.cross_entropy_(view, tgt.to(DEV), V, grad_scale=0.5)
+        z64 = z.double()
+        lse = torch.logsumexp(z64, dim=1)
+        inside = tgt < V
+        want_loss = lse - torch.where(inside, z64.gather(1, tgt.clamp(max=V - 1)[:, None])[:, 0], torch.zeros(M, dtype=torch.float64))
+        want_grad = torch.softmax(z64, dim=1)
+        for m in range(M):
+            if inside[m]:
+                want_grad[m, tgt[m]] -= 1.0
+        want_grad *= 0.5
+        tag = "M=%d V=%d Vpad=%d ld=%d" % (M, V, Vpad, ld)
+        assert_close(loss, want_loss, torch.float32 if dtype == torch.float32 else dtype, tag + " loss",
+                     10 if dtype == torch.float32 else 1)
+        assert_close(buf[:, :V], want_grad, dtype, tag + " gradient", 10 if dtype == torch.float32 else 1)
+        assert (buf[:, V:Vpad] == 0).all(), tag + " padding columns"
+        assert (buf[:, Vpad:] == 7.0).all(), tag + " columns beyond the padded width are not touched"
+
+
 def test_error_paths():
     """Bad arguments come back as status codes with a message; nothing is launched."""
     import ctypes
