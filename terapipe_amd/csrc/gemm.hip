@@ -756,6 +756,7 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     const long t64 = (long)((d->M + 63) / 64) * ((d->N + 63) / 64);
     int cfg, ns = 1;
     const long t256n = (d->N + 255) / 256;
+    const long t256 = (long)((d->M + 255) / 256) * t256n;
     if (d->M <= 64 && (long)d->N * d->K >= (64L << 20)) {
         // a short activation against a large weight: 64 x 256 x 64 tiles stream the weight with a quarter
         // of the activation re-reads of 64-wide tiles; k is split to about 200 workgroups
@@ -771,10 +772,19 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
         int maxs = d->K / 2048;
         if (ns > maxs) ns = maxs;
         if (ns > 8) ns = 8;
-    } else if (d->op == TP_GEMM_TN && d->K % 64 == 0 && (long)((d->M + 255) / 256) * ((d->N + 255) / 256) >= 192) {
-        // parameter gradients of a whole step: 256 x 256 tiles by eight waves (half the bytes per flop of a
-        // 128 x 128 tile through the 64 B/clk vector-memory path into LDS)
+    } else if ((d->op == TP_GEMM_TN || d->M >= 512) && d->K % 64 == 0 && t256 >= 192) {
+        // parameter gradients of a whole step, and any product of 512 rows or more with that many tiles (the LM
+        // head): 256 x 256 tiles by eight waves (half the bytes per flop of a 128 x 128 tile through the
+        // 64 B/clk vector-memory path into LDS)
         cfg = 19;
+    } else if (d->op != TP_GEMM_TN && d->M >= 512 && d->K % 64 == 0 && t256 >= 48 && d->K >= 8192) {
+        // the same tiles on a long k with too few of them for the chip (the LM head's data gradient, k =
+        // vocabulary): k is split to about one workgroup per CU
+        cfg = 19;
+        ns = (int)((256 + t256 - 1) / t256);
+        int maxs = d->K / 2048;
+        if (ns > maxs) ns = maxs;
+        if (ns > 8) ns = 8;
     } else if (t128 >= 144) {
         // short activations: the deeper ring keeps the weight stream going; parameter gradients (both
         // operands fetched with transpose reads): 128 x 128 x 32, four stages, two workgroups per CU

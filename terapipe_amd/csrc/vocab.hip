@@ -192,6 +192,22 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(T* __restrict__ x, long
     if (v < n) x[m * ld + v] = Elem<T>::from_float(Elem<T>::to_float(x[m * ld + v]) * sc);
 }
 
+// the same with 16-byte accesses (rows 16-byte aligned, n a whole number of chunks)
+template <typename T>
+__global__ __launch_bounds__(256) void scale_rows_vec_kernel(T* __restrict__ x, long ld, const float* __restrict__ scale, int nch) {
+    constexpr int CH = 16 / sizeof(T);
+    const long m = blockIdx.y;
+    const float sc = scale[m];
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= nch) return;
+    uint4* p = reinterpret_cast<uint4*>(x + m * ld) + c;
+    uint4 raw = *p;
+    T* e = reinterpret_cast<T*>(&raw);
+#pragma unroll
+    for (int i = 0; i < CH; ++i) e[i] = Elem<T>::from_float(Elem<T>::to_float(e[i]) * sc);
+    *p = raw;
+}
+
 static int vocab_status(const char* what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("%s: launch failed: %s", what, hipGetErrorString(e)); return TP_ERR_LAUNCH; }
@@ -270,6 +286,17 @@ extern "C" int tp_scale_rows(void* x, int64_t ld, const float* scale, int M, int
     if (!x || !scale || M <= 0 || N <= 0 || ld < N) { set_error("tp_scale_rows: bad argument"); return TP_ERR_ARG; }
     if (dtype < TP_F32 || dtype > TP_BF16) { set_error("tp_scale_rows: bad dtype %d", dtype); return TP_ERR_ARG; }
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const int ch = dtype == TP_F32 ? 4 : 8;
+    if (N % ch == 0 && ld % ch == 0 && ((uintptr_t)x & 15) == 0) {
+        const int nch = N / ch;
+        dim3 vgrid((nch + 255) / 256, M);
+        switch (dtype) {
+        case TP_F32: scale_rows_vec_kernel<float><<<vgrid, 256, 0, s>>>((float*)x, ld, scale, nch); break;
+        case TP_F16: scale_rows_vec_kernel<f16><<<vgrid, 256, 0, s>>>((f16*)x, ld, scale, nch); break;
+        default: scale_rows_vec_kernel<bf16><<<vgrid, 256, 0, s>>>((bf16*)x, ld, scale, nch); break;
+        }
+        return vocab_status("tp_scale_rows");
+    }
     dim3 grid((N + 255) / 256, M);
     switch (dtype) {
     case TP_F32: scale_rows_kernel<float><<<grid, 256, 0, s>>>((float*)x, ld, scale, N); break;

@@ -51,18 +51,21 @@ class VocabParallelEmbedding(nn.Module):
         return _EmbeddingFunction.apply(input_, self.weight)
 
 
-def _pad8(n):
-    return (n + 7) // 8 * 8
+VOCAB_PAD = 64      # the 256-row GEMM tiles take whole 64-wide k-tiles: the data-gradient GEMM has k = vocabulary
+
+
+def _pad_vocab(n):
+    return (n + VOCAB_PAD - 1) // VOCAB_PAD * VOCAB_PAD
 
 
 class _LMHeadFunction(torch.autograd.Function):
-    """logits = h W^T with the vocabulary padded to a multiple of 8 columns for the GEMM (the padding rows
+    """logits = h W^T with the vocabulary padded to a multiple of 64 columns for the GEMMs (the padding rows
     of the weight copy are zero; the padding columns of the logits are ignored by the loss)."""
 
     @staticmethod
     def forward(ctx, h2d, weight):
         V, E = weight.shape
-        Vp = _pad8(V)
+        Vp = _pad_vocab(V)
         wp = weight
         if Vp != V:
             wp = torch.zeros(Vp, E, dtype=weight.dtype, device=weight.device)
@@ -88,7 +91,7 @@ class _LMHeadFunction(torch.autograd.Function):
 
 
 def lm_head_logits(h2d, weight):
-    """[M, E] x [V, E]^T -> [M, pad8(V)]; columns >= V are padding (see vocab_parallel_cross_entropy's
+    """[M, E] x [V, E]^T -> [M, V rounded up to a multiple of 64]; columns >= V are padding (see vocab_parallel_cross_entropy's
     `vocab_size`).  The usual GPT weight tying passes the embedding weight."""
     return _LMHeadFunction.apply(h2d, weight)
 

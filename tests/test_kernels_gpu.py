@@ -531,7 +531,7 @@ def test_embedding_lm_head_cross_entropy(dtype, M, E, V):
         emb.weight.copy_(W.to(DEV))
     x = emb(ids.to(DEV))
     logits = ta.lm_head_logits(x.view(M, E), emb.weight)
-    assert logits.shape == (M, (V + 7) // 8 * 8)
+    assert logits.shape == (M, (V + 63) // 64 * 64)
     loss = ta.vocab_parallel_cross_entropy(logits, tgt.to(DEV), vocab_size=V)
     scale = _rnd((M,), torch.float32, g).abs() + 0.5
     (loss * scale.to(DEV)).sum().backward()
@@ -581,6 +581,23 @@ def test_cross_entropy_vector_and_scalar_paths(dtype):
         assert_close(buf[:, :V], want_grad, dtype, tag + " gradient", 10 if dtype == torch.float32 else 1)
         assert (buf[:, V:Vpad] == 0).all(), tag + " padding columns"
         assert (buf[:, Vpad:] == 7.0).all(), tag + " columns beyond the padded width are not touched"
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_scale_rows_vector_and_scalar_paths(dtype):
+    """tp_scale_rows (x[m, :] *= scale[m]) on rows that allow 16-byte accesses and on rows that do not; columns
+    beyond the given width stay as they were."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(6)
+    for (M, N, ld) in [(5, 1024, 1024), (5, 1000, 1032), (4, 1003, 1003), (3, 64, 65)]:
+        x = _rnd((M, ld), dtype, g)
+        sc = _rnd((M,), torch.float32, g)
+        buf = x.to(DEV).clone()
+        ops.scale_rows_(buf[:, :N], sc.to(DEV))
+        want = x.double().clone()
+        want[:, :N] *= sc.double()[:, None]
+        assert_close(buf, want, dtype, "M=%d N=%d ld=%d" % (M, N, ld))
+        assert torch.equal(buf[:, N:].cpu(), x[:, N:])
 
 
 def test_error_paths():
