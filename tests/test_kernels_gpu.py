@@ -146,6 +146,33 @@ def test_gemm_every_tile_configuration(dtype, cfg):
             assert_close(acc, ref.sum(0), dtype, "colsum cfg %d split %d" % (cfg, ks))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_gemm_large_products_take_the_tall_tiles(dtype):
+    """Products of 512 rows and more that the plan gives to the 256 x 256 tiles on its own (the LM head's
+    shapes in small): many tiles with unsplit k, and few tiles on a long k that is split -- ragged extents,
+    against the fp64 product."""
+    ops = _ops()
+    from terapipe_amd import _lib as L
+    g = torch.Generator(device=DEV).manual_seed(91)
+
+    def rnd(r, c, sc=1.0):
+        return (torch.randn(r, c, generator=g, device=DEV) * sc).to(dtype)
+    # NT, 4 x 50 tiles, unsplit
+    A, B = rnd(1000, 192), rnd(12600, 192, 0.1)
+    C = torch.empty(1000, 12600, dtype=dtype, device=DEV)
+    ops.gemm(L.TP_GEMM_NT, A, B, 1000, 12600, 192, C=C)
+    assert_close(C, A.double() @ B.double().t(), dtype, "NT 1000x12600x192")
+    # NN, 4 x 13 tiles, k = 8256 split four ways
+    A, B = rnd(1000, 8256), rnd(8256, 3104, 0.02)
+    d = L.GemmDesc()
+    d.op, d.dtype, d.epilogue, d.M, d.N, d.K = L.TP_GEMM_NN, ops.tp_dtype(dtype), L.TP_EPI_STORE, 1000, 3104, 8256
+    d.A, d.lda, d.B, d.ldb, d.C, d.ldc = A.data_ptr(), 8256, B.data_ptr(), 3104, A.data_ptr(), 3104
+    assert L.load().tp_gemm_splits(d) == 4
+    C = torch.empty(1000, 3104, dtype=dtype, device=DEV)
+    ops.gemm(L.TP_GEMM_NN, A, B, 1000, 3104, 8256, C=C)
+    assert_close(C, A.double() @ B.double(), dtype, "NN 1000x3104x8256")
+
+
 def _group(ops, L, items, dtype, force_cfg=None):
     """Runs items [(op, A, B, M, N, K)] once through gemm_grouped and once one by one; returns both outputs."""
     Cs_g = [torch.zeros(M, N, dtype=dtype, device=DEV) for (_, _, _, M, N, K) in items]
