@@ -964,14 +964,13 @@ static int group_cfg(const tp_gemm_desc* descs, int n) {
 template <typename T>
 static void launch_group(const tp_gemm_desc* descs, int n, int cfg, hipStream_t s) {
     constexpr bool AKM = false, BKM = false;     // TN: both operands token-major
-    GemmPlan pb;
-    pb.cfg = cfg;
     GemmGroupArgs ga;
     int tiles = 0;
     for (int i = 0; i < n; ++i) {
-        GemmPlan p = pb;
-        p.gx = (descs[i].N + kCfgs[pb.cfg].bn - 1) / kCfgs[pb.cfg].bn;
-        p.gy = (descs[i].M + kCfgs[pb.cfg].bm - 1) / kCfgs[pb.cfg].bm;
+        GemmPlan p;                 // every member on the group's tiles, its whole k in one piece
+        p.cfg = cfg;
+        p.gx = (descs[i].N + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn;
+        p.gy = (descs[i].M + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm;
         p.kper = descs[i].K; p.nsplit = 1;
         ga.g[i] = fill_args(&descs[i], p, nullptr);
         ga.first_tile[i] = tiles;
@@ -980,7 +979,7 @@ static void launch_group(const tp_gemm_desc* descs, int n, int cfg, hipStream_t 
     }
     for (int i = n; i < kGroupMax; ++i) { ga.g[i] = ga.g[0]; ga.first_tile[i] = tiles; ga.tiles_x[i] = 1; }
     ga.n = n;
-    if (pb.cfg == 19) gemm_tall_kernel<T, AKM, BKM, 256, 256, 64, 4, 2, 2, true><<<dim3(tiles), 512, 0, s>>>(ga);
+    if (cfg == 19) gemm_tall_kernel<T, AKM, BKM, 256, 256, 64, 4, 2, 2, true><<<dim3(tiles), 512, 0, s>>>(ga);
     else gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4, true><<<dim3(tiles), 512, 0, s>>>(ga);
 }
 }  // namespace tp
