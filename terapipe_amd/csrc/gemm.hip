@@ -26,13 +26,14 @@ struct GemmArgs {
     float* partial;  // [nsplit][M][N] fp32 when nsplit > 1
 };
 
-// Several GEMMs of one tile configuration in one launch (unsplit k): workgroup w works on tile
-// w - first_tile[p] of problem p, the last p whose first_tile is <= w.
+// Several GEMMs of one tile configuration in one launch (unsplit k): workgroup w works on one of the
+// tiles_x[p] x tiles_y[p] tiles of problem p, the last p whose first_tile is <= w.
 constexpr int kGroupMax = 4;
 struct GemmGroupArgs {
     GemmArgs g[kGroupMax];
     int first_tile[kGroupMax];
     int tiles_x[kGroupMax];
+    int tiles_y[kGroupMax];
     int n;
 };
 
@@ -369,6 +370,22 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_dma_kernel(GemmArgs a) {
 // Tiles are loaded with ClampTileDma (whole k-tiles only) and the operand fetches of k-step s+1 are issued
 // before the MFMAs of k-step s.
 // ---------------------------------------------------------------------------------------------
+// Which tile of a tx x ty tile grid the t-th workgroup of a launch (or of a problem of a grouped launch) takes.
+// Workgroups go to the eight XCDs in turn, and each XCD has its own L2.  The tiles are laid out as a sequence
+// that sweeps bands of four tile rows column by column, and XCD slot j = t mod 8 takes the j-th eighth of that
+// sequence in order: the 32 tiles an XCD works on at a time form a 4 x 8 block that shares 12 operand slabs per
+// k-tile, whatever the tile grid's width (with tiles numbered row by row a grid eight tiles wide gives an XCD one
+// column: 33 slabs for 32 tiles).  A bijection of [0, tx * ty); every slot gets its share of the tiles to within one.
+__device__ __forceinline__ void xcd_tile(int t, int tx, int ty, int& tile_x, int& tile_y) {
+    const int n = tx * ty;
+    const int j = t & 7, q = n >> 3, r = n & 7;
+    const int seq = j * q + min(j, r) + (t >> 3);
+    const int band = seq / (4 * tx), within = seq - band * 4 * tx;
+    const int hb = min(4, ty - band * 4);
+    tile_x = within / hb;
+    tile_y = band * 4 + within % hb;
+}
+
 template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN, int STAGES, bool GROUPED = false>
 __global__ __launch_bounds__(WM * WN * 64)
 void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs>::type args) {
@@ -376,13 +393,13 @@ void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     int prob = 0, tile_x = blockIdx.x, tile_y = blockIdx.y;
     if constexpr (GROUPED) {
         static_assert(kGroupMax == 4, "the selects below are written out for four problems");
-        int first = 0, tx = args.tiles_x[0];
-        if (1 < args.n && (int)blockIdx.x >= args.first_tile[1]) { prob = 1; first = args.first_tile[1]; tx = args.tiles_x[1]; }
-        if (2 < args.n && (int)blockIdx.x >= args.first_tile[2]) { prob = 2; first = args.first_tile[2]; tx = args.tiles_x[2]; }
-        if (3 < args.n && (int)blockIdx.x >= args.first_tile[3]) { prob = 3; first = args.first_tile[3]; tx = args.tiles_x[3]; }
-        const int t = (int)blockIdx.x - first;
-        tile_y = t / tx;
-        tile_x = t % tx;
+        int first = 0, tx = args.tiles_x[0], ty = args.tiles_y[0];
+        if (1 < args.n && (int)blockIdx.x >= args.first_tile[1]) { prob = 1; first = args.first_tile[1]; tx = args.tiles_x[1]; ty = args.tiles_y[1]; }
+        if (2 < args.n && (int)blockIdx.x >= args.first_tile[2]) { prob = 2; first = args.first_tile[2]; tx = args.tiles_x[2]; ty = args.tiles_y[2]; }
+        if (3 < args.n && (int)blockIdx.x >= args.first_tile[3]) { prob = 3; first = args.first_tile[3]; tx = args.tiles_x[3]; ty = args.tiles_y[3]; }
+        xcd_tile((int)blockIdx.x - first, tx, ty, tile_x, tile_y);
+    } else if (gridDim.z == 1) {
+        xcd_tile((int)(blockIdx.y * gridDim.x + blockIdx.x), (int)gridDim.x, (int)gridDim.y, tile_x, tile_y);
     }
     // (constant indices only: a dynamically indexed kernel argument would be copied to scratch memory)
     const GemmArgs a = [&]() -> GemmArgs {
@@ -975,9 +992,10 @@ static void launch_group(const tp_gemm_desc* descs, int n, int cfg, hipStream_t 
         ga.g[i] = fill_args(&descs[i], p, nullptr);
         ga.first_tile[i] = tiles;
         ga.tiles_x[i] = p.gx;
+        ga.tiles_y[i] = p.gy;
         tiles += p.gx * p.gy;
     }
-    for (int i = n; i < kGroupMax; ++i) { ga.g[i] = ga.g[0]; ga.first_tile[i] = tiles; ga.tiles_x[i] = 1; }
+    for (int i = n; i < kGroupMax; ++i) { ga.g[i] = ga.g[0]; ga.first_tile[i] = tiles; ga.tiles_x[i] = 1; ga.tiles_y[i] = 1; }
     ga.n = n;
     if (cfg == 19) gemm_tall_kernel<T, AKM, BKM, 256, 256, 64, 4, 2, 2, true><<<dim3(tiles), 512, 0, s>>>(ga);
     else gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4, true><<<dim3(tiles), 512, 0, s>>>(ga);
