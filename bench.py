@@ -1,18 +1,24 @@
 #!/usr/bin/env python3
 """Headline benchmark: sliced GPT-layer-stack forward + reverse-slice backward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3|C4|C5|C1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3|C2|C4|C5|C1]
+    python bench.py --attention-grid            # the (T, P) micro-grid of the prefix-attention kernels
 
 One step = every sequence slice of one synthetic batch through the whole layer stack forward (K/V
 caches growing slice by slice), then the reverse-order slice backward, with the loss
 ``sum(y * R)`` for a fixed random R (inputs N(0,1), weights N(0,0.02), all resident in HBM before the
-timed region).  Prints ONE JSON line: tokens/s, the MFMA roofline of the GEMM kernels (algorithmic
-flops / kernel time, measured live: the GEMM calls of one recorded step replayed in a HIP graph between
-two HIP events), the HBM figure of the prefix-attention kernels, and the CPU oracle timed on this host's cores on a bounded sample.
+timed region).  Prints ONE JSON line: tokens/s of the workload (default C3, the GPT-3 13B stage share),
+the MFMA roofline of its GEMM kernels (algorithmic flops / kernel time, measured live: the GEMM calls
+of one recorded step replayed in a HIP graph between two HIP events; also per GEMM shape next to the
+bound min(MFMA peak, operand bytes / HBM peak) allows), the HBM figure of the prefix-attention
+kernels of the 32-token-slice workload C5, the same figures in short for the other 16-bit workloads, and
+the CPU oracle timed on this host's cores on a bounded sample.
 """
 import argparse
+import gc
 import json
 import os
+import re
 import sys
 import time
 
@@ -26,10 +32,6 @@ if ROOT not in sys.path:
 PEAK_MFMA_16BIT = 2.5e15     # dense fp16/bf16 MFMA flop/s
 PEAK_MFMA_FP32 = 157.3e12
 PEAK_HBM = 8.0e12            # bytes/s
-
-# HBM bytes per GEMM call (FETCH_SIZE + WRITE_SIZE of the GEMM kernels of one step / calls), from the two
-# rocprofv3 --pmc runs summarised in profiles/bench_C2_gemm_hbm_traffic.pmc.txt; only measured for C2
-PMC_GEMM_TRAFFIC_BYTES = {"C2": 32.86e6}
 
 WORKLOADS = {
     # name: layers, hidden, heads, ffn, seq, batch, dtype, slices, weight std
@@ -47,6 +49,7 @@ WORKLOADS = {
                n_layers=4, E=6144, H=48, F=24576, L=2048, B=2, dtype="bf16", slices=[32] * 64, std=0.02),
 }
 TORCH_DTYPE = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+GEMM_OPS = {0: "NT", 1: "NN", 2: "TN"}
 
 
 def gemm_flops_per_step(w):
@@ -56,14 +59,38 @@ def gemm_flops_per_step(w):
     return 3 * per_token_fwd * w["L"] * w["B"] * w["n_layers"]
 
 
-def attn_bytes_per_call(w, T, P, bwd):
+def attn_bytes_per_call(es, B, H, E, T, P, bwd):
     """Algorithmic HBM bytes of one prefix-attention call (one layer, one slice): elements x dtype size
     plus the fp32 LSE / delta vectors.  fwd (2T + 2S) B E; bwd (6T + 2S + 4P) B E."""
-    es = 4 if w["dtype"] == "f32" else 2
-    S, BE, BH = P + T, w["B"] * w["E"], w["B"] * w["H"]
+    S, BE, BH = P + T, B * E, B * H
     if not bwd:
         return (2 * T + 2 * S) * BE * es + 4 * BH * T
     return (6 * T + 2 * S + 4 * P) * BE * es + 8 * BH * T
+
+
+def gemm_shape_work(meta, es):
+    """(flops, algorithmic bytes) of one recorded GEMM call: a single (op, M, N, K) or, for a grouped launch,
+    a tuple of them.  Bytes: both operands in once, the result out once."""
+    metas = meta if isinstance(meta[0], tuple) else (meta,)
+    flops = sum(2 * M * N * K for (_, M, N, K) in metas)
+    nbytes = sum((M * K + N * K + M * N) * es for (_, M, N, K) in metas)
+    return flops, nbytes
+
+
+def gemm_shape_name(meta):
+    metas = meta if isinstance(meta[0], tuple) else (meta,)
+    return " + ".join("%s %dx%dx%d" % (GEMM_OPS[op], M, N, K) for (op, M, N, K) in metas)
+
+
+def pmc_traffic(workload):
+    """HBM bytes per GEMM launch of a step, from the committed summary of the two rocprofv3 --pmc runs
+    (FETCH_SIZE, WRITE_SIZE) over one step of this workload; None when no such summary is in the tree."""
+    path = os.path.join(ROOT, "profiles", "bench_%s_gemm_hbm_traffic.pmc.txt" % workload)
+    try:
+        m = re.search(r"traffic_bytes_per_gemm_launch:\s*([0-9.eE+]+)", open(path).read())
+    except OSError:
+        return None
+    return float(m.group(1)) if m else None
 
 
 def build_model(w, device):
@@ -118,7 +145,7 @@ def optimizer_step(layers, runner, x, R, reps=5):
             "note": "includes the host's build and upload of the tensor table each call"}
 
 
-def cpu_baseline(w, budget_layers=None):
+def cpu_baseline(w, sample_layers=None):
     """The CPU oracle (fp32 restatement of the reference path) on this host's cores, on a bounded
     sample: the full sequence and slice list through `sample_layers` layers of the stack; the
     whole-stack rate is that rate divided by n_layers / sample_layers."""
@@ -127,7 +154,7 @@ def cpu_baseline(w, budget_layers=None):
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
     flops_layer = gemm_flops_per_step(w) / w["n_layers"]
-    sample_layers = budget_layers or max(1, min(w["n_layers"], int(1.5e13 // flops_layer)))
+    sample_layers = sample_layers or max(1, min(w["n_layers"], int(0.8e13 // flops_layer)))
     ps = oracle.init_stack_params(sample_layers, w["E"], w["F"], w["std"], torch.float32, seed=0)
     for p in ps:
         for v in p.values():
@@ -145,17 +172,292 @@ def cpu_baseline(w, budget_layers=None):
                       "(%.1f s), scaled by the layer count" % (sample_layers, w["n_layers"], dt)}
 
 
+def _graph_ms(fns, reps=3):
+    """Average milliseconds of one pass over `fns` (callables that launch on the current stream): the pass is
+    captured into a HIP graph and the replays are bracketed by two HIP events on that stream, so no host
+    launch gap is inside the figure."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for fn in fns[:4]:
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for fn in fns:
+            fn()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def measure_workload(name, args, device, detail):
+    """Times `name`: tokens/s over args.steps steps after args.warmup, then (unless --no-roofline) the kernel
+    times of one recorded step per kind.  detail: also per GEMM shape."""
+    from terapipe_amd import ops
+    w = WORKLOADS[name]
+    layers, runner, x, R = build_model(w, device)
+    runner.use_hip_graph = args.graph
+    runner.slice_streams = args.slice_streams
+    runner.launch_replay = not (args.graph or args.no_launch_replay)
+    warmup, steps = (args.warmup, args.steps) if detail else (3, 5)
+    for _ in range(warmup):
+        one_step(layers, runner, x, R)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one_step(layers, runner, x, R)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    res = {"workload": "%s: %s" % (name, w["desc"]), "dtype": w["dtype"], "steps": steps, "warmup": warmup,
+           "ms_per_step": elapsed * 1e3 / steps, "tokens_per_s": w["L"] * w["B"] * steps / elapsed}
+    if args.no_roofline:
+        return res, (layers, runner, x, R)
+
+    # Kernel time per kind, measured live with HIP events: one step is recorded (every library call
+    # with its descriptor and buffers), then all calls of one kind are replayed back to back inside
+    # a HIP graph on the launch stream and the replay is bracketed by two events.  Replaying from a
+    # graph keeps host launch gaps out of the figure (events around single eager launches would
+    # include the time the GPU waits for the host).
+    runner.use_hip_graph = False
+    runner.launch_replay = False
+    with ops.CallRecorder() as rec:
+        one_step(layers, runner, x, R)
+    torch.cuda.synchronize()
+    # the recorded weight-gradient GEMMs write into this step's gradient tensors: keep them alive while
+    # the calls are replayed
+    recorded_grads = [p.grad for p in layers.parameters()]
+    es = 4 if w["dtype"] == "f32" else 2
+    peak = PEAK_MFMA_FP32 if w["dtype"] == "f32" else PEAK_MFMA_16BIT
+
+    def calls_of(tag):
+        # "attn_bwd" covers both launches of the attention backward of a slice: delta + dQ, and the
+        # one-pass dK/dV over all later positions
+        return [c for c in rec.calls if c[0] == tag or (tag == "attn_bwd" and c[0] == "attn_bwd_dkdv")]
+
+    gemm_calls = calls_of("gemm")
+    g_ms = _graph_ms([fn for _, _, fn in gemm_calls])
+    flops = gemm_flops_per_step(w)
+    achieved = flops / (g_ms * 1e-3)
+    # what the rooflines allow each launch: the larger of its MFMA time and the time to move its operands
+    # and result through HBM once
+    work = [gemm_shape_work(m, es) for _, m, _ in gemm_calls]
+    bound_s = sum(max(f / peak, b / PEAK_HBM) for f, b in work)
+    attainable = sum(f for f, _ in work) / bound_s
+    roof = {
+        "kernel": "tp::gemm_dma_kernel / tp::gemm_tall_kernel / tp::gemm_stream_kernel (all NT/NN/TN launches of one step, "
+                  "split-K reduce included)",
+        "bound": "mfma", "achieved": achieved / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
+        "frac": achieved / peak, "traffic": pmc_traffic(name),
+        "launches": len(gemm_calls), "avg_launch_us": g_ms * 1e3 / max(len(gemm_calls), 1),
+        "algorithmic_flops_per_step": flops, "kernel_ms_per_step": g_ms,
+        "attainable": attainable / 1e12, "attainable_frac": attainable / peak,
+        "achieved_over_attainable": achieved / attainable,
+        "attainable_note": "per launch min(MFMA peak, (A + B + C bytes) / 8 TB/s), summed over the step's launches",
+        "method": "graph replay of the step's GEMM calls between two HIP events",
+    }
+    if detail:
+        groups = {}
+        for c in gemm_calls:
+            groups.setdefault(c[1], []).append(c[2])
+        per = []
+        for meta, fns in groups.items():
+            ms = _graph_ms(fns)
+            f, b = gemm_shape_work(meta, es)
+            us = ms * 1e3 / len(fns)
+            bound_us = max(f / peak, b / PEAK_HBM) * 1e6
+            per.append({"gemm": gemm_shape_name(meta), "calls": len(fns), "avg_us": round(us, 2),
+                        "tflops": round(f / us / 1e6, 1), "bound_us": round(bound_us, 2),
+                        "bound": "mfma" if f / peak >= b / PEAK_HBM else "hbm",
+                        "frac_of_bound": round(bound_us / us, 3)})
+        per.sort(key=lambda r: -r["avg_us"] * r["calls"])
+        roof["per_gemm"] = per
+    if args.slice_streams > 1:
+        # the same GEMM calls as the step issues them: spread over the slice streams, so that a launch
+        # which fills part of the chip runs beside its neighbours'.  Launched from the host (closures
+        # bound to their descriptors), bracketed by two events on the current stream.  Every chain has a
+        # k-split workspace of its own, as the runner's streams have.
+        chains = [torch.cuda.Stream() for _ in range(args.slice_streams)]
+        ws_bytes = max([b.numel() for b in ops.Workspace._bufs.values()] + [1 << 20])
+        chain_ws = [torch.empty(ws_bytes, dtype=torch.uint8, device=device) for _ in chains]
+        main = torch.cuda.current_stream()
+
+        def spread():
+            for st in chains:
+                st.wait_stream(main)
+            for i, (_, _, fn) in enumerate(gemm_calls):
+                k = i % len(chains)
+                if fn(chains[k].cuda_stream, ws=chain_ws[k]):
+                    raise RuntimeError("replayed GEMM failed")
+            for st in chains:
+                main.wait_stream(st)
+        spread()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(3):
+            spread()
+        e1.record()
+        torch.cuda.synchronize()
+        c_ms = e0.elapsed_time(e1) / 3
+        roof["shared_chip"] = {
+            "chains": len(chains), "kernel_ms_per_step": c_ms, "achieved": flops / (c_ms * 1e-3) / 1e12,
+            "frac": flops / (c_ms * 1e-3) / peak,
+            "method": "the step's GEMM calls issued round-robin over the slice streams, as the step overlaps them"}
+        del chain_ws
+    res["roofline"] = roof
+    attn = {}
+    kt = {"gemm": round(g_ms, 3)}
+    has_suffix = any(c[0] == "attn_bwd_dkdv" for c in rec.calls)
+    for tag in ("attn_fwd", "attn_bwd"):
+        calls = calls_of(tag)
+        ms = _graph_ms([fn for _, _, fn in calls]) if calls else 0.0
+        metas = [m for t, m, _ in calls if t == tag]     # one per slice and layer
+        nbytes = sum(attn_bytes_per_call(es, w["B"], w["H"], w["E"], T, P, tag == "attn_bwd") for (_b, _h, _d, T, P) in metas)
+        gbs = nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+        attn[tag] = {"calls": len(metas), "launches_per_call": 2 if tag == "attn_bwd" and has_suffix else 1,
+                     "kernel_ms_per_step": ms, "algorithmic_GB_per_step": nbytes / 1e9,
+                     "achieved_GBps": gbs, "frac_of_hbm_peak": gbs * 1e9 / PEAK_HBM}
+        kt[tag] = round(ms, 3)
+    for tag in ("layernorm_fwd", "layernorm_bwd"):
+        calls = calls_of(tag)
+        kt[tag] = round(_graph_ms([fn for _, _, fn in calls]) if calls else 0.0, 3)
+    res["roofline_attention"] = {"bound": "hbm", "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+                                 "slice_tokens": sorted(set(w["slices"])), **attn}
+    res["kernel_time_ms_per_step"] = kt
+    del recorded_grads
+    return res, (layers, runner, x, R)
+
+
+def attention_grid(device, reps=5):
+    """The (T, P) micro-grid of the prefix-attention kernels, as the reference profiles a layer per
+    (seqlen, attention_cache_len) (terapipe_latency_model.py:180-193): slice length T in {32, 64, 128}, prefix P
+    in {0, 256, ..., 1792, 2048 - T} of a 2048-token sequence, head dimension 128, bf16, at the (batch, heads) of
+    workloads C5 (2, 48) and C4 (1, 96).  Per point: the forward call, the backward as the sliced runner issues
+    it (delta + dQ against the prefix, then dK/dV of the slice's keys against every later query position), and
+    the backward with gradient caches (the reference's per-call contract: dK/dV of all S keys, prefix rows
+    read-modify-written).  Each call is timed alone on the chip over `sets` rotating sets of buffers larger
+    together than the memory-side cache, replayed from a HIP graph between two HIP events; GB/s are the
+    reference algorithm's bytes of the call (fwd (2T+2S) B E, bwd (6T+2S+4P) B E, + fp32 row statistics)."""
+    from terapipe_amd import ops
+    L, Dh, dt, es = 2048, 128, torch.bfloat16, 2
+    out = []
+    for wl, (B, H) in (("C5", (2, 48)), ("C4", (1, 96))):
+        BH, E = B * H, H * Dh
+        sets = 6
+        g = torch.Generator(device=device).manual_seed(7)
+        bufs = []
+        for _ in range(sets):
+            b = dict(q=torch.randn(BH, L, Dh, generator=g, device=device).to(dt) * Dh ** -0.5,
+                     k=torch.randn(BH, L, Dh, generator=g, device=device).to(dt),
+                     v=torch.randn(BH, L, Dh, generator=g, device=device).to(dt),
+                     o=torch.empty(L, B, E, dtype=dt, device=device),
+                     d_o=torch.randn(L, B, E, generator=g, device=device).to(dt),
+                     lse=torch.zeros(BH, L, dtype=torch.float32, device=device),
+                     delta=torch.zeros(BH, L, dtype=torch.float32, device=device),
+                     dqkv=torch.empty(128 * B, 3 * E, dtype=dt, device=device),
+                     gk=torch.zeros(BH, L, Dh, dtype=torch.float32, device=device),
+                     gv=torch.zeros(BH, L, Dh, dtype=torch.float32, device=device))
+            bufs.append(b)
+        # every position's lse / delta / o must be valid for the one-pass dK/dV: one forward + dQ sweep first
+        for b in bufs:
+            for P in range(0, L, 128):
+                ops.attn_prefix_fwd(b["q"][:, P:], b["k"], b["v"], B, H, Dh, 128, P, Dh ** -0.5, out=b["o"][P:P + 128],
+                                    lse=b["lse"][:, P:], q_bh_rows=L, stat_bh_rows=L)
+                ops.attn_prefix_bwd(b["q"][:, P:], b["k"], b["v"], b["o"][P:P + 128], b["lse"][:, P:], b["d_o"][P:P + 128],
+                                    b["dqkv"], None, None, B, H, Dh, 128, P, Dh ** -0.5, False, False, False,
+                                    delta=b["delta"][:, P:], q_bh_rows=L, stat_bh_rows=L, dq_only=True)
+        torch.cuda.synchronize()
+        for T in (32, 64, 128):
+            rows = []
+            for P in sorted(set(list(range(0, L - T, 256)) + [L - T])):
+                def fwd(b, T=T, P=P):
+                    ops.attn_prefix_fwd(b["q"][:, P:], b["k"], b["v"], B, H, Dh, T, P, Dh ** -0.5, out=b["o"][P:P + T],
+                                        lse=b["lse"][:, P:], q_bh_rows=L, stat_bh_rows=L)
+
+                def dq(b, T=T, P=P):
+                    ops.attn_prefix_bwd(b["q"][:, P:], b["k"], b["v"], b["o"][P:P + T], b["lse"][:, P:], b["d_o"][P:P + T],
+                                        b["dqkv"][:T * B], None, None, B, H, Dh, T, P, Dh ** -0.5, False, False, False,
+                                        delta=b["delta"][:, P:], q_bh_rows=L, stat_bh_rows=L, dq_only=True)
+
+                def dkdv(b, T=T, P=P):
+                    ops.attn_suffix_dkdv(b["k"], b["v"], b["q"], b["d_o"], b["lse"], b["delta"], b["dqkv"][:T * B], B, H, Dh,
+                                         P, T, L)
+
+                def bwd_cache(b, T=T, P=P):
+                    ops.attn_prefix_bwd(b["q"][:, P:], b["k"], b["v"], b["o"][P:P + T], b["lse"][:, P:], b["d_o"][P:P + T],
+                                        b["dqkv"][:T * B], b["gk"], b["gv"], B, H, Dh, T, P, Dh ** -0.5, True, True, False,
+                                        delta=b["delta"][:, P:], q_bh_rows=L, stat_bh_rows=L)
+
+                us = {}
+                for nm, fn in (("fwd", fwd), ("dq", dq), ("dkdv", dkdv), ("bwd_cache", bwd_cache)):
+                    us[nm] = _graph_ms([(lambda b=b, fn=fn: fn(b)) for b in bufs], reps) * 1e3 / sets
+                fb = attn_bytes_per_call(es, B, H, E, T, P, False)
+                bb = attn_bytes_per_call(es, B, H, E, T, P, True)
+                rows.append({"P": P, "fwd_us": round(us["fwd"], 2), "fwd_GBps": round(fb / us["fwd"] / 1e3, 1),
+                             "dq_us": round(us["dq"], 2), "dkdv_us": round(us["dkdv"], 2),
+                             "bwd_cache_us": round(us["bwd_cache"], 2), "bwd_cache_GBps": round(bb / us["bwd_cache"] / 1e3, 1),
+                             "fwd_bytes": fb, "bwd_bytes": bb})
+            out.append({"heads_of": wl, "batch": B, "heads": H, "T": T, "points": rows})
+        del bufs
+        gc.collect()
+        torch.cuda.empty_cache()
+    # a whole sequence of slices of T tokens visits every P = 0, T, 2T, ...: the dQ call of the slice at P and the
+    # one-pass dK/dV call of the slice at L - T - P do, together, the work the reference's backward of (T, P) does
+    for grp in out:
+        pts = {r["P"]: r for r in grp["points"]}
+        for r in grp["points"]:
+            mirror = pts.get(L - grp["T"] - r["P"])
+            if mirror is not None:
+                r["bwd_runner_us"] = round(r["dq_us"] + mirror["dkdv_us"], 2)
+                r["bwd_runner_GBps"] = round(r["bwd_bytes"] / r["bwd_runner_us"] / 1e3, 1)
+    return {"metric": "prefix-attention kernel time and achieved HBM GB/s per (T, P)", "unit": "us, GB/s",
+            "dtype": "bf16", "head_dim": Dh, "seq": L, "peak_GBps": PEAK_HBM / 1e9,
+            "method": "each call alone on the chip over 6 rotating buffer sets, HIP-graph replay between two HIP events",
+            "grid": out}
+
+
+def _short(res):
+    """The other workloads' figures in short."""
+    s = {"workload": res["workload"], "ms_per_step": round(res["ms_per_step"], 3),
+         "tokens_per_s": round(res["tokens_per_s"], 1)}
+    if "roofline" in res:
+        r = res["roofline"]
+        s["gemm"] = {"kernel_ms_per_step": round(r["kernel_ms_per_step"], 3), "achieved_TFLOPs": round(r["achieved"], 1),
+                     "frac": round(r["frac"], 4), "attainable_frac": round(r["attainable_frac"], 4)}
+        if "shared_chip" in r:
+            s["gemm"]["shared_chip_frac"] = round(r["shared_chip"]["frac"], 4)
+        a = res["roofline_attention"]
+        s["attention"] = {k: {"kernel_ms_per_step": round(a[k]["kernel_ms_per_step"], 3),
+                              "achieved_GBps": round(a[k]["achieved_GBps"], 1),
+                              "frac_of_hbm_peak": round(a[k]["frac_of_hbm_peak"], 4)} for k in ("attn_fwd", "attn_bwd")}
+        s["kernel_time_ms_per_step"] = res["kernel_time_ms_per_step"]
+    return s
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="C3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="with the default workload C3 the line also carries the prefix-attention roofline measured on C5 "
+                         "(32-token slices) and short figures for C2, C4 and C5; this leaves them out")
+    ap.add_argument("--attention-grid", action="store_true",
+                    help="print the (T, P) micro-grid of the prefix-attention kernels instead of the step benchmark")
     ap.add_argument("--copy-calibration", action="store_true",
-                    help="also run one plain 256 MiB device copy (torch copy_ kernel) before the steps: the "
-                         "known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
+                    help="also run one plain 256 MiB device fill and one 256 MiB copy before the steps: the "
+                         "known-size kernels that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     ap.add_argument("--slice-streams", type=int, default=3,
                     help="streams the runner spreads consecutive slices over (1 = one chain of kernels); slice "
                          "i+1 of layer l runs beside slice i of layer l+1, which fills the CUs the short kernels "
@@ -178,154 +480,61 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
-    w = WORKLOADS[args.workload]
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    from terapipe_amd import ops
-
-    layers, runner, x, R = build_model(w, device)
+    if args.attention_grid:
+        print(json.dumps(attention_grid(device)))
+        return
     if args.graph and (args.eager or args.slice_streams != 1):
         print("bench.py: --graph replays a single-stream capture; use it with --slice-streams 1 and without --eager",
               file=sys.stderr)
         sys.exit(2)
-    runner.use_hip_graph = args.graph
-    runner.slice_streams = args.slice_streams
-    runner.launch_replay = not (args.graph or args.no_launch_replay)
+    w = WORKLOADS[args.workload]
     if args.copy_calibration:
         src = torch.ones(64 << 20, dtype=torch.int32, device=device)
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    for _ in range(args.warmup):
-        one_step(layers, runner, x, R)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        one_step(layers, runner, x, R)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
-    tokens = w["L"] * w["B"]
-    value = tokens * args.steps / elapsed
 
+    res, model = measure_workload(args.workload, args, device, detail=True)
     out = {
         "metric": "sliced-layer fwd+bwd tokens/s on 1 MI355X; % MFMA peak (GEMM), % HBM BW (attn)",
-        "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": res["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w["dtype"], "data": "synthetic",
-        "config": {"workload": "%s: %s" % (args.workload, w["desc"]),
+        "config": {"workload": res["workload"],
                    "loss": "sum(y * R), R ~ N(0,1) fixed", "optimizer_step": "outside the timed step (--optimizer times it separately)",
                    "launch": "HIP-graph replay of forward and of backward" if args.graph else
                              ("eager, every kernel launched from the host" if args.no_launch_replay else
                               "eager, recorded launches re-issued from the host"),
                    "slice_streams": args.slice_streams},
     }
-
-    if not args.no_roofline:
-        # Kernel time per kind, measured live with HIP events: one step is recorded (every library call
-        # with its descriptor and buffers), then all calls of one kind are replayed back to back inside
-        # a HIP graph on the launch stream and the replay is bracketed by two events.  Replaying from a
-        # graph keeps host launch gaps out of the figure (events around single eager launches would
-        # include the time the GPU waits for the host).
-        runner.use_hip_graph = False
-        runner.launch_replay = False
-        with ops.CallRecorder() as rec:
-            one_step(layers, runner, x, R)
-        torch.cuda.synchronize()
-        # the recorded weight-gradient GEMMs write into this step's gradient tensors: keep them alive while
-        # the calls are replayed
-        recorded_grads = [p.grad for p in layers.parameters()]
-
-        def replay_ms(tag, reps=3):
-            # "attn_bwd" covers both launches of the attention backward of a slice: delta + dQ, and the
-            # one-pass dK/dV over all later positions
-            calls = [c for c in rec.calls if c[0] == tag or (tag == "attn_bwd" and c[0] == "attn_bwd_dkdv")]
-            if not calls:
-                return 0, 0.0, []
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                for _, _, fn in calls[:4]:
-                    fn()
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                for _, _, fn in calls:
-                    fn()
-            g.replay()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(reps):
-                g.replay()
-            e1.record()
-            torch.cuda.synchronize()
-            return len(calls), e0.elapsed_time(e1) / reps, [m for _, m, _ in calls]
-
-        g_calls, g_ms, _ = replay_ms("gemm")
-        flops = gemm_flops_per_step(w)
-        peak = PEAK_MFMA_FP32 if w["dtype"] == "f32" else PEAK_MFMA_16BIT
-        achieved = flops / (g_ms * 1e-3) if g_ms > 0 else 0.0
-        out["roofline"] = {
-            "kernel": "tp::gemm_dma_kernel / tp::gemm_tall_kernel (all NT/NN/TN launches of one step, split-K reduce included)",
-            "bound": "mfma", "achieved": achieved / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
-            "frac": achieved / peak, "traffic": PMC_GEMM_TRAFFIC_BYTES.get(args.workload),
-            "launches": g_calls, "avg_launch_us": g_ms * 1e3 / max(g_calls, 1),
-            "algorithmic_flops_per_step": flops, "kernel_ms_per_step": g_ms,
-            "method": "graph replay of the step's GEMM calls between two HIP events",
-        }
-        if args.slice_streams > 1:
-            # the same GEMM calls as the step issues them: spread over the slice streams, so that a launch
-            # which fills part of the chip runs beside its neighbours'.  Launched from the host (closures
-            # bound to their descriptors), bracketed by two events on the current stream.
-            chains = [torch.cuda.Stream() for _ in range(args.slice_streams)]
-            calls = [c for c in rec.calls if c[0] == "gemm"]
-            main = torch.cuda.current_stream()
-
-            def spread():
-                for st in chains:
-                    st.wait_stream(main)
-                for i, (_, _, fn) in enumerate(calls):
-                    if fn(chains[i % len(chains)].cuda_stream):
-                        raise RuntimeError("replayed GEMM failed")
-                for st in chains:
-                    main.wait_stream(st)
-            spread()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(3):
-                spread()
-            e1.record()
-            torch.cuda.synchronize()
-            c_ms = e0.elapsed_time(e1) / 3
-            out["roofline"]["shared_chip"] = {
-                "chains": len(chains), "kernel_ms_per_step": c_ms, "achieved": flops / (c_ms * 1e-3) / 1e12,
-                "frac": flops / (c_ms * 1e-3) / peak,
-                "method": "the step's GEMM calls issued round-robin over the slice streams, as the step overlaps them"}
-        attn = {}
-        kt = {"gemm": round(g_ms, 3)}
-        for tag in ("attn_fwd", "attn_bwd"):
-            c, ms, metas = replay_ms(tag)
-            nbytes = sum(attn_bytes_per_call(w, T, P, tag == "attn_bwd") for (_b, _h, _d, T, P) in metas) / \
-                (2 if tag == "attn_bwd" and any(c[0] == "attn_bwd_dkdv" for c in rec.calls) else 1)
-            gbs = nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
-            if tag == "attn_bwd" and any(cc[0] == "attn_bwd_dkdv" for cc in rec.calls):
-                c //= 2      # two library calls per slice backward
-            attn[tag] = {"calls": c, "kernel_ms_per_step": ms, "algorithmic_GB_per_step": nbytes / 1e9,
-                         "achieved_GBps": gbs, "frac_of_hbm_peak": gbs * 1e9 / PEAK_HBM}
-            kt[tag] = round(ms, 3)
-        for tag in ("layernorm_fwd", "layernorm_bwd"):
-            kt[tag] = round(replay_ms(tag)[1], 3)
-        out["roofline_attention"] = {"bound": "hbm", "peak": PEAK_HBM / 1e9, "unit": "GB/s", **attn}
-        out["kernel_time_ms_per_step"] = kt
-
-        del recorded_grads
-
+    for k in ("roofline", "kernel_time_ms_per_step"):
+        if k in res:
+            out[k] = res[k]
+    if "roofline_attention" in res:
+        out["roofline_attention"] = dict(res["roofline_attention"], workload=args.workload)
     if args.optimizer and w["dtype"] != "f32":
-        out["optimizer_step"] = optimizer_step(layers, runner, x, R)
+        out["optimizer_step"] = optimizer_step(*model)
+    del model
+    gc.collect()
+    torch.cuda.empty_cache()
+
+    if args.workload == "C3" and not args.no_other_workloads and not args.no_roofline:
+        # the prefix-attention target is stated for slices of at most 128 tokens: C5 (32-token slices) gives the
+        # line's roofline_attention, the 13B workload's own attention figures move to roofline_attention_C3
+        others = {}
+        for name in ("C5", "C4", "C2"):
+            r, m = measure_workload(name, args, device, detail=False)
+            del m
+            gc.collect()
+            torch.cuda.empty_cache()
+            others[name] = _short(r)
+            if name == "C5":
+                out["roofline_attention_C3"] = out["roofline_attention"]
+                out["roofline_attention"] = dict(r["roofline_attention"], workload="C5")
+        out["other_workloads"] = others
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)

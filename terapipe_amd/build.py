@@ -30,8 +30,20 @@ def hipcc_path():
     raise RuntimeError("hipcc not found")
 
 
-def build(verbose=True, jobs=4):
-    """Compiles every source to an object (in parallel) and links the shared library."""
+def _stale(src_path, obj):
+    """True unless obj is newer than its source and every header the sources share."""
+    if not os.path.exists(obj):
+        return True
+    deps = [src_path, os.path.join(CSRC, "common.h"), os.path.join(CSRC, "gemm_tuned.inc"),
+            os.path.join(os.path.dirname(HERE), "include", "terapipe_hip.h")]
+    t = os.path.getmtime(obj)
+    return any(os.path.getmtime(d) > t for d in deps if os.path.exists(d))
+
+
+def build(verbose=True, jobs=7, incremental=False):
+    """Compiles every source to an object (in parallel) and links the shared library.  incremental: leave
+    objects alone that are newer than their source and the shared headers (a development convenience;
+    the default compiles everything)."""
     hipcc = hipcc_path()
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
@@ -41,6 +53,8 @@ def build(verbose=True, jobs=4):
     for src in SOURCES:
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
         objs.append(obj)
+        if incremental and not _stale(os.path.join(CSRC, src), obj):
+            continue
         cmd = [hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
         procs.append((src, cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
         while sum(1 for _, _, p in procs if p.poll() is None) >= jobs:
@@ -62,5 +76,5 @@ def build(verbose=True, jobs=4):
 
 
 if __name__ == "__main__":
-    build()
+    build(incremental="--incremental" in sys.argv[1:])
     sys.exit(0)

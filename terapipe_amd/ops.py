@@ -37,31 +37,6 @@ def _require_cuda(*tensors):
             raise _lib.TeraPipeHipError("terapipe_amd kernels need CUDA/HIP tensors; there is no CPU path")
 
 
-class KernelTimer:
-    """Optional per-call HIP-event timing of the library calls (used by bench.py for the roofline
-    figures).  While active, every wrapped call is bracketed by two events on the current stream."""
-    active = None
-
-    def __init__(self):
-        self.records = []   # (tag, meta, start_event, end_event)
-
-    def __enter__(self):
-        KernelTimer.active = self
-        return self
-
-    def __exit__(self, *exc):
-        KernelTimer.active = None
-
-    def summary(self):
-        """{tag: (calls, total_ms, [meta...])} -- call after torch.cuda.synchronize()."""
-        out = {}
-        for tag, meta, e0, e1 in self.records:
-            c, ms, metas = out.get(tag, (0, 0.0, []))
-            metas.append(meta)
-            out[tag] = (c + 1, ms + e0.elapsed_time(e1), metas)
-        return out
-
-
 class CallRecorder:
     """Records every library call made while active as (tag, meta, replay) where replay(stream=None) issues
     the same call again with the same descriptor and buffers, on the given stream handle or else on the
@@ -98,25 +73,6 @@ def _on(stream):
     return _stream() if stream is None else stream
 
 
-class _timed:
-    __slots__ = ("tag", "meta", "e0")
-
-    def __init__(self, tag, meta=None):
-        self.tag, self.meta = tag, meta
-
-    def __enter__(self):
-        if KernelTimer.active is not None:
-            self.e0 = torch.cuda.Event(enable_timing=True)
-            self.e0.record()
-        return self
-
-    def __exit__(self, *exc):
-        if KernelTimer.active is not None:
-            e1 = torch.cuda.Event(enable_timing=True)
-            e1.record()
-            KernelTimer.active.records.append((self.tag, self.meta, self.e0, e1))
-
-
 # (op, M, N, K) -> (tile configuration, k splits): overrides the library's plan for that shape.  A tuning hook:
 # terapipe_amd.tune_gemm's in-step search fills it to time whole steps with one shape's plan changed.
 GEMM_PLAN_OVERRIDE = {}
@@ -124,17 +80,30 @@ GEMM_PLAN_OVERRIDE = {}
 
 class Workspace:
     """A grow-only scratch tensor per device and stream (torch-owned), handed to calls that need
-    workspace: kernels of different streams may run at the same time and must not share partial sums."""
+    workspace: kernels of different streams may run at the same time and must not share partial sums.
+    A buffer that is outgrown is kept for the life of the process, never returned to torch's allocator:
+    recorded launches and captured HIP graphs hold its raw address and may run again at any time."""
     _bufs = {}
+    _superseded = []
 
     @classmethod
-    def get(cls, nbytes, device):
-        key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
+    def get(cls, nbytes, device, stream=None):
+        """The buffer of `stream` (a raw stream handle; default: the current stream), grown to nbytes if needed."""
+        if stream is None:
+            stream = torch.cuda.current_stream(device).cuda_stream
+        key = (device.type, device.index, stream)
         buf = cls._bufs.get(key)
         if buf is None or buf.numel() < nbytes:
+            if buf is not None:
+                cls._superseded.append(buf)
             buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
             cls._bufs[key] = buf
         return buf
+
+    @classmethod
+    def size(cls, device, stream):
+        buf = cls._bufs.get((device.type, device.index, stream))
+        return 0 if buf is None else buf.numel()
 
 
 class PendingReduce:
@@ -162,13 +131,11 @@ def layernorm_fwd(x2d, gamma, beta, eps=1e-5, out=None, mean=None, rstd=None):
     if pend is not None:
         a = (_p(pend.ws), pend.nsplit, _p(pend.bias), _p(pend.residual), _p(x2d), _p(gamma), _p(beta), _p(y), _p(mean),
              _p(rstd), M, E, eps, tp_dtype(x2d.dtype))
-        with _timed("layernorm_fwd", (M, E)):
-            _lib.check(lib.tp_layernorm_fwd_partials(*a, _stream()), "tp_layernorm_fwd_partials")
-        _record("layernorm_fwd", (M, E), lambda s=None: lib.tp_layernorm_fwd_partials(*a, _on(s)))
+        _lib.check(lib.tp_layernorm_fwd_partials(*a, _stream()), "tp_layernorm_fwd_partials")
+        _record("layernorm_fwd", (M, E), lambda s=None, keep=pend: lib.tp_layernorm_fwd_partials(*a, _on(s)))
         return y, mean, rstd
-    with _timed("layernorm_fwd", (M, E)):
-        _lib.check(lib.tp_layernorm_fwd(_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps,
-                                        tp_dtype(x2d.dtype), _stream()), "tp_layernorm_fwd")
+    _lib.check(lib.tp_layernorm_fwd(_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps,
+                                    tp_dtype(x2d.dtype), _stream()), "tp_layernorm_fwd")
     if CallRecorder.active is not None:
         a = (_p(x2d), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), M, E, eps, tp_dtype(x2d.dtype))
         _record("layernorm_fwd", (M, E), lambda s=None: lib.tp_layernorm_fwd(*a, _on(s)))
@@ -189,14 +156,12 @@ def layernorm_bwd(dy, x2d, mean, rstd, gamma, dres, dgamma_acc, dbeta_acc, colsu
     if pend is not None:
         a = (_p(pend.ws), pend.nsplit, _p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx), _p(dgamma_acc),
              _p(dbeta_acc), _p(colsum_dres_acc), _p(colsum_dx_acc), M, E, tp_dtype(x2d.dtype))
-        with _timed("layernorm_bwd", (M, E)):
-            _lib.check(lib.tp_layernorm_bwd_partials(*a, _stream()), "tp_layernorm_bwd_partials")
-        _record("layernorm_bwd", (M, E), lambda s=None: lib.tp_layernorm_bwd_partials(*a, _on(s)))
+        _lib.check(lib.tp_layernorm_bwd_partials(*a, _stream()), "tp_layernorm_bwd_partials")
+        _record("layernorm_bwd", (M, E), lambda s=None, keep=pend: lib.tp_layernorm_bwd_partials(*a, _on(s)))
         return dx
-    with _timed("layernorm_bwd", (M, E)):
-        _lib.check(lib.tp_layernorm_bwd(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx),
-                                        _p(dgamma_acc), _p(dbeta_acc), _p(colsum_dres_acc), _p(colsum_dx_acc),
-                                        M, E, tp_dtype(x2d.dtype), _stream()), "tp_layernorm_bwd")
+    _lib.check(lib.tp_layernorm_bwd(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx),
+                                    _p(dgamma_acc), _p(dbeta_acc), _p(colsum_dres_acc), _p(colsum_dx_acc),
+                                    M, E, tp_dtype(x2d.dtype), _stream()), "tp_layernorm_bwd")
     if CallRecorder.active is not None:
         a = (_p(dy), _p(x2d), _p(mean), _p(rstd), _p(gamma), _p(dres), _p(dx), _p(dgamma_acc), _p(dbeta_acc),
              _p(colsum_dres_acc), _p(colsum_dx_acc), M, E, tp_dtype(x2d.dtype))
@@ -248,11 +213,12 @@ def gemm(op, A, B, M, N, K, C=None, epilogue=TP_EPI_STORE, bias=None, residual=N
             d.defer_reduce = 1
     need = lib.tp_gemm_workspace_bytes(ctypes.byref(d))
     ws = Workspace.get(need, A.device) if need else None
-    with _timed("gemm", (op, M, N, K)):
-        _lib.check(lib.tp_gemm(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()), "tp_gemm")
+    _lib.check(lib.tp_gemm(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()), "tp_gemm")
     if CallRecorder.active is not None:
-        wsp, wsn = _p(ws), (ws.numel() if ws is not None else 0)
-        _record("gemm", (op, M, N, K), lambda s=None: lib.tp_gemm(ctypes.byref(d), wsp, wsn, _on(s)))
+        # the closure holds the workspace tensor, not just its address: the memory stays allocated for as
+        # long as the recorded call can be re-issued
+        wsn = ws.numel() if ws is not None else 0
+        _record("gemm", (op, M, N, K), lambda s=None, ws=ws: lib.tp_gemm(ctypes.byref(d), _p(ws), wsn, _on(s)))
     if nsplit > 1:
         return PendingReduce(ws, nsplit, bias, residual, C)
     return C
@@ -284,9 +250,8 @@ def gemm_grouped(items, desc_sinks=None):
     ws = Workspace.get(need, items[0][1].device) if need else None
     wsp, wsn = _p(ws), (ws.numel() if ws is not None else 0)
     meta = tuple((op, M, N, K) for (op, _, _, M, N, K, _, _) in items)
-    with _timed("gemm", meta):
-        _lib.check(lib.tp_gemm_grouped(descs, n, wsp, wsn, _stream()), "tp_gemm_grouped")
-    _record("gemm", meta, lambda s=None: lib.tp_gemm_grouped(descs, n, wsp, wsn, _on(s)))
+    _lib.check(lib.tp_gemm_grouped(descs, n, wsp, wsn, _stream()), "tp_gemm_grouped")
+    _record("gemm", meta, lambda s=None, ws=ws: lib.tp_gemm_grouped(descs, n, _p(ws), wsn, _on(s)))
 
 
 def _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale, q_bh_rows=0,
@@ -319,13 +284,12 @@ def attn_prefix_fwd(q, k_cache, v_cache, batch, heads, head_dim, T, cache_len, q
     lib = _lib.load()
     need = lib.tp_attn_fwd_workspace_bytes(ctypes.byref(d))
     ws = Workspace.get(need, q.device) if need else None
-    with _timed("attn_fwd", (batch, heads, head_dim, T, cache_len)):
-        _lib.check(lib.tp_attn_prefix_fwd(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()),
-                   "tp_attn_prefix_fwd")
+    _lib.check(lib.tp_attn_prefix_fwd(ctypes.byref(d), _p(ws), ws.numel() if ws is not None else 0, _stream()),
+               "tp_attn_prefix_fwd")
     if CallRecorder.active is not None:
-        wsp, wsn = _p(ws), (ws.numel() if ws is not None else 0)
+        wsn = ws.numel() if ws is not None else 0
         _record("attn_fwd", (batch, heads, head_dim, T, cache_len),
-                lambda s=None: lib.tp_attn_prefix_fwd(ctypes.byref(d), wsp, wsn, _on(s)))
+                lambda s=None, ws=ws: lib.tp_attn_prefix_fwd(ctypes.byref(d), _p(ws), wsn, _on(s)))
     return o, lse
 
 
@@ -345,8 +309,7 @@ def attn_prefix_bwd(q, k_cache, v_cache, o, lse, d_o, dqkv, dk_cache, dv_cache, 
     d.accumulate_prefix, d.has_incoming, d.zero_slice_rows = int(accumulate_prefix), int(has_incoming), int(zero_slice_rows)
     d.colsum_dqkv_acc = _p(colsum_dqkv_acc)
     lib = _lib.load()
-    with _timed("attn_bwd", (batch, heads, head_dim, T, cache_len)):
-        _lib.check(lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()), "tp_attn_prefix_bwd")
+    _lib.check(lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _stream()), "tp_attn_prefix_bwd")
     _record("attn_bwd", (batch, heads, head_dim, T, cache_len),
             lambda s=None: lib.tp_attn_prefix_bwd(ctypes.byref(d), None, 0, _on(s)))
     return dqkv
@@ -367,8 +330,7 @@ def attn_suffix_dkdv(k_cache, v_cache, q_all, d_o_all, lse_all, delta_all, dqkv,
     d.q_all, d.d_o_all = q_all.data_ptr(), d_o_all.data_ptr()
     d.lse_all, d.delta_all, d.dqkv = lse_all.data_ptr(), delta_all.data_ptr(), dqkv.data_ptr()
     lib = _lib.load()
-    with _timed("attn_bwd", (batch, heads, head_dim, key_count, key_begin)):
-        _lib.check(lib.tp_attn_suffix_dkdv(ctypes.byref(d), _stream()), "tp_attn_suffix_dkdv")
+    _lib.check(lib.tp_attn_suffix_dkdv(ctypes.byref(d), _stream()), "tp_attn_suffix_dkdv")
     _record("attn_bwd_dkdv", (batch, heads, head_dim, key_count, key_begin),
             lambda s=None: lib.tp_attn_suffix_dkdv(ctypes.byref(d), _on(s)))
     return dqkv
@@ -379,9 +341,8 @@ def ln_param_grads(dy, x2d, mean, rstd, dgamma_acc, dbeta_acc):
     _require_cuda(dy, x2d, dgamma_acc, dbeta_acc)
     M, E = x2d.shape
     lib = _lib.load()
-    with _timed("ln_param_grads", (M, E)):
-        _lib.check(lib.tp_ln_param_grads(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(dgamma_acc), _p(dbeta_acc), M, E,
-                                         tp_dtype(x2d.dtype), _stream()), "tp_ln_param_grads")
+    _lib.check(lib.tp_ln_param_grads(_p(dy), _p(x2d), _p(mean), _p(rstd), _p(dgamma_acc), _p(dbeta_acc), M, E,
+                                     tp_dtype(x2d.dtype), _stream()), "tp_ln_param_grads")
     if CallRecorder.active is not None:
         a = (_p(dy), _p(x2d), _p(mean), _p(rstd), _p(dgamma_acc), _p(dbeta_acc), M, E, tp_dtype(x2d.dtype))
         _record("ln_param_grads", (M, E), lambda s=None: lib.tp_ln_param_grads(*a, _on(s)))

@@ -83,6 +83,30 @@ def test_argument_errors_without_gpu(lib):
     assert lib.tp_zero_words(None, 4, None) == 1
 
 
+def test_failed_replayed_launch_raises_the_library_error():
+    """A recorded launch that returns a status on replay surfaces as TeraPipeHipError."""
+    from terapipe_amd import _lib, terapipe
+    ran = []
+    with pytest.raises(_lib.TeraPipeHipError, match="replayed launch failed"):
+        terapipe._run_program([(lambda a: ran.append(a) or 0, 1), (lambda a: 4, 2), (lambda a: ran.append(a) or 0, 3)])
+    assert ran == [1]
+
+
+def test_hip_graph_with_slice_streams_is_refused():
+    """use_hip_graph with more than one slice stream is switched off (constructor and later attribute changes)."""
+    import terapipe_amd as ta
+    layers = ta.TransformerLayers(1, 128, 256, 2, dtype=torch.float16, device="cpu")
+    with pytest.raises(ValueError, match="slice_streams=1"):
+        ta.TeraPipe(layers, 1, 64, [1], [32, 32], use_hip_graph=True, slice_streams=3)
+    r = ta.TeraPipe(layers, 1, 64, [1], [32, 32], use_hip_graph=True)
+    assert r.slice_streams == 1 and not r.launch_replay
+    r.slice_streams = 2
+    with pytest.raises(ValueError):
+        r._check_mode()
+    r = ta.TeraPipe(layers, 1, 64, [1], [32, 32])
+    assert r.slice_streams == 3 and r.launch_replay
+
+
 def test_ops_refuse_cpu_tensors():
     """There is no CPU fallback: host tensors raise instead of computing."""
     from terapipe_amd import _lib, ops

@@ -89,8 +89,6 @@ GEMM_SHAPES = [
 def test_gemm_nt_nn_tn(dtype, M, N, K):
     ops = _ops()
     from terapipe_amd._lib import TP_GEMM_NN, TP_GEMM_NT, TP_GEMM_TN, TP_EPI_ACCUMULATE
-    if dtype == torch.float32 and M * N * K > 256 * 2048 * 2048:
-        pytest.skip("large shapes are covered in 16-bit")
     g = torch.Generator().manual_seed(M + 7 * N + 13 * K)
     sc = 1.0 / math.sqrt(K)
     # NT: C[M,N] = A[M,K] B[N,K]^T
@@ -268,13 +266,14 @@ def _tuned_entries():
     return sorted(by_weight.items())
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
 @pytest.mark.parametrize("key,shapes", _tuned_entries(), ids=lambda v: "-".join(map(str, v)) if isinstance(v, tuple) else "")
-def test_gemm_measured_plans_at_their_shapes(key, shapes):
+def test_gemm_measured_plans_at_their_shapes(key, shapes, dtype):
     """Every shape of the measured plan table (the benchmark geometries' own GEMMs, with the tile configuration
-    and k-split the table prescribes for them) against the fp32 library product of the same fp16 operands."""
+    and k-split the table prescribes for them) against the fp32 library product of the same 16-bit operands, in
+    both 16-bit types (the table is keyed by extents only: the 175B / 44B entries run in bf16)."""
     ops = _ops()
     from terapipe_amd import _lib as L
-    dtype = torch.float16
     g = torch.Generator(device=DEV).manual_seed(sum(v for v in key if isinstance(v, int)) % 65521)
     op = key[0]
     if op == "TN":
@@ -379,6 +378,9 @@ ATTN_CASES = [
     (7, 1, 1, 64, 5, 12),
     (1, 1, 1, 64, 0, 1),
     (64, 1, 2, 128, 0, 64),        # two waves
+    (32, 2, 48, 128, 2016, 2048),  # BASELINE config 5's last slice: 96 (batch, head) pairs, 32 queries, 2048 keys
+    (128, 1, 96, 128, 1920, 2048), # config 4's last slice
+    (160, 1, 40, 128, 1888, 2048), # config 3's last slice
 ]
 
 
@@ -446,6 +448,9 @@ SUFFIX_CASES = [
     (1, 3, 128, 200, [40, 7, 100, 33]),      # ragged: nothing aligned to the 32-row blocks
     (2, 1, 64, 64, [5, 1, 20]),              # caches longer than the sequence
     (1, 2, 128, 512, [128, 128, 128, 128]),
+    (2, 48, 128, 1024, [32] * 32),                             # BASELINE config 5's heads and slices (half its length)
+    (1, 96, 128, 1024, [128] * 8),                             # config 4's
+    (1, 40, 128, 2048, [512, 384, 320, 256, 224, 192, 160]),   # config 3's, whole
 ]
 
 

@@ -468,8 +468,12 @@ def test_runner_buffers_are_reused_across_steps():
         _check_param_grads(_param_grads(layers), go, torch.float32, "step %d" % seed)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=str)
-def test_hip_graph_replays_match_eager(dtype):
+@pytest.mark.parametrize("dtype,streams", [
+    (torch.float32, 1), (torch.bfloat16, 1),
+    pytest.param(torch.bfloat16, 3, marks=pytest.mark.skip(
+        reason="HIP-graph capture of the multi-stream step is switched off (TeraPipe raises): the one run of it at "
+               "24 layers x 8 slices ended in a host segmentation fault and no cause was established"))], ids=str)
+def test_hip_graph_replays_match_eager(dtype, streams):
     """use_hip_graph=True: step 1 runs eagerly and records, later steps replay the two graphs.  Several
     replays on different inputs, with eager work and synchronisations of the same process in between,
     each checked against an eager runner on the same layers (bit-identical: same kernels, same order)."""
@@ -478,8 +482,8 @@ def test_hip_graph_replays_match_eager(dtype):
     bs, ss = [1, 1], [32, 48, 16]
     ps = make_params(n_layers, E, Fd, dtype, seed=6)
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps, "gelu")
-    # three slice lanes as well (16 bit): the recorded graphs then hold the cross-stream dependencies
-    graph_runner = ta.TeraPipe(layers, B, L, bs, ss, use_hip_graph=True, slice_streams=3)
+    # (with slice lanes the recorded graphs would also hold the cross-stream dependencies)
+    graph_runner = ta.TeraPipe(layers, B, L, bs, ss, use_hip_graph=True, slice_streams=streams)
     eager_runner = ta.TeraPipe(layers, B, L, bs, ss, slice_streams=1, launch_replay=False)
 
     def step(runner, x, dy):
@@ -592,6 +596,112 @@ def test_latency_measurement_feeds_the_planner():
     grid = lm.fit_latency_grid(samples, 1, L, layers_per_stage=n_layers)
     scheme, latency = lm.best_plan(grid, 1, L, pipelinelen=4)
     assert scheme is not None and sum(scheme[0][1]) == L and latency >= 0 and latency == latency
+
+
+def test_planned_and_uniform_slices_run_as_the_latency_grid_predicts():
+    """Plan -> run -> predicted against measured (the reference's evaluate_split, latency_model.py:155-163) on two
+    layers of the GPT-3 13B width (hidden 5120, 40 heads, FFN 20480, fp16), 1024 positions: the latency grid is
+    measured through the HIP path at slice lengths that are multiples of 64, the planner picks the slices for an
+    8-stage pipeline on that grid, and both its plan and the uniform 4 x 256 plan are then run on this stage; the
+    sum of the grid's slice latencies (pipeline length 1: what one stage spends on a sequence) is within 10 % of the
+    measured step in both cases."""
+    ta = _mods()
+    from terapipe_amd import latency_model as lm
+    dtype = torch.float16
+    n_layers, E, H, Fd, L, step = 2, 5120, 40, 20480, 1024, 64
+    layers = ta.TransformerLayers(n_layers, E, Fd, H, dtype=dtype, device=DEV)
+    g = torch.Generator(device=DEV).manual_seed(3)
+    with torch.no_grad():
+        for p in layers.parameters():
+            if p.dim() == 2:
+                p.copy_((torch.randn(p.shape, generator=g, device=DEV) * 0.02).to(dtype))
+    lens = [64, 128, 192, 256, 320, 384, 448, 512, 640, 768, 1024]
+    samples = lm.measure_layer_latency(layers, 1, L, lens, reps=3)
+    assert all(t > 0 and t == t for t in samples.values())
+    grid = lm.fit_latency_grid(samples, 1, L, layers_per_stage=n_layers, step_gap=step)
+    scheme, planned_latency = lm.best_plan(grid, 1, L, pipelinelen=8, step_gap=step)
+    assert scheme is not None and sum(scheme[0][1]) == L and all(s % step == 0 for s in scheme[0][1])
+    uniform = [256] * 4
+    # the planner's optimum is no worse than the uniform plan on the grid it was given
+    assert planned_latency <= lm.evaluate_split(grid, [(1, uniform)], 8, step_gap=step) * (1 + 1e-9)
+    x = torch.randn(L, 1, E, generator=g, device=DEV).to(dtype)
+    r = torch.randn(L, 1, E, generator=g, device=DEV).to(dtype)
+    for name, slices in (("planned", scheme[0][1]), ("uniform", uniform)):
+        predicted = lm.evaluate_split(grid, [(1, slices)], 1, step_gap=step)
+        runner = ta.TeraPipe(layers, 1, L, [1], slices, slice_streams=1, launch_replay=False)
+        times = []
+        for i in range(5):
+            for p in layers.parameters():
+                p.grad = None
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            (runner(x) * r).sum().backward()
+            e1.record()
+            torch.cuda.synchronize()
+            if i:
+                times.append(e0.elapsed_time(e1) * 1e-3)
+        measured = float(np.median(times))
+        print("%s slices %s: predicted %.3f ms, measured %.3f ms" % (name, slices, predicted * 1e3, measured * 1e3), flush=True)
+        assert abs(predicted - measured) <= 0.10 * measured, \
+            "%s plan %s: predicted %.3f ms, measured %.3f ms" % (name, slices, predicted * 1e3, measured * 1e3)
+
+
+def test_replay_survives_a_larger_workspace_on_the_same_stream():
+    """A recorded step holds its k-split workspaces: a larger k-split GEMM on the same stream between two
+    re-issued steps makes the workspace pool grow, and the re-issued step must still write its partial sums into
+    memory that is its own (results equal to an eager runner's, step by step)."""
+    ta = _mods()
+    from terapipe_amd import _lib as L, ops
+    dtype = torch.float16
+    n_layers, E, H, Fd, Ls, B = 2, 256, 2, 1024, 128, 1
+    ss = [32, 64, 32]
+    ps = make_params(n_layers, E, Fd, dtype, seed=44)
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    fast = ta.TeraPipe(layers, B, Ls, [B], ss, slice_streams=1, launch_replay=True)
+    plain = ta.TeraPipe(layers, B, Ls, [B], ss, slice_streams=1, launch_replay=False)
+
+    def step(runner, seed):
+        g = torch.Generator().manual_seed(seed)
+        x = torch.randn(Ls, B, E, generator=g).to(dtype).to(DEV)
+        dy = (torch.randn(Ls, B, E, generator=g) * 0.1).to(dtype).to(DEV)
+        for p in layers.parameters():
+            p.grad = None
+        xd = x.clone().requires_grad_(True)
+        y = runner(xd)
+        (y * dy).sum().backward()
+        return y.detach().clone(), xd.grad.clone(), [p.grad.clone() for p in layers.parameters()]
+
+    def check(seed, tag):
+        y0, dx0, g0 = step(plain, seed)
+        y1, dx1, g1 = step(fast, seed)
+        torch.cuda.synchronize()
+        assert torch.equal(y1, y0), tag + " y"
+        assert torch.equal(dx1, dx0), tag + " dx"
+        for a, b in zip(g1, g0):
+            assert_close(a, b, dtype, tag + " parameter gradient", 1.0)
+
+    for seed in (1, 2, 3):                 # as written, recorded, re-issued
+        check(seed, "step %d" % seed)
+    assert isinstance(fast._sbufs.fwd_program, list)
+    dev = torch.device(DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    before = ops.Workspace.size(dev, stream)
+    # a k-split product on the same stream that needs more workspace than anything so far
+    M, K, ks = 512, 2048, 8
+    N = max(4096, (before // (ks * M * 4) // 256 + 1) * 256)     # whatever earlier tests left the pool at
+    assert ks * M * N * 4 > before
+    A = (torch.randn(M, K, device=DEV) * K ** -0.5).to(dtype)
+    Bm = torch.randn(N, K, device=DEV).to(dtype)
+    C = torch.empty(M, N, dtype=dtype, device=DEV)
+    ops.gemm(L.TP_GEMM_NT, A, Bm, M, N, K, C=C, ksplit=ks)
+    assert ops.Workspace.size(dev, stream) >= ks * M * N * 4 > before
+    # memory that torch may now hand out: were the old workspace freed, these tensors would land in it
+    junk = [torch.full((before // 4 + 1,), float("nan"), device=DEV) for _ in range(4)]
+    check(4, "re-issued step after the workspace grew")
+    check(5, "second re-issued step after the workspace grew")
+    assert all(torch.isnan(j).all() for j in junk), "a re-issued launch wrote into memory it no longer owns"
+    assert_close(C, A.float() @ Bm.float().t(), dtype, "the large product itself")
 
 
 def test_default_runner_matches_single_stream_at_c2_shape():

@@ -1,5 +1,7 @@
 """Slice planner (tp_plan_slices, host code: runs without a GPU) against the oracle's restatement of
-latency_model.py:97-152 and against exhaustive enumeration on tiny grids."""
+latency_model.py:97-152 and against exhaustive enumeration on tiny grids.  Every test is collected twice, once
+unmarked and once marked `gpu`, so that both the CPU run and the run on the GPU box include it (the planner is
+host code of the same shared library on either machine)."""
 import math
 
 import numpy as np
@@ -7,6 +9,9 @@ import pytest
 
 from oracle import planner_oracle as po
 from terapipe_amd import latency_model as lm
+
+
+BOTH_RUNS = pytest.mark.parametrize("run", [pytest.param("cpu-run"), pytest.param("gpu-box-run", marks=pytest.mark.gpu)])
 
 
 def _grid(B, N, seed, kind="smooth"):
@@ -22,9 +27,10 @@ def _grid(B, N, seed, kind="smooth"):
     return g
 
 
+@BOTH_RUNS
 @pytest.mark.parametrize("B,N,pipe,kind,seed", [(1, 5, 1, "random", 0), (2, 5, 4, "random", 1), (3, 6, 8, "smooth", 2),
                                                 (2, 7, 3, "random", 3), (1, 8, 24, "smooth", 4)])
-def test_planner_matches_oracle_and_brute_force(B, N, pipe, kind, seed):
+def test_planner_matches_oracle_and_brute_force(B, N, pipe, kind, seed, run):
     g = _grid(B, N, seed, kind)
     lat = np.sort(np.unique(g[np.isfinite(g)]))
     for max_latency in (math.inf, float(lat[len(lat) // 2]), float(lat[len(lat) // 4]), float(lat[0]) * 0.5):
@@ -45,15 +51,17 @@ def test_planner_matches_oracle_and_brute_force(B, N, pipe, kind, seed):
         assert final >= po.brute_force_best(g.tolist(), B, N, pipe, max_latency) - 1e-12
 
 
+@BOTH_RUNS
 @pytest.mark.parametrize("B,N,pipe,kind,seed", [(2, 5, 4, "random", 5), (2, 6, 6, "smooth", 6), (1, 7, 12, "random", 7)])
-def test_best_plan_sweep_reaches_the_exhaustive_optimum(B, N, pipe, kind, seed):
+def test_best_plan_sweep_reaches_the_exhaustive_optimum(B, N, pipe, kind, seed, run):
     g = _grid(B, N, seed, kind)
     scheme, latency = lm.best_plan(g, B, N * lm.STEP_GAP, pipe, gap=0.0)
     assert latency == pytest.approx(po.brute_force_best(g.tolist(), B, N, pipe, math.inf), rel=1e-12)
     assert lm.evaluate_split(g, scheme, pipe) == pytest.approx(latency, rel=1e-12)
 
 
-def test_fit_latency_grid_reproduces_a_linear_model():
+@BOTH_RUNS
+def test_fit_latency_grid_reproduces_a_linear_model(run):
     B, S = 2, 64
     truth = lambda b, s, c: 1e-3 + 2e-5 * b * s + (3e-7 * b * s + 1e-7 * b * c + 5e-9 * b * s * c if c else 0.0)
     samples = {(b, s, c): truth(b, s, c) for b in (1, 2) for s in (8, 16, 32, 64) for c in (0, 8, 24, 48) if s + c <= S}
