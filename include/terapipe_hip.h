@@ -5,7 +5,8 @@
  * point below replaces the ATen call(s) the reference makes at the cited lines.  Conventions:
  *   - every pointer is a raw device pointer owned by the caller (PyTorch owns all memory); the
  *     library never allocates or frees device memory and keeps no state between calls
- *     (exception, stated at its declaration: none in this version);
+ *     (one exception, stated at its declaration: tp_gemm_static_ws keeps its k-split partial sums in a
+ *     device array of the library's own);
  *   - `stream` is a hipStream_t passed as void*; launches are asynchronous on it, no internal syncs;
  *   - every function returns 0 on success or a tp_status code; tp_last_error() gives the message of
  *     the calling thread's last failure.  Nothing throws, nothing aborts;
@@ -146,6 +147,19 @@ int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_bytes, void
 int tp_gemm_grouped(const tp_gemm_desc* descs, int n, void* workspace, size_t workspace_bytes, void* stream);
 /* the tile configuration of the single launch tp_gemm_grouped makes for this group; 0 = member by member */
 int tp_gemm_group_cfg(const tp_gemm_desc* descs, int n);
+
+/* tp_gemm for callers that cannot allocate device memory or pass a workspace (code under HIP-graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference: it exists for those
+ * callers only.  The k-split partial sums go to a TP_GEMM_STATIC_WS_BYTES array that the library holds in every
+ * GPU's memory from load to process exit; the call allocates and frees nothing.  Same kernels, same plan, same
+ * result bits as tp_gemm with a caller workspace.  A product whose plan needs more than the array holds is
+ * refused with TP_ERR_WORKSPACE (tp_gemm_workspace_bytes(d) > tp_gemm_static_ws_capacity()), defer_reduce with
+ * TP_ERR_ARG.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two
+ * threads) race on the partial sums; nothing in it needs to start at zero.  The first call on a device looks up
+ * the array's address on that device (the device must be current, as for every launch). */
+#define TP_GEMM_STATIC_WS_BYTES (64u << 20)
+size_t tp_gemm_static_ws_capacity(void);
+int tp_gemm_static_ws(const tp_gemm_desc* d, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Prefix-cached causal attention (attn_helper, transformer_models.py:235-245, with the mask of :220

@@ -102,6 +102,8 @@ SYMBOLS = {
     "tp_gemm_splits": (c_int, [ctypes.POINTER(GemmDesc)]),
     "tp_gemm_workspace_bytes": (c_size_t, [ctypes.POINTER(GemmDesc)]),
     "tp_gemm": (c_int, [ctypes.POINTER(GemmDesc), c_void_p, c_size_t, c_void_p]),
+    "tp_gemm_static_ws_capacity": (c_size_t, []),
+    "tp_gemm_static_ws": (c_int, [ctypes.POINTER(GemmDesc), c_void_p]),
     "tp_gemm_grouped": (c_int, [ctypes.POINTER(GemmDesc), c_int, c_void_p, c_size_t, c_void_p]),
     "tp_gemm_group_cfg": (c_int, [ctypes.POINTER(GemmDesc), c_int]),
     "tp_attn_fwd_workspace_bytes": (c_size_t, [ctypes.POINTER(AttnDesc)]),

@@ -4,6 +4,8 @@
 // (k is the slow dimension: fetched with the gfx950 LDS transpose read), see common.h.
 #include "common.h"
 
+#include <mutex>
+
 namespace tp {
 
 struct GemmArgs {
@@ -1001,6 +1003,65 @@ static void launch_group(const tp_gemm_desc* descs, int n, int cfg, hipStream_t 
     else gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4, true><<<dim3(tiles), 512, 0, s>>>(ga);
 }
 }  // namespace tp
+
+// ---------------------------------------------------------------------------------------------
+// Workspace for callers that cannot allocate (tp_gemm_static_ws): the k-split partial sums go to a
+// file-scope device array instead of a caller's buffer.  In host code the array's name is only a
+// stand-in; its device address is asked for once per device and kept.
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[TP_GEMM_STATIC_WS_BYTES];
+
+namespace tp {
+static constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// device address of `scratch` on the CURRENT device (nullptr + error text on failure)
+static void* scratch_on_current_device() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("tp_gemm_static_ws: hipGetDevice failed or device index %d out of range: %s", dev, hipGetErrorString(e));
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            set_error("tp_gemm_static_ws: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace tp
+
+extern "C" size_t tp_gemm_static_ws_capacity(void) { return (size_t)TP_GEMM_STATIC_WS_BYTES; }
+
+extern "C" int tp_gemm_static_ws(const tp_gemm_desc* d, void* stream) {
+    int rc = tp::validate_gemm(d);
+    if (rc != TP_OK) return rc;
+    if (d->defer_reduce) {
+        tp::set_error("tp_gemm_static_ws: defer_reduce hands the workspace to a later call; use tp_gemm");
+        return TP_ERR_ARG;
+    }
+    tp::GemmPlan p = tp::plan_gemm(d);
+    const size_t need = p.nsplit > 1 ? (size_t)p.nsplit * d->M * d->N * sizeof(float) : 0;
+    if (need > (size_t)TP_GEMM_STATIC_WS_BYTES) {
+        tp::set_error("tp_gemm_static_ws: this product needs %zu bytes of k-split workspace, the built-in one holds %zu "
+                      "(M=%d N=%d K=%d, %d splits); use tp_gemm with a caller workspace",
+                      need, (size_t)TP_GEMM_STATIC_WS_BYTES, d->M, d->N, d->K, p.nsplit);
+        return TP_ERR_WORKSPACE;
+    }
+    void* ws = nullptr;
+    if (need > 0) {
+        ws = tp::scratch_on_current_device();
+        if (!ws) return TP_ERR_LAUNCH;
+    }
+    return tp_gemm(d, ws, need, stream);
+}
 
 extern "C" int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_bytes, void* stream) {
     int rc = tp::validate_gemm(d);
