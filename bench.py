@@ -341,7 +341,8 @@ def attention_grid(device, reps=5):
     (seqlen, attention_cache_len) (terapipe_latency_model.py:180-193): slice length T in {32, 64, 128}, prefix P
     in {0, 256, ..., 1792, 2048 - T} of a 2048-token sequence, head dimension 128, bf16, at the (batch, heads) of
     workloads C5 (2, 48) and C4 (1, 96).  Per point: the forward call, the backward as the sliced runner issues
-    it (delta + dQ against the prefix, then dK/dV of the slice's keys against every later query position), and
+    it (delta + dQ of the slice at P against its prefix, plus the one-pass dK/dV launch of the slice at the
+    mirrored position L - T - P, which covers the same number of query-key blocks), and
     the backward with gradient caches (the reference's per-call contract: dK/dV of all S keys, prefix rows
     read-modify-written).  Each call is timed alone on the chip over `sets` rotating sets of buffers larger
     together than the memory-side cache, replayed from a HIP graph between two HIP events; GB/s are the
@@ -388,8 +389,11 @@ def attention_grid(device, reps=5):
                                         delta=b["delta"][:, P:], q_bh_rows=L, stat_bh_rows=L, dq_only=True)
 
                 def dkdv(b, T=T, P=P):
+                    # the one-pass dK/dV of the slice at the mirrored position L - T - P: it visits as many (query,
+                    # key) blocks as this slice has prefix + diagonal blocks, so over a whole sequence of T-token
+                    # slices the pairs (dQ at P, dK/dV at L - T - P) are exactly the backward launches of a step
                     ops.attn_suffix_dkdv(b["k"], b["v"], b["q"], b["d_o"], b["lse"], b["delta"], b["dqkv"][:T * B], B, H, Dh,
-                                         P, T, L)
+                                         L - T - P, T, L)
 
                 def bwd_cache(b, T=T, P=P):
                     ops.attn_prefix_bwd(b["q"][:, P:], b["k"], b["v"], b["o"][P:P + T], b["lse"][:, P:], b["d_o"][P:P + T],
@@ -401,23 +405,16 @@ def attention_grid(device, reps=5):
                     us[nm] = _graph_ms([(lambda b=b, fn=fn: fn(b)) for b in bufs], reps) * 1e3 / sets
                 fb = attn_bytes_per_call(es, B, H, E, T, P, False)
                 bb = attn_bytes_per_call(es, B, H, E, T, P, True)
+                run_us = us["dq"] + us["dkdv"]
                 rows.append({"P": P, "fwd_us": round(us["fwd"], 2), "fwd_GBps": round(fb / us["fwd"] / 1e3, 1),
-                             "dq_us": round(us["dq"], 2), "dkdv_us": round(us["dkdv"], 2),
+                             "dq_us": round(us["dq"], 2), "dkdv_mirror_us": round(us["dkdv"], 2),
+                             "bwd_runner_us": round(run_us, 2), "bwd_runner_GBps": round(bb / run_us / 1e3, 1),
                              "bwd_cache_us": round(us["bwd_cache"], 2), "bwd_cache_GBps": round(bb / us["bwd_cache"] / 1e3, 1),
                              "fwd_bytes": fb, "bwd_bytes": bb})
             out.append({"heads_of": wl, "batch": B, "heads": H, "T": T, "points": rows})
         del bufs
         gc.collect()
         torch.cuda.empty_cache()
-    # a whole sequence of slices of T tokens visits every P = 0, T, 2T, ...: the dQ call of the slice at P and the
-    # one-pass dK/dV call of the slice at L - T - P do, together, the work the reference's backward of (T, P) does
-    for grp in out:
-        pts = {r["P"]: r for r in grp["points"]}
-        for r in grp["points"]:
-            mirror = pts.get(L - grp["T"] - r["P"])
-            if mirror is not None:
-                r["bwd_runner_us"] = round(r["dq_us"] + mirror["dkdv_us"], 2)
-                r["bwd_runner_GBps"] = round(r["bwd_bytes"] / r["bwd_runner_us"] / 1e3, 1)
     return {"metric": "prefix-attention kernel time and achieved HBM GB/s per (T, P)", "unit": "us, GB/s",
             "dtype": "bf16", "head_dim": Dh, "seq": L, "peak_GBps": PEAK_HBM / 1e9,
             "method": "each call alone on the chip over 6 rotating buffer sets, HIP-graph replay between two HIP events",
