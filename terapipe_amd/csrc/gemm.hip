@@ -2,31 +2,11 @@
 // size 1.  One templated kernel covers the three operand layouts and the three dtypes: an operand is
 // either "k-major" (k contiguous in memory: fetched from LDS with ds_read_b128) or "mn-major"
 // (k is the slow dimension: fetched with the gfx950 LDS transpose read), see common.h.
-#include "common.h"
+#include "gemm_args.h"
 
 #include <mutex>
 
 namespace tp {
-
-struct GemmArgs {
-    const void* A; const void* B; void* C;
-    long lda, ldb, ldc;
-    int M, N, K;
-    int epi;
-    const void* bias;
-    const void* resid; long ldr;
-    const void* aux; long ldaux;
-    void* aux_out; long ldauxo;
-    float* colsum;
-    void* q; void* kc; void* vc;
-    int batch, heads, hd, T, P;
-    long cache_rows;
-    long q_rows;     // rows per (batch, head) block of q
-    float qscale;
-    int kper;        // k extent handled by one split
-    int nsplit;
-    float* partial;  // [nsplit][M][N] fp32 when nsplit > 1
-};
 
 // Several GEMMs of one tile configuration in one launch (unsplit k): workgroup w works on one of the
 // tiles_x[p] x tiles_y[p] tiles of problem p, the last p whose first_tile is <= w.
@@ -39,128 +19,10 @@ struct GemmGroupArgs {
     int n;
 };
 
-__device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
-__device__ __forceinline__ float gelu_erf_grad(float z) {
-    float cdf = 0.5f * (1.0f + erff(z * 0.70710678118654752f));
-    float pdf = 0.3989422804014327f * __expf(-0.5f * z * z);
-    return cdf + z * pdf;
-}
-
-// Applies the epilogue to 8 consecutive columns of one output row (col0 is a multiple of 8) and
-// returns the values written in v (for the column sums).
-template <typename T>
-__device__ __forceinline__ void epilogue_vec8(const GemmArgs& a, int row, int col0, float* v) {
-    typedef Elem<T> E;
-    constexpr int CH = E::CH;          // elements per 16-byte access
-    constexpr int NV = 8 / CH;         // 16-byte accesses per 8 columns
-    auto ld8 = [&](const void* base, long off, float* out) {
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            uint4 raw = *reinterpret_cast<const uint4*>(reinterpret_cast<const T*>(base) + off + i * CH);
-            const T* h = reinterpret_cast<const T*>(&raw);
-#pragma unroll
-            for (int e = 0; e < CH; ++e) out[i * CH + e] = E::to_float(h[e]);
-        }
-    };
-    auto st8 = [&](void* base, long off, const float* in) {
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            uint4 raw;
-            T* h = reinterpret_cast<T*>(&raw);
-#pragma unroll
-            for (int e = 0; e < CH; ++e) h[e] = E::from_float(in[i * CH + e]);
-            *reinterpret_cast<uint4*>(reinterpret_cast<T*>(base) + off + i * CH) = raw;
-        }
-    };
-    float t[8];
-    const long co = (long)row * a.ldc + col0;
-    switch (a.epi) {
-    case TP_EPI_STORE:
-        st8(a.C, co, v);
-        break;
-    case TP_EPI_ACCUMULATE:
-        ld8(a.C, co, t);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) t[e] += v[e];
-        st8(a.C, co, t);
-        break;
-    case TP_EPI_BIAS:
-        ld8(a.bias, col0, t);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] += t[e];
-        st8(a.C, co, v);
-        break;
-    case TP_EPI_BIAS_RELU:
-        ld8(a.bias, col0, t);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { v[e] += t[e]; v[e] = v[e] > 0.f ? v[e] : 0.f; }
-        st8(a.C, co, v);
-        break;
-    case TP_EPI_BIAS_GELU:
-        ld8(a.bias, col0, t);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] += t[e];
-        if (a.aux_out) st8(a.aux_out, (long)row * a.ldauxo + col0, v);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = gelu_erf(v[e]);
-        st8(a.C, co, v);
-        break;
-    case TP_EPI_BIAS_RESIDUAL:
-        ld8(a.bias, col0, t);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] += t[e];
-        ld8(a.resid, (long)row * a.ldr + col0, t);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] += t[e];
-        st8(a.C, co, v);
-        break;
-    case TP_EPI_RELU_GRAD:
-        ld8(a.aux, (long)row * a.ldaux + col0, t);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = t[e] > 0.f ? v[e] : 0.f;
-        st8(a.C, co, v);
-        break;
-    case TP_EPI_GELU_GRAD:
-        ld8(a.aux, (long)row * a.ldaux + col0, t);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] *= gelu_erf_grad(t[e]);
-        st8(a.C, co, v);
-        break;
-    case TP_EPI_QKV_SCATTER: {
-        ld8(a.bias, col0, t);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] += t[e];
-        const int hd3 = 3 * a.hd;
-        const int head = col0 / hd3, w = col0 - head * hd3;
-        const int part = w / a.hd, d = w - part * a.hd;
-        const int tt = row / a.batch, b = row - tt * a.batch;
-        const long bh = (long)b * a.heads + head;
-        if (part == 0) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) t[e] = v[e] * a.qscale;
-            st8(a.q, (bh * a.q_rows + tt) * a.hd + d, t);
-        } else {
-            st8(part == 1 ? a.kc : a.vc, (bh * a.cache_rows + a.P + tt) * a.hd + d, v);
-        }
-        break;
-    }
-    }
-}
-
 // Epilogue shared by the GEMM kernels.  Each wave transposes one 32x32 accumulator block at a time
 // through its own LDS staging block so that a lane ends up with 8 consecutive columns of a row: 16-byte
 // stores and a vector epilogue.  Lane -> (row = lane / 4 + 16 * pass, columns 8 * (lane % 4) .. + 7).
 // `stage_base` must hold 32 * 36 floats per wave and must no longer be read as tile data by any wave.
-// Compile-time loop: the body sees the index as a constant, so arrays indexed by it stay in registers even
-// when the body is too large for the unroller's budget (a rolled loop over the accumulator blocks would put
-// the whole accumulator array in scratch memory, main loop included).
-template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (N > 0) {
-        static_for<N - 1>(f);
-        f(std::integral_constant<int, N - 1>{});
-    }
-}
-
 template <typename T, int TM, int TN, int WM, int WN>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, float16v (&acc)[TM][TN], float* stage_base,
                                               int m0, int n0) {
@@ -706,7 +568,30 @@ static const TileCfg kCfgs[] = {
     {256, 128, 64, 3},   // 18: tall tile, 64 x 128 each
     {256, 256, 64, 2},   // 19: tall tile, 8 waves (4 x 2) of 64 x 128
     {256, 256, 32, 4},   // 20: the same with half the k-tile and twice the stages
+    // 21 and up: the weight-streaming kernel (gemm_stream.hip; NT and NN): whole-slice row tiles of 64 * RB rows,
+    // separate activation / weight rings (stages = the weight ring's)
+    {192, 128, 64, 5},   // 21
+    {256, 128, 64, 4},   // 22
+    {256, 128, 64, 6},   // 23: two activation stages
+    {192, 80, 64, 8},    // 24: NT only
+    {256, 80, 64, 6},    // 25: NT only
+    {128, 128, 64, 7},   // 26
+    {256, 64, 64, 8},    // 27
+    {192, 64, 64, 10},   // 28
+    {256, 128, 64, 4},   // 29: eight waves
+    {192, 128, 64, 5},   // 30: eight waves
+    {192, 128, 64, 5},   // 31: sixteen waves
+    {256, 128, 64, 4},   // 32: sixteen waves
+    {192, 256, 64, 3},   // 33: sixteen waves, 256 columns
+    {256, 256, 64, 3},   // 34: sixteen waves, 256 columns
+    {128, 256, 64, 3},   // 35: sixteen waves
+    {64, 256, 64, 4},    // 36: sixteen waves
+    {128, 128, 64, 7},   // 37: sixteen waves
+    {64, 128, 64, 8},    // 38: sixteen waves
+    {128, 256, 64, 3},   // 39: eight waves
+    {64, 256, 64, 4},    // 40: eight waves
 };
+static constexpr int kFirstStreamCfg = 21;
 static constexpr int kNumCfgs = (int)(sizeof(kCfgs) / sizeof(kCfgs[0]));
 
 // Measured plans: for NT / NN the weight extents (N, K) match exactly and M (tokens of the slice) picks the
@@ -828,6 +713,8 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     if (forced_split) ns = forced_split;
     // the tall tiles load whole k-tiles only, and the 160 / 192 wide ones exist for the k-major weight (NT)
     if (cfg >= 17 && (d->K % 64 || (cfg == 17 && d->op != TP_GEMM_NT))) cfg = 5;
+    // the streaming kernel: NT and NN only; tiles whose width is not a power of two need the k-major weight (NT)
+    if (cfg >= kFirstStreamCfg && (d->op == TP_GEMM_TN || ((cfg == 24 || cfg == 25) && d->op != TP_GEMM_NT))) cfg = 5;
     p.cfg = cfg;
     p.gx = (d->N + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn;
     p.gy = (d->M + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm;
@@ -860,10 +747,14 @@ static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
 
 template <typename T>
 static void launch_gemm(const tp_gemm_desc* d, const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
-    switch (d->op) {
-    case TP_GEMM_NT: launch_cfg<T, true, true>(p, a, s); break;
-    case TP_GEMM_NN: launch_cfg<T, true, false>(p, a, s); break;
-    default: launch_cfg<T, false, false>(p, a, s); break;
+    if (p.cfg >= kFirstStreamCfg) {
+        launch_gemm_stream(p.cfg, d->op, d->dtype, dim3(p.gx, p.gy, p.nsplit), a, s);
+    } else {
+        switch (d->op) {
+        case TP_GEMM_NT: launch_cfg<T, true, true>(p, a, s); break;
+        case TP_GEMM_NN: launch_cfg<T, true, false>(p, a, s); break;
+        default: launch_cfg<T, false, false>(p, a, s); break;
+        }
     }
     if (p.nsplit > 1 && !d->defer_reduce) {
         dim3 grid((d->N + 255) / 256, (d->M + 31) / 32);

@@ -32,6 +32,9 @@ DEFAULT_GEOMETRIES = [
     "6144:24576:64:4096",                                   # 44B shape, 32-token slices x batch 2
 ]
 DMA_CFGS = [3, 5, 8, 10, 11, 12, 13, 17, 18, 19, 20]
+# the weight-streaming kernel's configurations (NT and NN only; 24 and 25 NT only): cfg -> rows of its row tile
+STREAM_CFGS = {21: 192, 22: 256, 24: 192, 25: 256, 26: 128, 29: 256, 30: 192, 31: 192, 32: 256, 33: 192, 34: 256,
+               35: 128, 36: 64, 37: 128, 38: 64}
 SPLITS = [1, 2, 3, 4, 6, 8]
 OPS = {"NT": _lib.TP_GEMM_NT, "NN": _lib.TP_GEMM_NN, "TN": _lib.TP_GEMM_TN}
 
@@ -108,9 +111,12 @@ def sweep(op, M, N, K, dtype, device, log, pair=False):
         time_it = lambda **kw: _time_us(lambda i: ops.gemm(code, A, Bs[i % nb], M, N, K, C=C, **kw))
     auto = time_it()
     results = []
-    for cfg in DMA_CFGS:
+    for cfg in DMA_CFGS + (sorted(STREAM_CFGS) if op != "TN" and K % 64 == 0 else []):
         for ns in SPLITS:
-            if K // ns < 512 or (cfg >= 17 and (M < 192 or K % 64)) or (cfg == 17 and op != "NT"):
+            if K // ns < 512 or (17 <= cfg <= 20 and (M < 192 or K % 64)) or (cfg == 17 and op != "NT"):
+                continue
+            if cfg in STREAM_CFGS and ((cfg in (24, 25) and op != "NT") or STREAM_CFGS[cfg] < M // 2 or
+                                       STREAM_CFGS[cfg] >= 2 * M):
                 continue
             try:
                 t = time_it(tile_cfg=cfg, ksplit=ns)

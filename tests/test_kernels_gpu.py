@@ -112,7 +112,7 @@ def test_gemm_nt_nn_tn(dtype, M, N, K):
         assert_close(W, 2 * ref, dtype, "TN accumulate")
 
 
-TILE_CFGS = [3, 5, 8, 10, 11, 12, 13, 17, 18, 19, 20]
+TILE_CFGS = [3, 5, 8, 10, 11, 12, 13, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
