@@ -78,6 +78,21 @@ int tp_layernorm_bwd_partials(const float* partials, int nsplit, void* dy_out, c
 int tp_ln_param_grads(const void* dy, const void* x, const float* mean, const float* rstd,
                       float* dgamma_acc, float* dbeta_acc, int M, int E, int dtype, void* stream);
 
+/* Every vector-parameter gradient of a layer in one launch: the sums autograd accumulates over the slices of a step
+ * into the four bias .grad (mpu/layers.py:256, :346-347: column sums of the linears' output gradients) and the two
+ * nn.LayerNorm weight / bias .grad pairs (transformer_models.py:275, :280), each taken over ALL rows of the step.
+ * Up to 8 problems; a problem with x == NULL is a column sum (acc0[N] += sum_m dy[m, :]), otherwise the LayerNorm
+ * pair (acc0[N] += sum_m dy * (x - mean) * rstd, acc1[N] += sum_m dy).  fp32 accumulators, added to. */
+typedef struct tp_vecgrad_desc {
+    const void* dy;             /* [M, ld] rows of `dtype` */
+    const void* x;              /* [M, ld] LayerNorm input, or NULL for a column sum */
+    const float* mean; const float* rstd;   /* [M], with x */
+    float* acc0; float* acc1;   /* [N] fp32; acc1 only with x */
+    int64_t ld;
+    int32_t M, N;
+} tp_vecgrad_desc;
+int tp_vec_param_grads(const tp_vecgrad_desc* descs, int n, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * GEMMs that mpu.ColumnParallelLinear / RowParallelLinear reduce to at tensor-parallel size 1
  * (F.linear at mpu/layers.py:256 and :335, and their autograd backward), with the elementwise work
@@ -192,8 +207,8 @@ typedef struct tp_attn_desc {
     float q_scale;
     float* colsum_dqkv_acc;             /* optional [3*H*Dh] fp32: += column sums of dqkv (in_proj bias grad) */
     int32_t reserved;                   /* 0 = automatic; bits 0-7: number of key-range splits of the forward (tuning, tests) */
-    int32_t reserved2;                  /* tuning, tests.  bit 0: the tile-sharing forward kernel with a split/merge pass;
-                                           bit 1 / bit 2: force the eight-wave / the four-wave form of the 16-bit forward kernel */
+    int32_t reserved2;                  /* tuning, tests.  bit 1 / bit 2: force the eight-wave / the four-wave form of the
+                                           16-bit forward kernel */
     int64_t q_bh_rows;                  /* rows per (b,h) block of q: 0 = T; see tp_gemm_desc.q_bh_rows */
     int64_t stat_bh_rows;               /* entries per (b,h) block of lse and delta: 0 = T */
     int32_t dq_only;                    /* backward: 1 = compute delta and the q part of dqkv only; dK/dV of the

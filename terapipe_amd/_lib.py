@@ -73,6 +73,12 @@ class AttnSuffixDesc(ctypes.Structure):
     ]
 
 
+class VecGradDesc(ctypes.Structure):
+    """Mirror of ``tp_vecgrad_desc``."""
+    _fields_ = [("dy", c_void_p), ("x", c_void_p), ("mean", c_void_p), ("rstd", c_void_p),
+                ("acc0", c_void_p), ("acc1", c_void_p), ("ld", c_int64), ("M", c_int32), ("N", c_int32)]
+
+
 class AdamTensor(ctypes.Structure):
     """Mirror of ``tp_adam_tensor``."""
     _fields_ = [("master", c_void_p), ("grad", c_void_p), ("exp_avg", c_void_p), ("exp_avg_sq", c_void_p),
@@ -99,6 +105,7 @@ SYMBOLS = {
     "tp_ln_param_grads": (c_int, [c_void_p] * 6 + [c_int, c_int, c_int, c_void_p]),
     "tp_layernorm_fwd_partials": (c_int, [c_void_p, c_int] + [c_void_p] * 8 + [c_int, c_int, c_float, c_int, c_void_p]),
     "tp_layernorm_bwd_partials": (c_int, [c_void_p, c_int] + [c_void_p] * 11 + [c_int, c_int, c_int, c_void_p]),
+    "tp_vec_param_grads": (c_int, [ctypes.POINTER(VecGradDesc), c_int, c_int, c_void_p]),
     "tp_gemm_splits": (c_int, [ctypes.POINTER(GemmDesc)]),
     "tp_gemm_workspace_bytes": (c_size_t, [ctypes.POINTER(GemmDesc)]),
     "tp_gemm": (c_int, [ctypes.POINTER(GemmDesc), c_void_p, c_size_t, c_void_p]),

@@ -474,425 +474,10 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_kernel(AttnArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// 16-bit kernels with direct global->LDS tile loads and a STAGES-deep ring of LDS tiles
-// (see TileDma in common.h).  Same arithmetic and register layouts as the kernels above; one
-// s_waitcnt vmcnt + s_barrier per tile instead of register staging and two barriers.
+// 16-bit kernels: direct global->LDS tile loads, per-wave rings, 32 x 32 MFMA blocks
 // ------------------------------------------------------------------------------------------------
-
-// One key tile of the forward for one wave: S^T against the tile's NKB * 32 keys, online softmax
-// update of (m, lsum), O^T += V^T P^T.
-template <typename T, int DH, int NKB>
-__device__ __forceinline__ void attn_fwd_tile(const T* sK, const T* sV, const typename Elem<T>::opnd_t* qreg,
-                                              float16v* oacc, float& m, float& lsum, int key0, int P, int tq,
-                                              int lane) {
-    typedef Elem<T> E;
-    constexpr int NDB = DH / 32, NKS = DH / E::KSTEP;
-    const int g = lane >> 5, li = lane & 31;
-    float16v sacc[NKB];
-#pragma unroll
-    for (int kb = 0; kb < NKB; ++kb) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
-        typename E::opnd_t kop[NKS];
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) kop[ks] = fetch_km<T, DH>(sK, kb * 32 + li, ks * E::KSTEP, lane);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) sacc[kb] = E::mfma(kop[ks], qreg[ks], sacc[kb]);
-    }
-    float mt = -INFINITY;
-    if (key0 + NKB * 32 - 1 > P + (tq - li)) {      // wave-uniform: some key of the tile is masked for some row
-#pragma unroll
-        for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                int key = key0 + kb * 32 + acc_row(j, g);
-                float sc = key > P + tq ? -INFINITY : sacc[kb][j];
-                sacc[kb][j] = sc;
-                mt = fmaxf(mt, sc);
-            }
-    } else {
-#pragma unroll
-        for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-            for (int j = 0; j < 16; ++j) mt = fmaxf(mt, sacc[kb][j]);
-    }
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-    const float m_new = fmaxf(m, mt);
-    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = fast_exp2((m - m_safe) * kLog2e);
-    const float mneg = -m_safe * kLog2e;
-    float psum = 0.f;
-#pragma unroll
-    for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            float p = fast_exp2(fmaf(sacc[kb][j], kLog2e, mneg));   // exp(s - m); -inf -> 0
-            sacc[kb][j] = p;
-            psum += p;
-        }
-    lsum = lsum * alpha + psum;
-    m = m_new;
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {   // wave-uniform: some row's running maximum moved
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
-    }
-#pragma unroll
-    for (int kb = 0; kb < NKB; ++kb) mfma_acc_as_b<T, DH>(oacc, sV, kb * 32, sacc[kb], lane);
-}
-
-template <typename T, int DH, int NW, int BN, int STAGES>
-__global__ __launch_bounds__(NW * 64) void attn_fwd_dma_kernel(AttnArgs a) {
-    typedef Elem<T> E;
-    static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
-    constexpr int NT = NW * 64, NKB = BN / 32, NDB = DH / 32, NKS = DH / E::KSTEP;
-    constexpr int TILE = BN * DH;                       // elements of one K or V tile
-    typedef RowSlideDma<T, BN, DH, NT> D;
-    constexpr int NLOAD = 2 * D::N;
-    static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
-    __shared__ __attribute__((aligned(16))) T ring[STAGES * 2 * TILE];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, li = lane & 31;
-    const int bh = blockIdx.y, b = bh / a.H, h = bh - b * a.H;
-    const int T_ = a.T, P = a.P, S = a.P + a.T;
-    const int q0w = (blockIdx.x * NW + wave) * 32;
-    const int tq = q0w + li;
-    const int q_wg_end = min(T_, (int)(blockIdx.x + 1) * NW * 32);
-    const int kv_end = P + q_wg_end;
-    const int ntiles = (kv_end + BN - 1) / BN;
-    const int tps = (ntiles + a.nsplit - 1) / a.nsplit;
-    const int t_beg = blockIdx.z * tps, t_end = min(ntiles, t_beg + tps);
-    const int nt = max(t_end - t_beg, 0);
-
-    typename E::opnd_t qreg[NKS];
-    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), tq < T_, g);
-    wait_vmcnt<0>();   // plain loads done before the counted tile loads start
-
-    float16v oacc[NDB];
-#pragma unroll
-    for (int db = 0; db < NDB; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
-    float m = -INFINITY, lsum = 0.f;
-
-    const T* Kb = reinterpret_cast<const T*>(a.kc) + (long)bh * a.cache_rows * DH;
-    const T* Vb = reinterpret_cast<const T*>(a.vc) + (long)bh * a.cache_rows * DH;
-    D dma;
-    dma.init(DH, tid);
-    auto issue = [&](int it) {
-        // rows past S are clamped to row S-1 (finite, masked); tiles past the range reload the last
-        // rows, which keeps the per-tile load count uniform
-        const int stage = it % STAGES;
-        const int row0 = (t_beg + it) * BN;
-        dma.issue(ring + stage * 2 * TILE, Kb, row0, S, tid);
-        dma.issue(ring + stage * 2 * TILE + TILE, Vb, row0, S, tid);
-    };
-#pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) issue(s);
-    for (int it = 0; it < nt; ++it) {
-        wait_vmcnt<NLOAD * (STAGES - 2)>();
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        issue(it + STAGES - 1);
-        const T* sK = ring + (it % STAGES) * 2 * TILE;
-        const T* sV = sK + TILE;
-        const int key0 = (t_beg + it) * BN;
-        if (q0w < T_ && key0 <= P + q0w + 31)
-            attn_fwd_tile<T, DH, NKB>(sK, sV, qreg, oacc, m, lsum, key0, P, tq, lane);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    }
-    wait_vmcnt<0>();
-
-    const float ltot = lsum + __shfl_xor(lsum, 32, 64);
-    if (tq < T_) {
-        const float inv = ltot > 0.f ? 1.0f / ltot : 0.f;
-        const float lse = ltot > 0.f ? m + logf(ltot) : -INFINITY;
-        if (a.nsplit == 1) {
-            T* O = reinterpret_cast<T*>(a.o) + ((long)tq * a.B + b) * ((long)a.H * DH) + (long)h * DH;
-#pragma unroll
-            for (int db = 0; db < NDB; ++db)
-#pragma unroll
-                for (int jq = 0; jq < 4; ++jq) {
-                    int dh = db * 32 + 8 * jq + 4 * g;
-                    store4<T>(O + dh, oacc[db][4 * jq] * inv, oacc[db][4 * jq + 1] * inv,
-                              oacc[db][4 * jq + 2] * inv, oacc[db][4 * jq + 3] * inv);
-                }
-            if (g == 0) a.lse[(long)bh * a.st_bhs + tq] = lse;
-        } else {
-            const long BH = (long)a.B * a.H;
-            float* PO = a.part_o + (((long)blockIdx.z * BH + bh) * T_ + tq) * DH;
-#pragma unroll
-            for (int db = 0; db < NDB; ++db)
-#pragma unroll
-                for (int jq = 0; jq < 4; ++jq) {
-                    int dh = db * 32 + 8 * jq + 4 * g;
-                    *reinterpret_cast<float4*>(PO + dh) =
-                        make_float4(oacc[db][4 * jq] * inv, oacc[db][4 * jq + 1] * inv,
-                                    oacc[db][4 * jq + 2] * inv, oacc[db][4 * jq + 3] * inv);
-                }
-            if (g == 0) a.part_lse[((long)blockIdx.z * BH + bh) * T_ + tq] = lse;
-        }
-    }
-}
-
-// dQ with the key tiles streamed through the LDS ring.
-template <typename T, int DH, int NW, int BN, int STAGES>
-__global__ __launch_bounds__(NW * 64) void attn_bwd_dq_dma_kernel(AttnArgs a) {
-    typedef Elem<T> E;
-    static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
-    constexpr int NT = NW * 64, NKB = BN / 32, NDB = DH / 32, NKS = DH / E::KSTEP;
-    constexpr int TILE = BN * DH;
-    typedef RowSlideDma<T, BN, DH, NT> D;
-    constexpr int NLOAD = 2 * D::N;
-    static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
-    __shared__ __attribute__((aligned(16))) T ring[STAGES * 2 * TILE];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, li = lane & 31;
-    const int bh = blockIdx.y, b = bh / a.H, h = bh - b * a.H;
-    const int T_ = a.T, P = a.P, S = a.P + a.T;
-    const long EE = (long)a.H * DH;
-    const int q0w = (blockIdx.x * NW + wave) * 32;
-    const int tq = q0w + li;
-    const int q_wg_end = min(T_, (int)(blockIdx.x + 1) * NW * 32);
-    const int kv_end = P + q_wg_end;
-    const int nt = (kv_end + BN - 1) / BN;
-
-    typename E::opnd_t qreg[NKS], doreg[NKS];
-    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), tq < T_, g);
-    load_row_operands<T, DH>(doreg, reinterpret_cast<const T*>(a.d_o) + ((long)tq * a.B + b) * EE + (long)h * DH, tq < T_, g);
-    const float lse_q = tq < T_ ? a.lse[(long)bh * a.st_bhs + tq] : 0.f;
-    const float delta_q = tq < T_ ? a.delta[(long)bh * a.st_bhs + tq] : 0.f;
-    const float lse_neg = -lse_q * kLog2e;
-    wait_vmcnt<0>();
-
-    float16v dq[NDB];
-#pragma unroll
-    for (int db = 0; db < NDB; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
-
-    const T* Kb = reinterpret_cast<const T*>(a.kc) + (long)bh * a.cache_rows * DH;
-    const T* Vb = reinterpret_cast<const T*>(a.vc) + (long)bh * a.cache_rows * DH;
-    D dma;
-    dma.init(DH, tid);
-    auto issue = [&](int it) {
-        const int stage = it % STAGES;
-        dma.issue(ring + stage * 2 * TILE, Kb, it * BN, S, tid);
-        dma.issue(ring + stage * 2 * TILE + TILE, Vb, it * BN, S, tid);
-    };
-#pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) issue(s);
-    for (int it = 0; it < nt; ++it) {
-        wait_vmcnt<NLOAD * (STAGES - 2)>();
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        issue(it + STAGES - 1);
-        const T* sK = ring + (it % STAGES) * 2 * TILE;
-        const T* sV = sK + TILE;
-        const int key0 = it * BN;
-        if (q0w < T_ && key0 <= P + q0w + 31) {
-#pragma unroll
-            for (int kb = 0; kb < NKB; ++kb) {
-                float16v sacc, pacc;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; pacc[r] = 0.f; }
-                typename E::opnd_t kop[NKS], vop[NKS];
-#pragma unroll
-                for (int ks = 0; ks < NKS; ++ks) {
-                    kop[ks] = fetch_km<T, DH>(sK, kb * 32 + li, ks * E::KSTEP, lane);
-                    vop[ks] = fetch_km<T, DH>(sV, kb * 32 + li, ks * E::KSTEP, lane);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int ks = 0; ks < NKS; ++ks) {
-                    sacc = E::mfma(kop[ks], qreg[ks], sacc);
-                    pacc = E::mfma(vop[ks], doreg[ks], pacc);
-                }
-                if (key0 + kb * 32 + 31 > P + q0w) {     // wave-uniform: the block touches the causal boundary
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        int key = key0 + kb * 32 + acc_row(j, g);
-                        float p = key > P + tq ? 0.f : fast_exp2(fmaf(sacc[j], kLog2e, lse_neg));
-                        pacc[j] = p * (pacc[j] - delta_q);
-                    }
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        float p = fast_exp2(fmaf(sacc[j], kLog2e, lse_neg));
-                        pacc[j] = p * (pacc[j] - delta_q);
-                    }
-                }
-                mfma_acc_as_b<T, DH>(dq, sK, kb * 32, pacc, lane);
-            }
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    }
-    wait_vmcnt<0>();
-    if (tq < T_) {
-        T* dst = reinterpret_cast<T*>(a.dqkv) + ((long)tq * a.B + b) * (3 * EE) + (long)h * 3 * DH;
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-            for (int jq = 0; jq < 4; ++jq) {
-                int dh = db * 32 + 8 * jq + 4 * g;
-                store4<T>(dst + dh, dq[db][4 * jq] * a.qscale, dq[db][4 * jq + 1] * a.qscale,
-                          dq[db][4 * jq + 2] * a.qscale, dq[db][4 * jq + 3] * a.qscale);
-            }
-    }
-}
-
-// dK / dV with the query blocks (Q and dO tiles of 32 rows) streamed through the LDS ring; the LSE and
-// delta vectors of the whole slice are staged in LDS once (T <= kMaxTLds).
+// the gradient-cache dK/dV kernel stages the lse / delta vectors of the whole slice in LDS once (T <= kMaxTLds)
 static constexpr int kMaxTLds = 4096;
-
-template <typename T, typename GT, int DH, int NW, int STAGES>
-__global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_dma_kernel(AttnArgs a) {
-    typedef Elem<T> E;
-    static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
-    constexpr int NT = NW * 64, NDB = DH / 32, NKS = DH / E::KSTEP;
-    constexpr int TILE = 32 * DH;
-    typedef RowSlideDma<T, 32, DH, NT> D;
-    constexpr int NLOAD = 2 * D::N;
-    static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
-    __shared__ __attribute__((aligned(16))) T ring[STAGES * 2 * TILE];
-    extern __shared__ __attribute__((aligned(16))) float stats[];   // lse[Tpad], delta[Tpad]
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, li = lane & 31;
-    const int bh = blockIdx.y, b = bh / a.H, h = bh - b * a.H;
-    const int T_ = a.T, P = a.P, S = a.P + a.T;
-    const long EE = (long)a.H * DH;
-    const int key0wg = blockIdx.x * NW * 32;
-    const int key0w = key0wg + wave * 32;
-    const int key = key0w + li;
-    const int nqb = (T_ + 31) / 32;
-    const int Tpad = nqb * 32;
-    float* sLse = stats;
-    float* sDelta = stats + Tpad;
-
-    typename E::opnd_t kreg[NKS], vreg[NKS];
-    load_row_operands<T, DH>(kreg, reinterpret_cast<const T*>(a.kc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
-    load_row_operands<T, DH>(vreg, reinterpret_cast<const T*>(a.vc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
-    for (int t = tid; t < Tpad; t += NT) {
-        sLse[t] = t < T_ ? -a.lse[(long)bh * a.st_bhs + t] * kLog2e : 0.f;     // stored as -lse * log2(e)
-        sDelta[t] = t < T_ ? a.delta[(long)bh * a.st_bhs + t] : 0.f;
-    }
-    wait_vmcnt<0>();
-    __syncthreads();
-
-    float16v dk[NDB], dv[NDB];
-#pragma unroll
-    for (int db = 0; db < NDB; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
-
-    const T* Qb = reinterpret_cast<const T*>(a.q) + (long)bh * a.q_bhs;
-    const T* dOb = reinterpret_cast<const T*>(a.d_o) + (long)b * EE + (long)h * DH;  // row t at stride B*E
-    const int qb_start = key0wg > P ? (key0wg - P) / 32 : 0;
-    const int nt = nqb - qb_start;
-    D dmaq, dmado;
-    dmaq.init(DH, tid);
-    dmado.init((long)a.B * EE, tid);
-    auto issue = [&](int it) {
-        // query rows past T are clamped to row T-1: finite data whose P and dS are forced to zero
-        const int stage = it % STAGES;
-        dmaq.issue(ring + stage * 2 * TILE, Qb, (qb_start + it) * 32, T_, tid);
-        dmado.issue(ring + stage * 2 * TILE + TILE, dOb, (qb_start + it) * 32, T_, tid);
-    };
-#pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) issue(s);
-    for (int it = 0; it < nt; ++it) {
-        wait_vmcnt<NLOAD * (STAGES - 2)>();
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        issue(it + STAGES - 1);
-        const T* sQ = ring + (it % STAGES) * 2 * TILE;
-        const T* sdO = sQ + TILE;
-        const int qb = qb_start + it;
-        if (key0w < S && key0w <= P + qb * 32 + 31) {
-            float16v sacc, pacc;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; pacc[r] = 0.f; }
-            typename E::opnd_t qop[NKS], doop[NKS];
-#pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) {
-                qop[ks] = fetch_km<T, DH>(sQ, li, ks * E::KSTEP, lane);
-                doop[ks] = fetch_km<T, DH>(sdO, li, ks * E::KSTEP, lane);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) {
-                sacc = E::mfma(qop[ks], kreg[ks], sacc);
-                pacc = E::mfma(doop[ks], vreg[ks], pacc);
-            }
-#pragma unroll
-            for (int jq = 0; jq < 4; ++jq) {
-                float4 l4 = *reinterpret_cast<const float4*>(sLse + qb * 32 + 8 * jq + 4 * g);
-                float4 d4 = *reinterpret_cast<const float4*>(sDelta + qb * 32 + 8 * jq + 4 * g);
-                const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
-                const float dl[4] = {d4.x, d4.y, d4.z, d4.w};
-                // wave-uniform: every (query, key) pair of the block is visible and in range
-                const bool all_visible = (qb * 32 + 32 <= T_) && (key0w + 31 <= P + qb * 32) && (key0w + 32 <= S);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    int j = 4 * jq + e;
-                    int t = qb * 32 + 8 * jq + 4 * g + e;
-                    float p = fast_exp2(fmaf(sacc[j], kLog2e, lv[e]));
-                    if (!all_visible) {
-                        bool vis = (t < T_) && (key <= P + t) && (key < S);
-                        p = vis ? p : 0.f;
-                    }
-                    float ds = p * (pacc[j] - dl[e]);
-                    sacc[j] = p;
-                    pacc[j] = ds;
-                }
-            }
-            mfma_acc_as_b<T, DH>(dv, sdO, 0, sacc, lane);
-            mfma_acc_as_b<T, DH>(dk, sQ, 0, pacc, lane);
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    }
-    wait_vmcnt<0>();
-
-    if (key < S) {
-        GT* gK = reinterpret_cast<GT*>(a.gk) + ((long)bh * a.cache_rows + key) * DH;
-        GT* gV = reinterpret_cast<GT*>(a.gv) + ((long)bh * a.cache_rows + key) * DH;
-        if (key < P) {
-#pragma unroll
-            for (int db = 0; db < NDB; ++db)
-#pragma unroll
-                for (int jq = 0; jq < 4; ++jq) {
-                    int dh = db * 32 + 8 * jq + 4 * g;
-                    float ok[4] = {0.f, 0.f, 0.f, 0.f}, ov[4] = {0.f, 0.f, 0.f, 0.f};
-                    if (a.accumulate_prefix) { load4<GT>(gK + dh, ok); load4<GT>(gV + dh, ov); }
-                    store4<GT>(gK + dh, ok[0] + dk[db][4 * jq], ok[1] + dk[db][4 * jq + 1],
-                               ok[2] + dk[db][4 * jq + 2], ok[3] + dk[db][4 * jq + 3]);
-                    store4<GT>(gV + dh, ov[0] + dv[db][4 * jq], ov[1] + dv[db][4 * jq + 1],
-                               ov[2] + dv[db][4 * jq + 2], ov[3] + dv[db][4 * jq + 3]);
-                }
-        } else {
-            const int t = key - P;
-            T* dst = reinterpret_cast<T*>(a.dqkv) + ((long)t * a.B + b) * (3 * EE) + (long)h * 3 * DH;
-#pragma unroll
-            for (int db = 0; db < NDB; ++db)
-#pragma unroll
-                for (int jq = 0; jq < 4; ++jq) {
-                    int dh = db * 32 + 8 * jq + 4 * g;
-                    float ok[4] = {0.f, 0.f, 0.f, 0.f}, ov[4] = {0.f, 0.f, 0.f, 0.f};
-                    if (a.has_incoming) { load4<GT>(gK + dh, ok); load4<GT>(gV + dh, ov); }
-                    store4<T>(dst + DH + dh, ok[0] + dk[db][4 * jq], ok[1] + dk[db][4 * jq + 1],
-                              ok[2] + dk[db][4 * jq + 2], ok[3] + dk[db][4 * jq + 3]);
-                    store4<T>(dst + 2 * DH + dh, ov[0] + dv[db][4 * jq], ov[1] + dv[db][4 * jq + 1],
-                              ov[2] + dv[db][4 * jq + 2], ov[3] + dv[db][4 * jq + 3]);
-                    if (a.zero_slice_rows) {
-                        store4<GT>(gK + dh, 0.f, 0.f, 0.f, 0.f);
-                        store4<GT>(gV + dh, 0.f, 0.f, 0.f, 0.f);
-                    }
-                }
-        }
-    }
-}
 
 // Workgroups are dealt to the eight XCDs round-robin by linear id.  This maps the linear id to
 // (batch*head, block) so that all blocks of one (batch, head) run on the same XCD and its K / V / Q / dO
@@ -1899,7 +1484,7 @@ struct FwdPlan { int nw, bn, nsplit, qblocks; };
 
 static FwdPlan plan_fwd(const tp_attn_desc* d) {
     FwdPlan p;
-    if (d->dtype != TP_F32 && !(d->reserved2 & 1)) {
+    if (d->dtype != TP_F32) {
         // 16-bit: one workgroup per 32 queries whose four waves split the key range and merge in LDS
         p.nw = 0; p.bn = 32; p.nsplit = 1; p.qblocks = (d->T + 31) / 32;
         // bn doubles as the wave count of this kernel: 8 = eight waves with one tile buffer each, faster
@@ -1946,14 +1531,9 @@ template <typename T, int DH>
 static void launch_fwd(const FwdPlan& p, const AttnArgs& a, hipStream_t s) {
     dim3 grid(p.qblocks, a.B * a.H, p.nsplit);
     if constexpr (sizeof(T) == 2) {
-        if (p.nw == 0) {
-            if (p.bn == 8) attn_fwd2_kernel<T, DH, 8, 1><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 512, 0, s>>>(a);
-            else attn_fwd2_kernel<T, DH, 4><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 256, 0, s>>>(a);
-            return;
-        }
-        if (p.nw == 4) attn_fwd_dma_kernel<T, DH, 4, 64, 3><<<grid, 256, 0, s>>>(a);
-        else if (p.nw == 2) attn_fwd_dma_kernel<T, DH, 2, 64, 3><<<grid, 128, 0, s>>>(a);
-        else attn_fwd_dma_kernel<T, DH, 1, 32, 3><<<grid, 64, 0, s>>>(a);
+        if (p.bn == 8) attn_fwd2_kernel<T, DH, 8, 1><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 512, 0, s>>>(a);
+        else attn_fwd2_kernel<T, DH, 4><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 256, 0, s>>>(a);
+        return;
     } else {
         if (p.nw == 4) attn_fwd_kernel<T, DH, 4, 64><<<grid, 256, 0, s>>>(a);
         else if (p.nw == 2) attn_fwd_kernel<T, DH, 2, 64><<<grid, 128, 0, s>>>(a);

@@ -257,32 +257,8 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
 }
 
-template <typename T, int ROWS, int COLS, int NT> struct TileDma {
-    static constexpr int CPR = COLS / 8;
-    static constexpr int TOTAL = ROWS * CPR;
-    static constexpr int N = TOTAL / NT;
-    static_assert(TOTAL % NT == 0 && NT % 64 == 0, "tile must split evenly over the waves");
-    // issues the N loads of this thread for the tile whose first element is (r0, c0)
-    static __device__ __forceinline__ void issue(T* lds, const T* __restrict__ base, long ld, int r0, int c0,
-                                                 int rmax, int cmax, int tid) {
-        const int lane = tid & 63, wave = tid >> 6;
-#pragma unroll
-        for (int i = 0; i < N; ++i) {
-            const int p0 = (i * (NT / 64) + wave) * 64;
-            const int p = p0 + lane;
-            const int row = p / CPR, pc = p % CPR;
-            const int lc = pc ^ swz16<COLS>(row);
-            const int gr = r0 + row, gc = c0 + lc * 8;
-            const void* src = (gr < rmax && gc < cmax) ? (const void*)(base + (long)gr * ld + gc)
-                                                       : (const void*)g_zero_chunk;
-            dma16(src, lds + p0 * 8);
-        }
-    }
-};
-
-// The same tile loads for a tile that slides along one axis in equal steps (the k loop of a GEMM, the
-// key loop of attention): the per-lane source pointers are computed once, every step is one 64-bit add
-// per load.  `ALONG_COLS` says whether the tile slides along its columns (k-major operand) or its rows.
+// Tile loads for a tile that slides along one axis in equal steps (the k loop of a GEMM): the per-lane source
+// pointers are computed once, every step is one 64-bit add per load.  `ALONG_COLS` says whether the tile slides along its columns (k-major operand) or its rows.
 // Lanes whose fixed coordinate is outside the matrix point at the zero chunk with stride 0; the sliding
 // coordinate is checked only on the steps the caller flags as possibly partial.
 template <typename T, int ROWS, int COLS, int NT, bool ALONG_COLS> struct SlidingTileDma {
@@ -338,19 +314,9 @@ template <typename T, int ROWS, int COLS, int NT, bool ALONG_COLS> struct Slidin
     }
 };
 
-// Tile loads for a ROWS x COLS tile (COLS = the full row of the source: no column bound) that slides
-// down the rows of a matrix: the source is a wave-uniform 64-bit base in SGPRs plus a loop-invariant
-// 32-bit per-lane byte offset, so a full tile costs no vector ALU work at all.  Rows at or beyond rmax
-// are CLAMPED to the last valid row instead of zero-filled: the caller must tolerate duplicated (finite)
-// data there -- the attention kernels do, every such row is masked.
-__device__ __forceinline__ void dma16_saddr(unsigned off, const void* sbase, const void* lds_wave_base) {
-    unsigned lds = (unsigned)(unsigned long)(__attribute__((address_space(3))) const void*)lds_wave_base;
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(off), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory");
-}
-
-// The same load with the LDS destination (byte address of the wave's first chunk, wave-uniform) given as
-// an integer, which spares the null check of a generic-to-LDS pointer cast per load.
+// Loads whose source is a wave-uniform 64-bit base in SGPRs plus a 32-bit per-lane byte offset (no vector ALU
+// work for the address), with the LDS destination (byte address of the wave's first chunk, wave-uniform) given
+// as an integer, which spares the null check of a generic-to-LDS pointer cast per load.
 __device__ __forceinline__ unsigned lds_addr(const void* p) {
     return (unsigned)(unsigned long)(__attribute__((address_space(3))) const void*)p;
 }
@@ -410,47 +376,6 @@ template <typename T, int ROWS, int COLS, int NT, bool ALONG_COLS> struct ClampT
         for (int i = 0; i < N; ++i)
             dma16_saddr_lds(off[i], o, lds_bytes + (unsigned)((i * (NT / 64) + wave_uniform) * 512 * (int)sizeof(T)));
         origin += step;
-    }
-};
-
-template <typename T, int ROWS, int COLS, int NT> struct RowSlideDma {
-    static constexpr int CPR = COLS / 8;
-    static constexpr int TOTAL = ROWS * CPR;
-    static constexpr int N = TOTAL / NT;
-    static_assert(TOTAL % NT == 0 && NT % 64 == 0, "tile must split evenly over the waves");
-    unsigned off[N];     // byte offset of this lane's chunk from the tile's first row
-    short row[N];        // its row inside the tile
-    unsigned col_bytes[N];
-    long ld_bytes;
-
-    __device__ __forceinline__ void init(long ld_elems, int tid) {
-        const int lane = tid & 63, wave = tid >> 6;
-        ld_bytes = ld_elems * (long)sizeof(T);
-#pragma unroll
-        for (int i = 0; i < N; ++i) {
-            const int p = (i * (NT / 64) + wave) * 64 + lane;
-            const int r = p / CPR, pc = p % CPR;
-            const int lc = pc ^ swz16<COLS>(r);
-            row[i] = (short)r;
-            col_bytes[i] = (unsigned)(lc * 8 * sizeof(T));
-            off[i] = (unsigned)(r * ld_bytes) + col_bytes[i];
-        }
-    }
-    // loads the tile whose first row is row0 of the matrix at `base` (row 0 of the matrix, wave-uniform)
-    __device__ __forceinline__ void issue(T* lds, const T* base, int row0, int rmax, int tid) const {
-        const int wave = tid >> 6;
-        if (row0 + ROWS <= rmax) {
-            const char* sbase = reinterpret_cast<const char*>(base) + (long)row0 * ld_bytes;
-#pragma unroll
-            for (int i = 0; i < N; ++i) dma16_saddr(off[i], sbase, lds + (i * (NT / 64) + wave) * 512);
-        } else {
-            const int last = rmax > 0 ? rmax - 1 : 0;
-#pragma unroll
-            for (int i = 0; i < N; ++i) {
-                const int r = min(row0 + (int)row[i], last);
-                dma16_saddr((unsigned)(r * ld_bytes) + col_bytes[i], base, lds + (i * (NT / 64) + wave) * 512);
-            }
-        }
     }
 };
 

@@ -543,56 +543,51 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmArgs a) {
 // ---------------------------------------------------------------------------------------------
 static constexpr int kNumCU = 256;  // MI355X
 
-// Tile configurations of the 16-bit direct-to-LDS kernel (4 waves, 2 x 2).  Index 0 is the
-// register-staged kernel (fp32, and the reference point for the others in tests).
+// Tile configurations of the 16-bit kernels by number (the numbers are what the measured plan table, the
+// `reserved` field of tp_gemm_desc and the tuning script refer to; numbers not listed do not exist).
 struct TileCfg { int bm, bn, bk, stages; };
-static const TileCfg kCfgs[] = {
-    {64, 64, 64, 2},     // 0: register-staged kernel's 16-bit tile (fp32 uses 64 x 64 x 16)
-    {64, 64, 64, 2},     // 1: (register-staged kernel)
-    {64, 64, 64, 2},     // 2: (register-staged kernel)
-    {128, 256, 64, 3},   // 3: 8 waves of 64 x 64
-    {64, 64, 64, 2},     // 4: (register-staged kernel)
-    {128, 128, 64, 2},   // 5
-    {64, 64, 64, 2},     // 6: (register-staged kernel)
-    {64, 64, 64, 2},     // 7: (register-staged kernel)
-    {64, 64, 64, 4},     // 8
-    {64, 64, 64, 2},     // 9: (register-staged kernel)
-    {128, 128, 32, 4},   // 10
-    {64, 256, 64, 3},    // 11
-    {64, 64, 128, 4},    // 12
-    {128, 128, 64, 3},   // 13
-    {64, 64, 64, 2},     // 14: (register-staged kernel)
-    {64, 64, 64, 2},     // 15: (register-staged kernel)
-    {64, 64, 64, 2},     // 16: (register-staged kernel)
-    {256, 160, 64, 3},   // 17: tall tile, 4 waves stacked in M, 64 x 160 each (NT only)
-    {256, 128, 64, 3},   // 18: tall tile, 64 x 128 each
-    {256, 256, 64, 2},   // 19: tall tile, 8 waves (4 x 2) of 64 x 128
-    {256, 256, 32, 4},   // 20: the same with half the k-tile and twice the stages
-    // 21 and up: the weight-streaming kernel (gemm_stream.hip; NT and NN): whole-slice row tiles of 64 * RB rows,
-    // separate activation / weight rings (stages = the weight ring's)
-    {192, 128, 64, 5},   // 21
-    {256, 128, 64, 4},   // 22
-    {256, 128, 64, 6},   // 23: two activation stages
-    {192, 80, 64, 8},    // 24: NT only
-    {256, 80, 64, 6},    // 25: NT only
-    {128, 128, 64, 7},   // 26
-    {256, 64, 64, 8},    // 27
-    {192, 64, 64, 10},   // 28
-    {256, 128, 64, 4},   // 29: eight waves
-    {192, 128, 64, 5},   // 30: eight waves
-    {192, 128, 64, 5},   // 31: sixteen waves
-    {256, 128, 64, 4},   // 32: sixteen waves
-    {192, 256, 64, 3},   // 33: sixteen waves, 256 columns
-    {256, 256, 64, 3},   // 34: sixteen waves, 256 columns
-    {128, 256, 64, 3},   // 35: sixteen waves
-    {64, 256, 64, 4},    // 36: sixteen waves
-    {128, 128, 64, 7},   // 37: sixteen waves
-    {64, 128, 64, 8},    // 38: sixteen waves
-    {128, 256, 64, 3},   // 39: eight waves
-    {64, 256, 64, 4},    // 40: eight waves
-};
+static bool tile_cfg(int id, TileCfg& c) {
+    switch (id) {
+    case 0: c = {64, 64, 64, 2}; return true;      // gemm_kernel, register-staged (fp32 runs it with 64 x 64 x 16 tiles)
+    // gemm_dma_kernel: four waves 2 x 2 (configuration 3: eight waves of 64 x 64)
+    case 3: c = {128, 256, 64, 3}; return true;
+    case 5: c = {128, 128, 64, 2}; return true;
+    case 8: c = {64, 64, 64, 4}; return true;
+    case 10: c = {128, 128, 32, 4}; return true;
+    case 11: c = {64, 256, 64, 3}; return true;
+    case 12: c = {64, 64, 128, 4}; return true;
+    case 13: c = {128, 128, 64, 3}; return true;
+    // gemm_tall_kernel: 256-row tiles
+    case 17: c = {256, 160, 64, 3}; return true;   // 4 waves stacked in M, 64 x 160 each (NT only)
+    case 18: c = {256, 128, 64, 3}; return true;   // 64 x 128 each
+    case 19: c = {256, 256, 64, 2}; return true;   // 8 waves (4 x 2) of 64 x 128
+    case 20: c = {256, 256, 32, 4}; return true;   // the same with half the k-tile and twice the stages
+    // gemm_stream_kernel (gemm_stream.hip; NT and NN): whole-slice row tiles of 64 * RB rows, separate activation /
+    // weight rings (stages = the weight ring's); 4 waves unless noted
+    case 21: c = {192, 128, 64, 5}; return true;
+    case 22: c = {256, 128, 64, 4}; return true;
+    case 23: c = {256, 128, 64, 6}; return true;   // two activation stages
+    case 24: c = {192, 80, 64, 8}; return true;    // NT only
+    case 25: c = {256, 80, 64, 6}; return true;    // NT only
+    case 26: c = {128, 128, 64, 7}; return true;
+    case 27: c = {256, 64, 64, 8}; return true;
+    case 28: c = {192, 64, 64, 10}; return true;
+    case 29: c = {256, 128, 64, 4}; return true;   // 8 waves
+    case 30: c = {192, 128, 64, 5}; return true;   // 8 waves
+    case 31: c = {192, 128, 64, 5}; return true;   // 16 waves
+    case 32: c = {256, 128, 64, 4}; return true;   // 16 waves
+    case 33: c = {192, 256, 64, 3}; return true;   // 16 waves
+    case 34: c = {256, 256, 64, 3}; return true;   // 16 waves
+    case 35: c = {128, 256, 64, 3}; return true;   // 16 waves
+    case 36: c = {64, 256, 64, 4}; return true;    // 16 waves
+    case 37: c = {128, 128, 64, 7}; return true;   // 16 waves
+    case 38: c = {64, 128, 64, 8}; return true;    // 16 waves
+    case 39: c = {128, 256, 64, 3}; return true;   // 8 waves
+    case 40: c = {64, 256, 64, 4}; return true;    // 8 waves
+    default: return false;
+    }
+}
 static constexpr int kFirstStreamCfg = 21;
-static constexpr int kNumCfgs = (int)(sizeof(kCfgs) / sizeof(kCfgs[0]));
 
 // Measured plans: for NT / NN the weight extents (N, K) match exactly and M (tokens of the slice) picks the
 // nearest measured M at or above it (at least half of it, so that a much shorter slice falls through to the
@@ -709,16 +704,18 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     if (const TunedPlan* t = find_tuned(d)) { cfg = t->cfg; ns = t->nsplit; }
     if (ns < 1) ns = 1;
     if (ns > 16) ns = 16;
-    if (forced_cfg >= 0 && forced_cfg < kNumCfgs) cfg = forced_cfg;
+    TileCfg tc;
+    if (forced_cfg >= 0 && tile_cfg(forced_cfg, tc)) cfg = forced_cfg;
     if (forced_split) ns = forced_split;
     // the tall tiles load whole k-tiles only, and the 160 / 192 wide ones exist for the k-major weight (NT)
     if (cfg >= 17 && (d->K % 64 || (cfg == 17 && d->op != TP_GEMM_NT))) cfg = 5;
     // the streaming kernel: NT and NN only; tiles whose width is not a power of two need the k-major weight (NT)
     if (cfg >= kFirstStreamCfg && (d->op == TP_GEMM_TN || ((cfg == 24 || cfg == 25) && d->op != TP_GEMM_NT))) cfg = 5;
     p.cfg = cfg;
-    p.gx = (d->N + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn;
-    p.gy = (d->M + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm;
-    finish_plan(d, p, kCfgs[cfg].bk, ns);
+    tile_cfg(cfg, tc);
+    p.gx = (d->N + tc.bn - 1) / tc.bn;
+    p.gy = (d->M + tc.bm - 1) / tc.bm;
+    finish_plan(d, p, tc.bk, ns);
     return p;
 }
 
@@ -879,8 +876,10 @@ static void launch_group(const tp_gemm_desc* descs, int n, int cfg, hipStream_t 
     for (int i = 0; i < n; ++i) {
         GemmPlan p;                 // every member on the group's tiles, its whole k in one piece
         p.cfg = cfg;
-        p.gx = (descs[i].N + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn;
-        p.gy = (descs[i].M + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm;
+        TileCfg tc;
+        tile_cfg(cfg, tc);
+        p.gx = (descs[i].N + tc.bn - 1) / tc.bn;
+        p.gy = (descs[i].M + tc.bm - 1) / tc.bm;
         p.kper = descs[i].K; p.nsplit = 1;
         ga.g[i] = fill_args(&descs[i], p, nullptr);
         ga.first_tile[i] = tiles;

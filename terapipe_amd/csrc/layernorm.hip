@@ -272,6 +272,82 @@ __global__ __launch_bounds__(256) void ln_param_grads_kernel(const T* __restrict
     }
 }
 
+// The vector-parameter gradients of a layer in ONE launch: up to kVecGradMax reductions over the rows of a step,
+// each either column sums of dy (a bias gradient) or the LayerNorm pair (dgamma += sum dy * xhat, dbeta += sum dy).
+// A block of 256 threads = 32 column chunks (8 columns, 16-byte loads for 16-bit types) x 8 row lanes covers
+// 256 columns x kVecGradRows rows of one problem; the row lanes are combined in LDS and every column then costs one
+// atomic per block.  Blocks are numbered problem by problem (first_block[]).
+constexpr int kVecGradMax = 8;
+constexpr int kVecGradRows = 128;
+struct VecGradProblem {
+    const void* dy; const void* x; const float* mean; const float* rstd;
+    float* acc0; float* acc1;
+    long ld; int M, N;
+};
+struct VecGradArgs {
+    VecGradProblem p[kVecGradMax];
+    int first_block[kVecGradMax + 1];
+    int n;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void vec_param_grads_kernel(VecGradArgs args) {
+    __shared__ float sg[8][256], sb[8][256];
+    int pi = 0;
+#pragma unroll
+    for (int i = 1; i < kVecGradMax; ++i)
+        if (i < args.n && (int)blockIdx.x >= args.first_block[i]) pi = i;
+    // (constant indices only: a dynamically indexed kernel argument would be copied to scratch memory)
+    VecGradProblem pr = args.p[0];
+    int first = args.first_block[0];
+#pragma unroll
+    for (int i = 1; i < kVecGradMax; ++i)
+        if (pi == i) { pr = args.p[i]; first = args.first_block[i]; }
+    const int ncb = (pr.N + 255) / 256;
+    const int local = (int)blockIdx.x - first;
+    const int cb = local % ncb, rb = local / ncb;
+    const int cl = threadIdx.x & 31, rl = threadIdx.x >> 5;
+    const int col0 = (cb * 32 + cl) * 8;
+    const int r0 = rb * kVecGradRows, r1 = min(pr.M, r0 + kVecGradRows);
+    const T* dy = reinterpret_cast<const T*>(pr.dy);
+    const T* x = reinterpret_cast<const T*>(pr.x);
+    float ag[8], ab[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { ag[e] = 0.f; ab[e] = 0.f; }
+    if (col0 < pr.N) {
+        for (int row = r0 + rl; row < r1; row += 8) {
+            float d[8];
+            load_chunk<T>(dy + (long)row * pr.ld + col0, d);
+            if constexpr (sizeof(T) == 4) load_chunk<T>(dy + (long)row * pr.ld + col0 + 4, d + 4);
+            if (x) {
+                const float mu = pr.mean[row], rs = pr.rstd[row];
+                float xv[8];
+                load_chunk<T>(x + (long)row * pr.ld + col0, xv);
+                if constexpr (sizeof(T) == 4) load_chunk<T>(x + (long)row * pr.ld + col0 + 4, xv + 4);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ag[e] += d[e] * (xv[e] - mu) * rs;
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ab[e] += d[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { sg[rl][cl * 8 + e] = ag[e]; sb[rl][cl * 8 + e] = ab[e]; }
+    __syncthreads();
+    const int c = threadIdx.x, col = cb * 256 + c;
+    if (col < pr.N) {
+        float tg = 0.f, tb = 0.f;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) { tg += sg[r][c]; tb += sb[r][c]; }
+        if (x) {
+            atomicAdd(pr.acc0 + col, tg);
+            atomicAdd(pr.acc1 + col, tb);
+        } else {
+            atomicAdd(pr.acc0 + col, tb);
+        }
+    }
+}
+
 static int ln_geometry(int E, int dtype, int* threads, int* maxc) {
     const int ch = dtype == TP_F32 ? 4 : 8;
     if (E <= 0 || E % ch) { set_error("layernorm: E=%d must be a positive multiple of %d", E, ch); return TP_ERR_UNSUPPORTED; }
@@ -414,4 +490,34 @@ extern "C" int tp_ln_param_grads(const void* dy, const void* x, const float* mea
     default: ln_param_grads_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)dy, (const bf16*)x, mean, rstd, dgamma_acc, dbeta_acc, M, E); break;
     }
     return check_launch("tp_ln_param_grads");
+}
+
+extern "C" int tp_vec_param_grads(const tp_vecgrad_desc* descs, int n, int dtype, void* stream) {
+    using namespace tp;
+    if (!descs || n < 1 || n > kVecGradMax) { set_error("tp_vec_param_grads: 1 to %d problems (n=%d)", kVecGradMax, n); return TP_ERR_ARG; }
+    if (dtype < TP_F32 || dtype > TP_BF16) { set_error("tp_vec_param_grads: bad dtype %d", dtype); return TP_ERR_ARG; }
+    VecGradArgs args;
+    int blocks = 0;
+    for (int i = 0; i < n; ++i) {
+        const tp_vecgrad_desc& d = descs[i];
+        if (!d.dy || !d.acc0 || d.M <= 0 || d.N <= 0 || d.N % 8 || d.ld < d.N || d.ld % 8) {
+            set_error("tp_vec_param_grads: problem %d: null pointer or bad shape (M=%d N=%d ld=%ld; N and ld multiples of 8)", i, d.M, d.N, (long)d.ld);
+            return TP_ERR_ARG;
+        }
+        if (d.x && (!d.mean || !d.rstd || !d.acc1)) { set_error("tp_vec_param_grads: problem %d: the LayerNorm pair needs mean, rstd and acc1", i); return TP_ERR_ARG; }
+        if (((uintptr_t)d.dy | (uintptr_t)d.x) & 15) { set_error("tp_vec_param_grads: problem %d: pointers must be 16-byte aligned", i); return TP_ERR_ARG; }
+        args.p[i] = {d.dy, d.x, d.mean, d.rstd, d.acc0, d.acc1, (long)d.ld, d.M, d.N};
+        args.first_block[i] = blocks;
+        blocks += ((d.N + 255) / 256) * ((d.M + kVecGradRows - 1) / kVecGradRows);
+    }
+    for (int i = n; i < kVecGradMax; ++i) { args.p[i] = args.p[0]; args.first_block[i] = blocks; }
+    args.first_block[kVecGradMax] = blocks;
+    args.n = n;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    switch (dtype) {
+    case TP_F32: vec_param_grads_kernel<float><<<blocks, 256, 0, s>>>(args); break;
+    case TP_F16: vec_param_grads_kernel<f16><<<blocks, 256, 0, s>>>(args); break;
+    default: vec_param_grads_kernel<bf16><<<blocks, 256, 0, s>>>(args); break;
+    }
+    return check_launch("tp_vec_param_grads");
 }

@@ -348,6 +348,28 @@ def ln_param_grads(dy, x2d, mean, rstd, dgamma_acc, dbeta_acc):
         _record("ln_param_grads", (M, E), lambda s=None: lib.tp_ln_param_grads(*a, _on(s)))
 
 
+def vec_param_grads(problems):
+    """Up to 8 reductions over the rows of a step in one launch.  problems: (dy, acc) for a column sum
+    (acc[N] += sum_m dy[m]) or (dy, x, mean, rstd, dgamma_acc, dbeta_acc) for a LayerNorm pair; every dy / x is a
+    2-D row-major tensor of one dtype, the accumulators are fp32."""
+    n = len(problems)
+    descs = (_lib.VecGradDesc * n)()
+    for d, pr in zip(descs, problems):
+        dy = pr[0]
+        _require_cuda(*pr)
+        d.dy, d.ld, d.M, d.N = dy.data_ptr(), dy.stride(0), dy.shape[0], dy.shape[1]
+        if len(pr) == 2:
+            d.acc0 = pr[1].data_ptr()
+        else:
+            _, x, mean, rstd, dg, db = pr
+            assert x.stride(0) == dy.stride(0)
+            d.x, d.mean, d.rstd, d.acc0, d.acc1 = x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), dg.data_ptr(), db.data_ptr()
+    lib = _lib.load()
+    dt = tp_dtype(problems[0][0].dtype)
+    _lib.check(lib.tp_vec_param_grads(descs, n, dt, _stream()), "tp_vec_param_grads")
+    _record("vec_param_grads", n, lambda s=None: lib.tp_vec_param_grads(descs, n, dt, _on(s)))
+
+
 def accum_cast(dst, src_f32, accumulate):
     _require_cuda(dst, src_f32)
     lib = _lib.load()

@@ -409,14 +409,13 @@ def _param_grads_layer(runner, bufs, l):
             sinks.append(bufs.wgrad_descs.setdefault((l, name), []) if bufs.recording else None)
             items.append((TP_GEMM_TN, dy, xin, n_out, n_in, R, g[name], epi))
         ops.gemm_grouped(items, sinks)
-        ops.colsum_acc(pb["dqkv"][l], sv["attn.in_proj.bias"])
-        ops.colsum_acc(pb["dh"][l], sv["attn.out_proj.bias"])
-        ops.colsum_acc(pb["dz1"][l], sv["fc1.bias"])
-        ops.colsum_acc(dy_out, sv["fc2.bias"])
-        ops.ln_param_grads(pb["dxn"][l], pb["x"][l], pb["mean1"][l], pb["rstd1"][l], sv["attn_ln.weight"],
-                           sv["attn_ln.bias"])
-        ops.ln_param_grads(pb["dhn"][l], pb["h"][l], pb["mean2"][l], pb["rstd2"][l], sv["fc_ln.weight"],
-                           sv["fc_ln.bias"])
+        # the eight vector-parameter gradients of the layer (four bias column sums, two LayerNorm pairs): one launch
+        ops.vec_param_grads([(pb["dqkv"][l], sv["attn.in_proj.bias"]),
+                             (pb["dh"][l], sv["attn.out_proj.bias"]),
+                             (pb["dz1"][l], sv["fc1.bias"]),
+                             (dy_out, sv["fc2.bias"]),
+                             (pb["dxn"][l], pb["x"][l], pb["mean1"][l], pb["rstd1"][l], sv["attn_ln.weight"], sv["attn_ln.bias"]),
+                             (pb["dhn"][l], pb["h"][l], pb["mean2"][l], pb["rstd2"][l], sv["fc_ln.weight"], sv["fc_ln.bias"])])
 
 
 def _timing_event(stream):

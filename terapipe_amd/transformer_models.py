@@ -302,10 +302,14 @@ class MultiheadLMAttentionWithCache(nn.Module):
 
     def __init__(self, embed_dim, num_heads, bias=True, device="cpu"):
         super().__init__()
-        assert bias, "the kernels fuse the projection biases; bias=False is not supported"
         self.embed_dim = embed_dim
         self.in_proj = ColumnParallelLinear(embed_dim, 3 * embed_dim, bias=bias, gather_output=False, device=device)
         self.out_proj = RowParallelLinear(embed_dim, embed_dim, bias=bias, input_is_parallel=True, device=device)
+        if not bias:
+            # the projection kernels fuse a bias: without one (reference transformer_models.py:197, :202-203)
+            # they are given zeros, which are no parameters and appear in no state dict
+            self.register_buffer("_no_in_bias", torch.zeros(3 * embed_dim, device=device), persistent=False)
+            self.register_buffer("_no_out_bias", torch.zeros(embed_dim, device=device), persistent=False)
         self.num_heads = num_heads
         self.head_dim = embed_dim // num_heads
         assert self.head_dim * num_heads == self.embed_dim, "embed_dim must be divisible by num_heads"
@@ -321,8 +325,10 @@ class MultiheadLMAttentionWithCache(nn.Module):
             k, v = _check_cache(full_cache, bsz, self.num_heads, self.head_dim, cache_len + tgt_len, x.dtype)
         else:
             assert cache_len == 0
-        res = _AttentionFunction.apply(self.num_heads, cache_len, x, k, v, self.in_proj.weight, self.in_proj.bias,
-                                       self.out_proj.weight, self.out_proj.bias)
+        b_in = self.in_proj.bias if self.in_proj.bias is not None else self._no_in_bias
+        b_out = self.out_proj.bias if self.out_proj.bias is not None else self._no_out_bias
+        res = _AttentionFunction.apply(self.num_heads, cache_len, x, k, v, self.in_proj.weight, b_in,
+                                       self.out_proj.weight, b_out)
         if full_cache is not None:
             return res[0], (res[1], res[2])
         return res, None

@@ -47,6 +47,7 @@ int main(void) {
          offsetof(tp_attn_suffix_desc, dqkv));
   printf("%zu %zu %zu %zu\n", sizeof(tp_adam_tensor), offsetof(tp_adam_tensor, n), sizeof(tp_adam_desc),
          offsetof(tp_adam_desc, tensors));
+  printf("%zu %zu %zu\n", sizeof(tp_vecgrad_desc), offsetof(tp_vecgrad_desc, ld), offsetof(tp_vecgrad_desc, N));
   return 0;
 }'''
     with tempfile.TemporaryDirectory() as d:
@@ -60,7 +61,8 @@ int main(void) {
                    A.colsum_dqkv_acc.offset, G.defer_reduce.offset, A.dq_only.offset, A.stat_bh_rows.offset,
                    ctypes.sizeof(S), S.q_all.offset, S.dqkv.offset,
                    ctypes.sizeof(_lib.AdamTensor), _lib.AdamTensor.n.offset, ctypes.sizeof(_lib.AdamDesc),
-                   _lib.AdamDesc.tensors.offset]
+                   _lib.AdamDesc.tensors.offset,
+                   ctypes.sizeof(_lib.VecGradDesc), _lib.VecGradDesc.ld.offset, _lib.VecGradDesc.N.offset]
 
 
 def test_argument_errors_without_gpu(lib):

@@ -157,6 +157,43 @@ def test_attention_module_alone(dtype):
         assert_close(layers.layers[0].param_dict()[n].grad, p32[n].grad, dtype, n)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_attention_module_without_bias(dtype):
+    """MultiheadLMAttentionWithCache(bias=False) (reference transformer_models.py:197, :202-203): no bias
+    parameters, no bias keys in the state dict, and the projections compute X W^T alone -- against the oracle
+    with zero biases."""
+    ta = _mods()
+    T, B, H, Dh, P, L = 24, 2, 2, 64, 40, 64
+    E = H * Dh
+    ps = make_params(1, E, 4 * E, dtype, seed=19)
+    for n in ("attn.in_proj.bias", "attn.out_proj.bias"):
+        ps[0][n] = torch.zeros_like(ps[0][n])
+    g = torch.Generator().manual_seed(14)
+    x, dy = torch.randn(T, B, E, generator=g).to(dtype), torch.randn(T, B, E, generator=g).to(dtype)
+    kc0, vc0 = torch.randn(B * H, L, Dh, generator=g).to(dtype), torch.randn(B * H, L, Dh, generator=g).to(dtype)
+    p32 = {k: v.clone().requires_grad_(True) for k, v in ps[0].items()}
+    xo = x.float().clone().requires_grad_(True)
+    ko, vo = kc0.float().clone().requires_grad_(True), vc0.float().clone().requires_grad_(True)
+    yo, _ = oracle.attention_forward(p32, "attn.", xo, H, (ko, vo), P)
+    yo.backward(dy.float())
+    attn = ta.MultiheadLMAttentionWithCache(E, H, bias=False, device=DEV).to(dtype)
+    assert sorted(attn.state_dict()) == ["in_proj.weight", "out_proj.weight"]
+    assert [n for n, _ in attn.named_parameters()] == ["in_proj.weight", "out_proj.weight"]
+    with torch.no_grad():
+        attn.in_proj.weight.copy_(ps[0]["attn.in_proj.weight"].to(dtype))
+        attn.out_proj.weight.copy_(ps[0]["attn.out_proj.weight"].to(dtype))
+    xd = x.to(DEV).requires_grad_(True)
+    kd, vd = kc0.to(DEV).clone().requires_grad_(True), vc0.to(DEV).clone().requires_grad_(True)
+    y, (k_out, v_out) = attn(xd, (kd, vd), P)
+    y.backward(dy.to(DEV))
+    assert_close(y, yo, dtype, "attn y")
+    assert_close(xd.grad, xo.grad, dtype, "attn dx")
+    assert_close(kd.grad, ko.grad, dtype, "attn d k_cache")
+    assert_close(vd.grad, vo.grad, dtype, "attn d v_cache")
+    assert_close(attn.in_proj.weight.grad, p32["attn.in_proj.weight"].grad, dtype, "d in_proj.weight")
+    assert_close(attn.out_proj.weight.grad, p32["attn.out_proj.weight"].grad, dtype, "d out_proj.weight")
+
+
 def _reference_style_loop(layers, x, dy, batch_slices, seq_slices):
     """The slice loop of the reference's TeraPipe.forward + TeraPipeBackwardPassHook.backward
     (terapipe.py:249-264, :182-191) driven through the layer-level autograd surface."""
