@@ -172,6 +172,33 @@ def cpu_baseline(w, sample_layers=None):
                       "(%.1f s), scaled by the layer count" % (sample_layers, w["n_layers"], dt)}
 
 
+def vendor_gemm_us(metas, dtype, device):
+    """{meta: microseconds} of torch.matmul on the products of each recorded GEMM call (a grouped call: its members
+    one after the other), each alone on the chip, weights rotating over several buffers."""
+    out = {}
+    for meta in metas:
+        members = meta if isinstance(meta[0], tuple) else (meta,)
+        fns = []
+        keep = []
+        for (op, M, N, K) in members:
+            nb = max(2, min(6, int(1.0e9 // (N * K * 2))))
+            if op == 2:      # TN: C[M, N] = A[K, M]^T B[K, N]
+                A = torch.randn(K, M, device=device, dtype=dtype)
+                Bs = [torch.randn(K, N, device=device, dtype=dtype) for _ in range(2)]
+                C = torch.empty(M, N, device=device, dtype=dtype)
+                fns += [(lambda A=A, B=B, C=C: torch.matmul(A.t(), B, out=C)) for B in Bs]
+            else:
+                A = torch.randn(M, K, device=device, dtype=dtype)
+                Bs = [torch.randn((N, K) if op == 0 else (K, N), device=device, dtype=dtype) for _ in range(nb)]
+                C = torch.empty(M, N, device=device, dtype=dtype)
+                fns += [(lambda A=A, B=B, C=C, op=op: torch.matmul(A, B.t() if op == 0 else B, out=C)) for B in Bs]
+            keep.append((A, Bs, C))
+        n_rounds = len(fns) // len(members) if len(members) > 1 else len(fns)
+        out[meta] = _graph_ms(fns) * 1e3 / (n_rounds if len(members) == 1 else 2)
+        del keep, fns
+    return out
+
+
 def _graph_ms(fns, reps=3):
     """Average milliseconds of one pass over `fns` (callables that launch on the current stream): the pass is
     captured into a HIP graph and the replays are bracketed by two HIP events on that stream, so no host
@@ -267,6 +294,7 @@ def measure_workload(name, args, device, detail):
         groups = {}
         for c in gemm_calls:
             groups.setdefault(c[1], []).append(c[2])
+        groups = dict(sorted(groups.items(), key=lambda kv: str(kv[0])))
         per = []
         for meta, fns in groups.items():
             ms = _graph_ms(fns)
@@ -277,6 +305,17 @@ def measure_workload(name, args, device, detail):
                         "tflops": round(f / us / 1e6, 1), "bound_us": round(bound_us, 2),
                         "bound": "mfma" if f / peak >= b / PEAK_HBM else "hbm",
                         "frac_of_bound": round(bound_us / us, 3)})
+        if not args.no_vendor_gemm:
+            # context only: the vendor library (hipBLASLt / rocBLAS behind torch.matmul) on the same products, plain
+            # (no fused epilogue), timed the same way over weights that rotate through more memory than the caches hold
+            vend = vendor_gemm_us(list(groups), TORCH_DTYPE[w["dtype"]], device)
+            vt = 0.0
+            for r, meta in zip(per, groups):
+                r["vendor_us"] = round(vend[meta], 2)
+                vt += vend[meta] * r["calls"]
+            roof["vendor_library"] = {"kernel_ms_per_step": vt * 1e-3, "achieved": flops / (vt * 1e-6) / 1e12,
+                                      "frac": flops / (vt * 1e-6) / peak,
+                                      "note": "torch.matmul on the same (op, M, N, K) list, plain products, context only"}
         per.sort(key=lambda r: -r["avg_us"] * r["calls"])
         roof["per_gemm"] = per
     if args.slice_streams > 1:
@@ -450,6 +489,8 @@ def main():
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="with the default workload C3 the line also carries the prefix-attention roofline measured on C5 "
                          "(32-token slices) and short figures for C2, C4 and C5; this leaves them out")
+    ap.add_argument("--no-vendor-gemm", action="store_true",
+                    help="leave out the vendor library's times on the same GEMM shapes (context beside the per-GEMM table)")
     ap.add_argument("--attention-grid", action="store_true",
                     help="print the (T, P) micro-grid of the prefix-attention kernels instead of the step benchmark")
     ap.add_argument("--copy-calibration", action="store_true",

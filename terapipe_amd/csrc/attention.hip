@@ -816,27 +816,6 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq2_kernel(AttnArgs a) {
     T* ring = reinterpret_cast<T*>(smem) + wave * (WAVE_RING / 2);
     const unsigned ring_lds = lds_addr(smem) + wave * WAVE_RING;
 
-    typename E::opnd_t qreg[NKS], doreg[NKS];
-    const long orow = ((long)tq * a.B + b) * EE + (long)h * DH;
-    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), qok, g);
-    load_row_operands<T, DH>(doreg, reinterpret_cast<const T*>(a.d_o) + orow, qok, g);
-    float delta_q;
-    {
-        typename E::opnd_t oreg[NKS];
-        load_row_operands<T, DH>(oreg, reinterpret_cast<const T*>(a.o) + orow, qok, g);
-        float s = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) {
-            const T* x = reinterpret_cast<const T*>(&oreg[ks]);
-            const T* y = reinterpret_cast<const T*>(&doreg[ks]);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) s = fmaf(E::to_float(x[e]), E::to_float(y[e]), s);
-        }
-        delta_q = s + __shfl_xor(s, 32, 64);
-    }
-    if (wave == 0 && g == 0 && qok) a.delta[(long)bh * a.st_bhs + tq] = delta_q;
-    const float lse_neg = qok ? -a.lse[(long)bh * a.st_bhs + tq] * kLog2e : 0.f;
-
     // lane-constant LDS addresses inside stage 0's K tile
     const T* pkm[NKS];
 #pragma unroll
@@ -896,8 +875,31 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq2_kernel(AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
 
-    wait_vmcnt<0>();                     // the row operands are in; tile loads are counted from here
+    // the first tile's loads go out before the query-side rows are asked for, so that the two round trips overlap
+    // (vector-memory operations complete in issue order: the first wait in the loop covers both)
     if (nt > 0) issue(0, t_beg);
+    typename E::opnd_t qreg[NKS], doreg[NKS];
+    const long orow = ((long)tq * a.B + b) * EE + (long)h * DH;
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), qok, g);
+    load_row_operands<T, DH>(doreg, reinterpret_cast<const T*>(a.d_o) + orow, qok, g);
+    float delta_q;
+    {
+        typename E::opnd_t oreg[NKS];
+        load_row_operands<T, DH>(oreg, reinterpret_cast<const T*>(a.o) + orow, qok, g);
+        float s = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            const T* x = reinterpret_cast<const T*>(&oreg[ks]);
+            const T* y = reinterpret_cast<const T*>(&doreg[ks]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s = fmaf(E::to_float(x[e]), E::to_float(y[e]), s);
+        }
+        delta_q = s + __shfl_xor(s, 32, 64);
+    }
+    if (wave == 0 && g == 0 && qok) a.delta[(long)bh * a.st_bhs + tq] = delta_q;
+    const float lse_neg = qok ? -a.lse[(long)bh * a.st_bhs + tq] * kLog2e : 0.f;
+
+
     auto step = [&](auto stage_c, int it) {
         constexpr int s = decltype(stage_c)::value;
         // the other stage was last read one iteration ago (lgkmcnt(0) below): refill it, then wait
@@ -1032,9 +1034,6 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
     T* ring = reinterpret_cast<T*>(smem) + wave * (WAVE_RING / 2);
     const unsigned ring_lds = lds_addr(smem) + wave * WAVE_RING;
 
-    typename E::opnd_t qreg[NKS];
-    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), qok, g);
-
     const T* pkm[NKS];
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) pkm[ks] = ring + km_offset<T, DH>(li, ks * 16, lane);
@@ -1094,13 +1093,16 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
         for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
     float m = -INFINITY, lsum = 0.f;
 
-    wait_vmcnt<0>();
-    if (STG == 2 && nt > 0) issue(0, t_beg);
+    // the first tile's loads go out before the query rows are asked for, so that the two round trips overlap
+    // (vector-memory operations complete in issue order: the first wait in the loop covers both)
+    if (nt > 0) issue(0, t_beg);
+    typename E::opnd_t qreg[NKS];
+    load_row_operands<T, DH>(qreg, reinterpret_cast<const T*>(a.q) + ((long)bh * a.q_bhs + (long)tq * DH), qok, g);
 
     auto step = [&](auto stage_c, int it) {
         constexpr int s = decltype(stage_c)::value;
         if constexpr (STG == 1) {
-            issue(0, t_beg + it);          // the wave's reads of the previous tile are complete (lgkmcnt below)
+            if (it > 0) issue(0, t_beg + it);   // the wave's reads of the previous tile are complete (lgkmcnt below)
             wait_vmcnt<0>();
         } else if (it + 1 < nt) {
             issue(s ^ 1, t_beg + it + 1);
@@ -1269,10 +1271,6 @@ __global__ __launch_bounds__(NW * 64) void attn_suffix_dkdv_kernel(SuffixArgs a)
     const float* sstat = reinterpret_cast<const float*>(smem + NW * WAVE_RING + wave * STAT_BYTES);
     const unsigned stat_lds = lds_addr(smem) + NW * WAVE_RING + wave * STAT_BYTES;
 
-    typename E::opnd_t kreg[NKS], vreg[NKS];
-    load_row_operands<T, DH>(kreg, reinterpret_cast<const T*>(a.kc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
-    load_row_operands<T, DH>(vreg, reinterpret_cast<const T*>(a.vc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
-
     const T* pkm[NKS];
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) pkm[ks] = ring + km_offset<T, DH>(li, ks * 16, lane);
@@ -1333,8 +1331,12 @@ __global__ __launch_bounds__(NW * 64) void attn_suffix_dkdv_kernel(SuffixArgs a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
 
-    wait_vmcnt<0>();
+    // the first tile's loads go out before the key rows are asked for, so that the two round trips overlap
+    // (vector-memory operations complete in issue order: the first wait in the loop covers both)
     if (nt > 0) issue(0, j_beg);
+    typename E::opnd_t kreg[NKS], vreg[NKS];
+    load_row_operands<T, DH>(kreg, reinterpret_cast<const T*>(a.kc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
+    load_row_operands<T, DH>(vreg, reinterpret_cast<const T*>(a.vc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
 
     auto step = [&](auto stage_c, int it) {
         constexpr int s = decltype(stage_c)::value;
