@@ -233,6 +233,7 @@ def measure_workload(name, args, device, detail):
     layers, runner, x, R = build_model(w, device)
     runner.use_hip_graph = args.graph
     runner.slice_streams = args.slice_streams
+    runner.fused_attn_bwd = not args.two_launch_attn_bwd
     runner.launch_replay = not (args.graph or args.no_launch_replay)
     warmup, steps = (args.warmup, args.steps) if detail else (3, 5)
     for _ in range(warmup):
@@ -379,11 +380,15 @@ def attention_grid(device, reps=5):
     """The (T, P) micro-grid of the prefix-attention kernels, as the reference profiles a layer per
     (seqlen, attention_cache_len) (terapipe_latency_model.py:180-193): slice length T in {32, 64, 128}, prefix P
     in {0, 256, ..., 1792, 2048 - T} of a 2048-token sequence, head dimension 128, bf16, at the (batch, heads) of
-    workloads C5 (2, 48) and C4 (1, 96).  Per point: the forward call, the backward as the sliced runner issues
-    it (delta + dQ of the slice at P against its prefix, plus the one-pass dK/dV launch of the slice at the
-    mirrored position L - T - P, which covers the same number of query-key blocks), and
-    the backward with gradient caches (the reference's per-call contract: dK/dV of all S keys, prefix rows
-    read-modify-written).  Each call is timed alone on the chip over `sets` rotating sets of buffers larger
+    workloads C5 (2, 48) and C4 (1, 96).  Per point: the forward call; the backward as the sliced runner issues
+    it -- ONE launch for the slice at P whose first half takes delta + dQ against the P keys before the slice and
+    whose second half takes dK/dV of the slice's keys over the L - P queries from the slice on, with the delta of three
+    slices' positions taken inside the launch as the three-stream runner has it (bwd_fused_us; its
+    two halves as separate launches: dq_us at P, and dkdv_mirror_us = the dK/dV launch of the slice at the mirrored
+    position L - T - P, which covers as many query-key blocks as dQ at P does); and the backward with gradient
+    caches (the reference's per-call contract: dK/dV of all S keys, prefix rows read-modify-written).  The fused
+    launch does a whole row AND a whole column of the causal triangle per slice, so its time hardly depends on P;
+    "sequence" sums bytes and times over the grid's positions, which is what a step over the whole sequence sees.  Each call is timed alone on the chip over `sets` rotating sets of buffers larger
     together than the memory-side cache, replayed from a HIP graph between two HIP events; GB/s are the
     reference algorithm's bytes of the call (fwd (2T+2S) B E, bwd (6T+2S+4P) B E, + fp32 row statistics)."""
     from terapipe_amd import ops
@@ -434,23 +439,36 @@ def attention_grid(device, reps=5):
                     ops.attn_suffix_dkdv(b["k"], b["v"], b["q"], b["d_o"], b["lse"], b["delta"], b["dqkv"][:T * B], B, H, Dh,
                                          L - T - P, T, L)
 
+                def fused(b, T=T, P=P):
+                    ops.attn_bwd_fused(b["q"][:, P:], b["k"], b["v"], b["o"][P:P + T], b["lse"][:, P:], b["d_o"][P:P + T],
+                                       b["dqkv"][:T * B], B, H, Dh, T, P, Dh ** -0.5, b["delta"][:, P:], b["q"], b["d_o"],
+                                       b["lse"], b["delta"], b["o"], L, own_delta_end=min(L, P + 3 * T), q_bh_rows=L,
+                                       stat_bh_rows=L)
+
                 def bwd_cache(b, T=T, P=P):
                     ops.attn_prefix_bwd(b["q"][:, P:], b["k"], b["v"], b["o"][P:P + T], b["lse"][:, P:], b["d_o"][P:P + T],
                                         b["dqkv"][:T * B], b["gk"], b["gv"], B, H, Dh, T, P, Dh ** -0.5, True, True, False,
                                         delta=b["delta"][:, P:], q_bh_rows=L, stat_bh_rows=L)
 
                 us = {}
-                for nm, fn in (("fwd", fwd), ("dq", dq), ("dkdv", dkdv), ("bwd_cache", bwd_cache)):
+                for nm, fn in (("fwd", fwd), ("dq", dq), ("dkdv", dkdv), ("fused", fused), ("bwd_cache", bwd_cache)):
                     us[nm] = _graph_ms([(lambda b=b, fn=fn: fn(b)) for b in bufs], reps) * 1e3 / sets
                 fb = attn_bytes_per_call(es, B, H, E, T, P, False)
                 bb = attn_bytes_per_call(es, B, H, E, T, P, True)
                 run_us = us["dq"] + us["dkdv"]
                 rows.append({"P": P, "fwd_us": round(us["fwd"], 2), "fwd_GBps": round(fb / us["fwd"] / 1e3, 1),
                              "dq_us": round(us["dq"], 2), "dkdv_mirror_us": round(us["dkdv"], 2),
-                             "bwd_runner_us": round(run_us, 2), "bwd_runner_GBps": round(bb / run_us / 1e3, 1),
+                             "bwd_two_launches_us": round(run_us, 2), "bwd_two_launches_GBps": round(bb / run_us / 1e3, 1),
+                             "bwd_fused_us": round(us["fused"], 2),
                              "bwd_cache_us": round(us["bwd_cache"], 2), "bwd_cache_GBps": round(bb / us["bwd_cache"] / 1e3, 1),
                              "fwd_bytes": fb, "bwd_bytes": bb})
-            out.append({"heads_of": wl, "batch": B, "heads": H, "T": T, "points": rows})
+            seq = {}
+            for nm, ub, uk in (("fwd", "fwd_bytes", "fwd_us"), ("bwd_fused", "bwd_bytes", "bwd_fused_us"),
+                               ("bwd_two_launches", "bwd_bytes", "bwd_two_launches_us"), ("bwd_cache", "bwd_bytes", "bwd_cache_us")):
+                gbs = sum(r[ub] for r in rows) / sum(r[uk] for r in rows) / 1e3
+                seq[nm + "_GBps"] = round(gbs, 1)
+                seq[nm + "_frac_of_hbm_peak"] = round(gbs * 1e9 / PEAK_HBM, 4)
+            out.append({"heads_of": wl, "batch": B, "heads": H, "T": T, "sequence": seq, "points": rows})
         del bufs
         gc.collect()
         torch.cuda.empty_cache()
@@ -493,6 +511,8 @@ def main():
                     help="leave out the vendor library's times on the same GEMM shapes (context beside the per-GEMM table)")
     ap.add_argument("--attention-grid", action="store_true",
                     help="print the (T, P) micro-grid of the prefix-attention kernels instead of the step benchmark")
+    ap.add_argument("--two-launch-attn-bwd", action="store_true",
+                    help="issue dQ and the one-pass dK/dV of a slice as two launches instead of one (comparison)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 256 MiB device fill and one 256 MiB copy before the steps: the "
                          "known-size kernels that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")

@@ -206,7 +206,8 @@ typedef struct tp_attn_desc {
                                            (grad_cache.data[index] = 0, transformer_models.py:189) */
     float q_scale;
     float* colsum_dqkv_acc;             /* optional [3*H*Dh] fp32: += column sums of dqkv (in_proj bias grad) */
-    int32_t reserved;                   /* 0 = automatic; bits 0-7: number of key-range splits of the forward (tuning, tests) */
+    int32_t reserved;                   /* 0 = automatic; bits 0-7: number of workgroups (fp32: splits) that share the key
+                                           range of a query block in the forward (tuning, tests) */
     int32_t reserved2;                  /* tuning, tests.  bit 1 / bit 2: force the eight-wave / the four-wave form of the
                                            16-bit forward kernel */
     int64_t q_bh_rows;                  /* rows per (b,h) block of q: 0 = T; see tp_gemm_desc.q_bh_rows */
@@ -216,6 +217,9 @@ typedef struct tp_attn_desc {
     int32_t reserved3;
 } tp_attn_desc;
 
+/* A forward call with few (batch, head) x 32-query blocks and a long key range spreads each block's keys over
+ * several workgroups; their fp32 partial results go through the caller's workspace and a second launch of the same
+ * call merges them.  The size query returns 0 when the call does not split. */
 size_t tp_attn_fwd_workspace_bytes(const tp_attn_desc* d);
 int tp_attn_prefix_fwd(const tp_attn_desc* d, void* workspace, size_t workspace_bytes, void* stream);
 size_t tp_attn_bwd_workspace_bytes(const tp_attn_desc* d);
@@ -243,6 +247,18 @@ typedef struct tp_attn_suffix_desc {
     void* dqkv;                         /* [T*B, 3*H*Dh] of the slice; the k and v parts are written */
 } tp_attn_suffix_desc;
 int tp_attn_suffix_dkdv(const tp_attn_suffix_desc* d, void* stream);
+
+/* tp_attn_prefix_bwd with dq_only = 1 and tp_attn_suffix_dkdv of the SAME slice as one launch (fp16 / bf16): the backward
+ * of attn_helper for one slice (transformer_models.py:229-240 under autograd, driven by terapipe.py:182-191) on a stage
+ * that keeps no gradient caches.  Half of the workgroups stream the keys before the slice (dQ, delta), the other half
+ * the queries after it (dK, dV) at the same time; the two descriptors must name the same slice (d->cache_len =
+ * sd->key_begin, d->T = sd->key_count, same caches and dqkv).  The dK/dV half reads sd->delta_all only for positions
+ * at or past own_delta_end and takes delta of [key_begin, own_delta_end) itself from d_o_all and o_all (the attention
+ * output, row = position, laid out as d_o_all): own_delta_end = end of the slice when every later slice's backward
+ * has completed, later when the launches that write the delta of the next slices may still be running (at most 4096
+ * positions from key_begin).  Same results as the two calls. */
+int tp_attn_bwd_fused(const tp_attn_desc* d, const tp_attn_suffix_desc* sd, const void* o_all, int32_t own_delta_end,
+                      void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * The two ends of the layer stack in the reference's end-to-end configuration (token ids in, next-token

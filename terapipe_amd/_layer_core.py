@@ -192,6 +192,18 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
                             st.cache_len, float(Dh) ** -0.5, accumulate_prefix, has_incoming, zero_slice_rows,
                             colsum_dqkv_acc=sa.get("attn.in_proj.bias"), delta=buf.delta,
                             q_bh_rows=st.q_bh_rows, stat_bh_rows=st.stat_bh_rows)
+    elif suffix.get("o_all") is not None and suffix["own_end"] - st.cache_len <= ops.FUSED_BWD_MAX_OWN:
+        # dQ of the slice and dK / dV of its keys over all later positions as one launch.  The dK/dV half takes delta
+        # of the positions up to own_end itself, so what it needs of the later slices is their dO (and, past own_end,
+        # their delta): the slice waits for the next slice's event and records its own BEFORE the launch
+        if buf.sync is not None:
+            buf.sync()
+        ops.attn_bwd_fused(st.q, st.k_cache, st.v_cache, st.o, st.lse, d_o, dqkv, B, heads, Dh, T, st.cache_len,
+                           float(Dh) ** -0.5, buf.delta, suffix["q_all"], suffix["d_o_all"], suffix["lse_all"],
+                           suffix["delta_all"], suffix["o_all"], suffix["q_end"], suffix["own_end"],
+                           q_bh_rows=st.q_bh_rows, stat_bh_rows=st.stat_bh_rows)
+        if "attn.in_proj.bias" in sa:
+            ops.colsum_acc(dqkv, sa["attn.in_proj.bias"])
     else:
         ops.attn_prefix_bwd(st.q, st.k_cache, st.v_cache, st.o, st.lse, d_o, dqkv, None, None, B, heads, Dh, T,
                             st.cache_len, float(Dh) ** -0.5, False, False, False, delta=buf.delta,

@@ -118,6 +118,7 @@ SYMBOLS = {
     "tp_attn_bwd_workspace_bytes": (c_size_t, [ctypes.POINTER(AttnDesc)]),
     "tp_attn_prefix_bwd": (c_int, [ctypes.POINTER(AttnDesc), c_void_p, c_size_t, c_void_p]),
     "tp_attn_suffix_dkdv": (c_int, [ctypes.POINTER(AttnSuffixDesc), c_void_p]),
+    "tp_attn_bwd_fused": (c_int, [ctypes.POINTER(AttnDesc), ctypes.POINTER(AttnSuffixDesc), c_void_p, c_int, c_void_p]),
     "tp_embedding_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "tp_embedding_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "tp_cross_entropy": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p]),

@@ -482,8 +482,8 @@ static constexpr int kMaxTLds = 4096;
 // Workgroups are dealt to the eight XCDs round-robin by linear id.  This maps the linear id to
 // (batch*head, block) so that all blocks of one (batch, head) run on the same XCD and its K / V / Q / dO
 // rows are fetched into one L2 only.  Launch with xcd_grid(BH, nblocks) workgroups; false = no work.
-__device__ __forceinline__ bool xcd_map(int BH, int& bh, int& blk) {
-    const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+__device__ __forceinline__ bool xcd_map(int BH, int& bh, int& blk, int id = blockIdx.x) {
+    const int xcd = id & 7, slot = id >> 3;
     const int nbh8 = (BH + 7) >> 3;
     bh = xcd + 8 * (slot % nbh8);
     blk = slot / nbh8;
@@ -781,8 +781,15 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv2_kernel(AttnArgs a) {
 // workgroup barrier inside the loop), and the NW partial dQ blocks are summed through LDS at the end.
 // The kernel also computes delta = rowsum(dO * O) for its queries and leaves it in a.delta for the
 // dK/dV kernel that follows on the stream.
+// LDS bytes of the dQ workgroup: NW private rings of two stages of K + V, reused for the reduction
+template <int DH, int NW> constexpr int dq2_smem_bytes() {
+    constexpr int ring = NW * 2 * 2 * 32 * DH * 2, epi = NW * 32 * (DH + 4) * 4;
+    return ring > epi ? ring : epi;
+}
+
+// The work of workgroup `wg_id` of xcd_grid(B*H, ceil(T/32)); `smem` = dq2_smem_bytes<DH, NW>() bytes, 16-byte aligned.
 template <typename T, int DH, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_bwd_dq2_kernel(AttnArgs a) {
+__device__ __forceinline__ void attn_bwd_dq2_body(const AttnArgs& a, unsigned char* smem, int wg_id) {
     typedef Elem<T> E;
     static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
     constexpr int NDB = DH / 32, NKS = DH / 16;
@@ -793,14 +800,11 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq2_kernel(AttnArgs a) {
     static_assert(NLOAD <= 63, "too many loads in flight for vmcnt");
     constexpr int WAVE_RING = 2 * 2 * TILE * 2;         // bytes: two stages of K + V
     constexpr int EPI_LD = DH + 4;
-    constexpr int EPI_BYTES = NW * 32 * EPI_LD * 4;
-    constexpr int SMEM = NW * WAVE_RING > EPI_BYTES ? NW * WAVE_RING : EPI_BYTES;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM];
 
     const int tid = threadIdx.x, lane = tid & 63, g = lane >> 5, li = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int bh, qblk;
-    if (!xcd_map(a.B * a.H, bh, qblk)) return;
+    if (!xcd_map(a.B * a.H, bh, qblk, wg_id)) return;
     const int b = bh / a.H, h = bh - b * a.H;
     const int T_ = a.T, P = a.P, S = a.P + a.T;
     const long EE = (long)a.H * DH;
@@ -991,6 +995,12 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq2_kernel(AttnArgs a) {
     }
 }
 
+template <typename T, int DH, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_bwd_dq2_kernel(AttnArgs a) {
+    __shared__ __attribute__((aligned(16))) unsigned char smem[dq2_smem_bytes<DH, NW>()];
+    attn_bwd_dq2_body<T, DH, NW>(a, smem, blockIdx.x);
+}
+
 // Forward, second generation.  A workgroup owns 32 queries of one (batch, head); its NW waves split the
 // key range, each streaming its own K / V tiles of 32 keys through a private two-stage LDS ring and
 // keeping its own online-softmax state; the NW partial (m, l, O) are merged through LDS at the end.
@@ -1027,8 +1037,16 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
     const bool qok = tq < T_;
     const int kv_end = P + min(T_, q0 + 32);
     const int ntiles = (kv_end + 31) / 32;
-    const int tpw = (ntiles + NW - 1) / NW;
-    const int t_beg = wave * tpw, t_end = min(ntiles, t_beg + tpw);
+    // the key tiles of this workgroup: all of them, or its share when gridDim.y workgroups split a block's keys
+    // (the grid's x extent is a multiple of eight, so they all stay on the XCD that xcd_map gives the block)
+    int wg_beg = 0, wg_end = ntiles;
+    if (a.nsplit > 1) {
+        const int per = (ntiles + a.nsplit - 1) / a.nsplit;
+        wg_beg = min(ntiles, (int)blockIdx.y * per);
+        wg_end = min(ntiles, wg_beg + per);
+    }
+    const int tpw = (wg_end - wg_beg + NW - 1) / NW;
+    const int t_beg = wg_beg + wave * tpw, t_end = min(wg_end, t_beg + tpw);
     const int nt = max(t_end - t_beg, 0);
 
     T* ring = reinterpret_cast<T*>(smem) + wave * (WAVE_RING / 2);
@@ -1201,13 +1219,22 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[db][r] *= f;
     acc_to_lds_rows<DH>(oacc, ebuf + wave * 32 * EPI_LD, lane);
-    if (wave == 0 && g == 0 && qok) a.lse[(long)bh * a.st_bhs + tq] = L > 0.f ? m_tot + logf(L) : -INFINITY;
+    // a workgroup that has a share of the keys only leaves its normalised output and its log-sum-exp as fp32
+    // partials; attn_fwd_merge_kernel weighs the shares together
+    const bool partial = a.nsplit > 1;
+    const long prow0 = ((long)blockIdx.y * (a.B * a.H) + bh) * T_;
+    if (wave == 0 && g == 0 && qok) {
+        const float lse_wg = L > 0.f ? m_tot + logf(L) : -INFINITY;
+        if (partial) a.part_lse[prow0 + tq] = lse_wg;
+        else a.lse[(long)bh * a.st_bhs + tq] = lse_wg;
+    }
     __syncthreads();
     constexpr int CPT = 32 * DH / (NW * 64);
     static_assert(CPT % 4 == 0 && DH % CPT == 0, "bad reduction split");
     const int row = tid / (DH / CPT), c0 = (tid % (DH / CPT)) * CPT;
     if (q0 + row < T_) {
         T* dst = reinterpret_cast<T*>(a.o) + ((long)(q0 + row) * a.B + b) * EE + (long)h * DH + c0;
+        float* pdst = a.part_o + (prow0 + q0 + row) * DH + c0;
 #pragma unroll
         for (int c = 0; c < CPT; c += 4) {
             float4 acc4 = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -1216,7 +1243,8 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
                 const float4 v = *reinterpret_cast<const float4*>(ebuf + (w * 32 + row) * EPI_LD + c0 + c);
                 acc4.x += v.x; acc4.y += v.y; acc4.z += v.z; acc4.w += v.w;
             }
-            store4<T>(dst + c, acc4.x, acc4.y, acc4.z, acc4.w);
+            if (partial) *reinterpret_cast<float4*>(pdst + c) = acc4;
+            else store4<T>(dst + c, acc4.x, acc4.y, acc4.z, acc4.w);
         }
     }
 }
@@ -1230,12 +1258,24 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
 struct SuffixArgs {
     const void* kc; const void* vc; const void* q; const void* d_o;
     const float* lse; const float* delta; void* dqkv;
+    const void* o_all;      // OWN_DELTA only: the attention output [.., B, H*Dh], row = position
+    int own_end;            // OWN_DELTA only: delta of the positions [P, own_end) is computed here
     int B, H, P, T, Lq;
     long cache_rows, q_bhs, st_bhs;
 };
 
-template <typename T, int DH, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_suffix_dkdv_kernel(SuffixArgs a) {
+// LDS bytes of the dK/dV workgroup: NW private rings of two stages of Q + dO and of (lse, delta) rows
+template <int DH, int NW> constexpr int suffix_smem_bytes() {
+    constexpr int ring = NW * (2 * 2 * 32 * DH * 2 + 2 * 256), epi = NW * 32 * (DH + 4) * 4;
+    return ring > epi ? ring : epi;
+}
+
+// The work of workgroup `wg_id` of xcd_grid(B*H, ceil(T/32)); `smem` = suffix_smem_bytes<DH, NW>() bytes.
+// OWN_DELTA: delta of the positions [P, own_end) -- the slice's own and those of the slices whose dQ launch may still
+// be running -- is not read from a.delta but taken here from dO and the attention output, into `own`
+// (ceil((own_end - P) / 32) * 32 floats of LDS).
+template <typename T, int DH, int NW, bool OWN_DELTA>
+__device__ __forceinline__ void attn_suffix_dkdv_body(const SuffixArgs& a, unsigned char* smem, float* own, int wg_id) {
     typedef Elem<T> E;
     static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
     constexpr int NDB = DH / 32, NKS = DH / 16;
@@ -1247,15 +1287,11 @@ __global__ __launch_bounds__(NW * 64) void attn_suffix_dkdv_kernel(SuffixArgs a)
     constexpr int WAVE_RING = 2 * 2 * TILE * 2;         // bytes: two stages of Q + dO
     constexpr int STAT_BYTES = 2 * 256;                 // per wave: two stages of 32 lse + 32 delta
     constexpr int EPI_LD = DH + 4;
-    constexpr int EPI_BYTES = NW * 32 * EPI_LD * 4;
-    constexpr int RING_ALL = NW * (WAVE_RING + STAT_BYTES);
-    constexpr int SMEM = RING_ALL > EPI_BYTES ? RING_ALL : EPI_BYTES;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM];
 
     const int tid = threadIdx.x, lane = tid & 63, g = lane >> 5, li = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int bh, kblk;
-    if (!xcd_map(a.B * a.H, bh, kblk)) return;
+    if (!xcd_map(a.B * a.H, bh, kblk, wg_id)) return;
     const int b = bh / a.H, h = bh - b * a.H;
     const int P = a.P, S = a.P + a.T, Lq = a.Lq;
     const long EE = (long)a.H * DH;
@@ -1337,6 +1373,27 @@ __global__ __launch_bounds__(NW * 64) void attn_suffix_dkdv_kernel(SuffixArgs a)
     typename E::opnd_t kreg[NKS], vreg[NKS];
     load_row_operands<T, DH>(kreg, reinterpret_cast<const T*>(a.kc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
     load_row_operands<T, DH>(vreg, reinterpret_cast<const T*>(a.vc) + ((long)bh * a.cache_rows + key) * DH, key < S, g);
+    if constexpr (OWN_DELTA) {
+        // delta = rowsum(dO * O) of the positions [key0, own_end), 32 positions per wave and pass: lane (li, g)
+        // takes half g of position li's row, as the dQ kernel does for its own rows
+        for (int blk = wave; key0 + blk * 32 < a.own_end; blk += NW) {
+            const int t = key0 + blk * 32 + li;
+            typename E::opnd_t oreg[NKS], doreg[NKS];
+            load_row_operands<T, DH>(oreg, reinterpret_cast<const T*>(a.o_all) + ((long)t * a.B + b) * EE + (long)h * DH, t < a.own_end, g);
+            load_row_operands<T, DH>(doreg, reinterpret_cast<const T*>(a.d_o) + ((long)t * a.B + b) * EE + (long)h * DH, t < a.own_end, g);
+            float sum = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                const T* x = reinterpret_cast<const T*>(&oreg[ks]);
+                const T* y = reinterpret_cast<const T*>(&doreg[ks]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sum = fmaf(E::to_float(x[e]), E::to_float(y[e]), sum);
+            }
+            sum += __shfl_xor(sum, 32, 64);
+            if (g == 0) own[blk * 32 + li] = sum;
+        }
+        __syncthreads();
+    }
 
     auto step = [&](auto stage_c, int it) {
         constexpr int s = decltype(stage_c)::value;
@@ -1359,6 +1416,18 @@ __global__ __launch_bounds__(NW * 64) void attn_suffix_dkdv_kernel(SuffixArgs a)
         for (int jq = 0; jq < 4; ++jq) {
             l4[jq] = *reinterpret_cast<const float4*>(sstat + s * 64 + 8 * jq + 4 * g);
             d4[jq] = *reinterpret_cast<const float4*>(sstat + s * 64 + 32 + 8 * jq + 4 * g);
+        }
+        if constexpr (OWN_DELTA) {
+            if (t0 < a.own_end) {           // wave-uniform: the block has positions whose delta is taken here
+#pragma unroll
+                for (int jq = 0; jq < 4; ++jq) {
+                    const int rel = t0 - key0 + 8 * jq + 4 * g;     // position - key0 of the float4's first entry
+                    if (t0 + 8 * jq + 4 * g + 0 < a.own_end) d4[jq].x = own[rel + 0];
+                    if (t0 + 8 * jq + 4 * g + 1 < a.own_end) d4[jq].y = own[rel + 1];
+                    if (t0 + 8 * jq + 4 * g + 2 < a.own_end) d4[jq].z = own[rel + 2];
+                    if (t0 + 8 * jq + 4 * g + 3 < a.own_end) d4[jq].w = own[rel + 3];
+                }
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         float16v sacc, pacc;
@@ -1459,6 +1528,27 @@ __global__ __launch_bounds__(NW * 64) void attn_suffix_dkdv_kernel(SuffixArgs a)
     }
 }
 
+template <typename T, int DH, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_suffix_dkdv_kernel(SuffixArgs a) {
+    __shared__ __attribute__((aligned(16))) unsigned char smem[suffix_smem_bytes<DH, NW>()];
+    attn_suffix_dkdv_body<T, DH, NW, false>(a, smem, nullptr, blockIdx.x);
+}
+
+// dQ (+ delta) of a slice and the one-pass dK / dV of the same slice as ONE launch: workgroups [0, n_dq) do the
+// work of attn_bwd_dq2_kernel, the others that of attn_suffix_dkdv_kernel, side by side on different CUs -- the dQ
+// side streams the keys before the slice, the dK/dV side the queries after it, so the two loads are complementary
+// and a call with few (batch, head) pairs fills twice as many CUs.  The dK/dV side does not wait for the delta
+// that the dQ side writes: it takes delta of the positions [P, own_end) from dO and O itself (dynamic LDS:
+// ceil((own_end - P) / 32) * 32 floats).  n_dq is a multiple of eight, so both sides keep the XCD placement of xcd_map.
+template <typename T, int DH>
+__global__ __launch_bounds__(256) void attn_bwd_fused_kernel(AttnArgs a, SuffixArgs sa, int n_dq) {
+    constexpr int SM = dq2_smem_bytes<DH, 4>() > suffix_smem_bytes<DH, 4>() ? dq2_smem_bytes<DH, 4>() : suffix_smem_bytes<DH, 4>();
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SM];
+    extern __shared__ __attribute__((aligned(16))) float own_delta[];
+    if ((int)blockIdx.x < n_dq) attn_bwd_dq2_body<T, DH, 4>(a, smem, blockIdx.x);
+    else attn_suffix_dkdv_body<T, DH, 4, true>(sa, smem, own_delta, (int)blockIdx.x - n_dq);
+}
+
 // ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
@@ -1489,6 +1579,20 @@ static FwdPlan plan_fwd(const tp_attn_desc* d) {
     if (d->dtype != TP_F32) {
         // 16-bit: one workgroup per 32 queries whose four waves split the key range and merge in LDS
         p.nw = 0; p.bn = 32; p.nsplit = 1; p.qblocks = (d->T + 31) / 32;
+        // A call with so few query blocks that over half of the CUs would get no workgroup, and a key range long
+        // enough to share (16 tiles of 32 keys per share), spreads each block's keys over as many workgroups as fit
+        // the chip; they leave fp32 partials in the workspace and the merge launch weighs them together.  Measured
+        // at 96 (batch, head) pairs of 32 queries: 28.4 against 31.1 us at 2048 keys, nothing gained below 1024.
+        const long wgs = (long)d->batch * d->heads * p.qblocks;
+        const int ntiles = (d->cache_len + d->T + 31) / 32;
+        if (d->reserved & 0xff) {
+            p.nsplit = (d->reserved & 0xff) > 16 ? 16 : (d->reserved & 0xff);
+        } else if (wgs * 5 <= kNumCU * 2) {
+            int ns = (int)(kNumCU / wgs);
+            if (ns > ntiles / 16) ns = ntiles / 16;
+            if (ns > 8) ns = 8;
+            if (ns >= 2) p.nsplit = ns;
+        }
         // bn doubles as the wave count of this kernel: 8 = eight waves with one tile buffer each, faster
         // from about twenty key tiles on (measured: 19 against 24 us at 2048 keys, 7.9 against 7.6 us at 256);
         // reserved2 bit 1 forces it, bit 2 forces four waves
@@ -1533,9 +1637,9 @@ template <typename T, int DH>
 static void launch_fwd(const FwdPlan& p, const AttnArgs& a, hipStream_t s) {
     dim3 grid(p.qblocks, a.B * a.H, p.nsplit);
     if constexpr (sizeof(T) == 2) {
-        if (p.bn == 8) attn_fwd2_kernel<T, DH, 8, 1><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 512, 0, s>>>(a);
-        else attn_fwd2_kernel<T, DH, 4><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 256, 0, s>>>(a);
-        return;
+        const dim3 g2(xcd_grid(a.B * a.H, (a.T + 31) / 32), p.nsplit);
+        if (p.bn == 8) attn_fwd2_kernel<T, DH, 8, 1><<<g2, 512, 0, s>>>(a);
+        else attn_fwd2_kernel<T, DH, 4><<<g2, 256, 0, s>>>(a);
     } else {
         if (p.nw == 4) attn_fwd_kernel<T, DH, 4, 64><<<grid, 256, 0, s>>>(a);
         else if (p.nw == 2) attn_fwd_kernel<T, DH, 2, 64><<<grid, 128, 0, s>>>(a);
@@ -1672,9 +1776,75 @@ extern "C" int tp_attn_prefix_bwd(const tp_attn_desc* d, void* workspace, size_t
     return TP_OK;
 }
 
+static int validate_suffix(const tp_attn_suffix_desc* d, const char* who);
+static tp::SuffixArgs make_suffix_args(const tp_attn_suffix_desc* d);
+
 extern "C" int tp_attn_suffix_dkdv(const tp_attn_suffix_desc* d, void* stream) {
     using namespace tp;
     const char* who = "tp_attn_suffix_dkdv";
+    int rc = validate_suffix(d, who);
+    if (rc != TP_OK) return rc;
+    SuffixArgs a = make_suffix_args(d);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const unsigned grid = xcd_grid(d->batch * d->heads, (d->key_count + 31) / 32);
+    if (d->dtype == TP_F16) {
+        if (d->head_dim == 64) attn_suffix_dkdv_kernel<f16, 64, 4><<<grid, 256, 0, s>>>(a);
+        else attn_suffix_dkdv_kernel<f16, 128, 4><<<grid, 256, 0, s>>>(a);
+    } else {
+        if (d->head_dim == 64) attn_suffix_dkdv_kernel<bf16, 64, 4><<<grid, 256, 0, s>>>(a);
+        else attn_suffix_dkdv_kernel<bf16, 128, 4><<<grid, 256, 0, s>>>(a);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("%s: launch failed: %s", who, hipGetErrorString(e)); return TP_ERR_LAUNCH; }
+    return TP_OK;
+}
+
+extern "C" int tp_attn_bwd_fused(const tp_attn_desc* d, const tp_attn_suffix_desc* sd, const void* o_all, int own_delta_end,
+                                 void* stream) {
+    using namespace tp;
+    const char* who = "tp_attn_bwd_fused";
+    int rc = validate_attn(d, true);
+    if (rc != TP_OK) return rc;
+    rc = validate_suffix(sd, who);
+    if (rc != TP_OK) return rc;
+    if (!d->dq_only) { set_error("%s: the backward descriptor must have dq_only set (no gradient caches on this path)", who); return TP_ERR_ARG; }
+    if (d->dtype != sd->dtype || d->batch != sd->batch || d->heads != sd->heads || d->head_dim != sd->head_dim ||
+        d->cache_len != sd->key_begin || d->T != sd->key_count || d->dqkv != sd->dqkv || d->k_cache != sd->k_cache ||
+        d->v_cache != sd->v_cache || (long)d->cache_rows != (long)sd->cache_rows) {
+        set_error("%s: the two descriptors do not describe the same slice (dtype, batch, heads, head_dim, cache_len = key_begin, "
+                  "T = key_count, dqkv, caches)", who);
+        return TP_ERR_ARG;
+    }
+    if (!o_all || ((uintptr_t)o_all & 15)) { set_error("%s: o_all must be a 16-byte aligned device pointer", who); return TP_ERR_ARG; }
+    if (own_delta_end < sd->key_begin + sd->key_count || own_delta_end > sd->q_end) {
+        set_error("%s: own_delta_end %d outside [key_begin + key_count, q_end] = [%d, %d]", who, own_delta_end,
+                  sd->key_begin + sd->key_count, sd->q_end);
+        return TP_ERR_ARG;
+    }
+    const int own_len = own_delta_end - sd->key_begin;
+    if (own_len > kMaxTLds) { set_error("%s: delta of up to %d positions is taken in the launch (got %d); use the two separate calls", who, kMaxTLds, own_len); return TP_ERR_UNSUPPORTED; }
+    AttnArgs a = make_args(d);
+    SuffixArgs sa = make_suffix_args(sd);
+    sa.o_all = o_all;
+    sa.own_end = own_delta_end;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const int n_dq = (int)xcd_grid(d->batch * d->heads, (d->T + 31) / 32);
+    const unsigned grid = (unsigned)n_dq + xcd_grid(d->batch * d->heads, (d->T + 31) / 32);
+    const size_t dyn = (size_t)((own_len + 31) / 32) * 32 * sizeof(float);
+    if (d->dtype == TP_F16) {
+        if (d->head_dim == 64) attn_bwd_fused_kernel<f16, 64><<<grid, 256, dyn, s>>>(a, sa, n_dq);
+        else attn_bwd_fused_kernel<f16, 128><<<grid, 256, dyn, s>>>(a, sa, n_dq);
+    } else {
+        if (d->head_dim == 64) attn_bwd_fused_kernel<bf16, 64><<<grid, 256, dyn, s>>>(a, sa, n_dq);
+        else attn_bwd_fused_kernel<bf16, 128><<<grid, 256, dyn, s>>>(a, sa, n_dq);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("%s: launch failed: %s", who, hipGetErrorString(e)); return TP_ERR_LAUNCH; }
+    return TP_OK;
+}
+
+static int validate_suffix(const tp_attn_suffix_desc* d, const char* who) {
+    using namespace tp;
     if (!d) { set_error("%s: null descriptor", who); return TP_ERR_ARG; }
     if (d->dtype != TP_F16 && d->dtype != TP_BF16) { set_error("%s: dtype %d not supported (fp16 / bf16)", who, d->dtype); return TP_ERR_UNSUPPORTED; }
     if (d->head_dim != 64 && d->head_dim != 128) { set_error("%s: head_dim %d not supported (64 or 128)", who, d->head_dim); return TP_ERR_UNSUPPORTED; }
@@ -1689,21 +1859,14 @@ extern "C" int tp_attn_suffix_dkdv(const tp_attn_suffix_desc* d, void* stream) {
     }
     if (!d->k_cache || !d->v_cache || !d->q_all || !d->d_o_all || !d->lse_all || !d->delta_all || !d->dqkv) { set_error("%s: null tensor", who); return TP_ERR_ARG; }
     if (((uintptr_t)d->k_cache | (uintptr_t)d->v_cache | (uintptr_t)d->q_all | (uintptr_t)d->d_o_all | (uintptr_t)d->dqkv) & 15) { set_error("%s: tensors must be 16-byte aligned", who); return TP_ERR_ARG; }
-    SuffixArgs a;
+    return TP_OK;
+}
+
+static tp::SuffixArgs make_suffix_args(const tp_attn_suffix_desc* d) {
+    tp::SuffixArgs a;
     a.kc = d->k_cache; a.vc = d->v_cache; a.q = d->q_all; a.d_o = d->d_o_all;
-    a.lse = d->lse_all; a.delta = d->delta_all; a.dqkv = d->dqkv;
+    a.lse = d->lse_all; a.delta = d->delta_all; a.dqkv = d->dqkv; a.o_all = nullptr; a.own_end = 0;
     a.B = d->batch; a.H = d->heads; a.P = d->key_begin; a.T = d->key_count; a.Lq = d->q_end;
     a.cache_rows = d->cache_rows; a.q_bhs = d->q_bh_rows * d->head_dim; a.st_bhs = d->stat_bh_rows;
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    const unsigned grid = xcd_grid(d->batch * d->heads, (d->key_count + 31) / 32);
-    if (d->dtype == TP_F16) {
-        if (d->head_dim == 64) attn_suffix_dkdv_kernel<f16, 64, 4><<<grid, 256, 0, s>>>(a);
-        else attn_suffix_dkdv_kernel<f16, 128, 4><<<grid, 256, 0, s>>>(a);
-    } else {
-        if (d->head_dim == 64) attn_suffix_dkdv_kernel<bf16, 64, 4><<<grid, 256, 0, s>>>(a);
-        else attn_suffix_dkdv_kernel<bf16, 128, 4><<<grid, 256, 0, s>>>(a);
-    }
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) { set_error("%s: launch failed: %s", who, hipGetErrorString(e)); return TP_ERR_LAUNCH; }
-    return TP_OK;
+    return a;
 }

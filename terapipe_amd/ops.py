@@ -336,6 +336,38 @@ def attn_suffix_dkdv(k_cache, v_cache, q_all, d_o_all, lse_all, delta_all, dqkv,
     return dqkv
 
 
+FUSED_BWD_MAX_OWN = 4096    # positions whose delta the fused backward launch can take itself (kept in LDS)
+
+
+def attn_bwd_fused(q, k_cache, v_cache, o, lse, d_o, dqkv, batch, heads, head_dim, T, cache_len, q_scale, delta,
+                   q_all, d_o_all, lse_all, delta_all, o_all, q_end, own_delta_end=None, q_bh_rows=0, stat_bh_rows=0):
+    """attn_prefix_bwd(dq_only=True) and attn_suffix_dkdv of the same slice as one launch (fp16 / bf16): writes
+    delta and all three parts of dqkv [T*B, 3*H*Dh].  Arguments as in the two calls; the slice is the positions
+    [cache_len, cache_len + T) and queries up to q_end take part in its dK / dV.  o_all [>= q_end, B, H*Dh] is the
+    attention output by position; delta of the positions [cache_len, own_delta_end) is taken inside the launch
+    (default: the slice's own), delta_all is read only from own_delta_end on."""
+    _require_cuda(q, k_cache, v_cache, d_o, dqkv, q_all, d_o_all, o_all)
+    d = _attn_desc(q, k_cache, v_cache, o, lse, batch, heads, head_dim, T, cache_len, q_scale, q_bh_rows, stat_bh_rows)
+    d.dq_only = 1
+    d.d_o, d.delta, d.dqkv = d_o.data_ptr(), delta.data_ptr(), dqkv.data_ptr()
+    d.grad_cache_dtype = d.dtype
+    sd = _lib.AttnSuffixDesc()
+    sd.dtype = d.dtype
+    sd.batch, sd.heads, sd.head_dim = batch, heads, head_dim
+    sd.key_begin, sd.key_count, sd.q_end = cache_len, T, q_end
+    sd.cache_rows, sd.q_bh_rows, sd.stat_bh_rows = k_cache.shape[1], q_all.shape[1], lse_all.shape[1]
+    sd.k_cache, sd.v_cache = k_cache.data_ptr(), v_cache.data_ptr()
+    sd.q_all, sd.d_o_all = q_all.data_ptr(), d_o_all.data_ptr()
+    sd.lse_all, sd.delta_all, sd.dqkv = lse_all.data_ptr(), delta_all.data_ptr(), dqkv.data_ptr()
+    own_end = cache_len + T if own_delta_end is None else int(own_delta_end)
+    o_ptr = o_all.data_ptr()
+    lib = _lib.load()
+    _lib.check(lib.tp_attn_bwd_fused(ctypes.byref(d), ctypes.byref(sd), o_ptr, own_end, _stream()), "tp_attn_bwd_fused")
+    _record("attn_bwd", (batch, heads, head_dim, T, cache_len),
+            lambda s=None: lib.tp_attn_bwd_fused(ctypes.byref(d), ctypes.byref(sd), o_ptr, own_end, _on(s)))
+    return dqkv
+
+
 def ln_param_grads(dy, x2d, mean, rstd, dgamma_acc, dbeta_acc):
     """dgamma_acc[E] += sum_m dy * xhat, dbeta_acc[E] += sum_m dy over all M rows (fp32 accumulators)."""
     _require_cuda(dy, x2d, dgamma_acc, dbeta_acc)

@@ -83,6 +83,7 @@ class _StackBuffers:
         L, Dh = runner.seq_len, layers.embedding_dim // layers.num_attention_heads
         self.dtype, self.device = dtype, device
         self.position_indexed = runner.suffix_dkdv and dtype != torch.float32     # the one-pass kernel is 16-bit
+        self.fused_attn_bwd = runner.fused_attn_bwd
         gdt = torch.float32 if runner.fp32_grad_cache else dtype
         kw = dict(dtype=dtype, device=device)
         f32 = dict(dtype=torch.float32, device=device)
@@ -321,6 +322,8 @@ def _backward_body(runner, ws, act, bufs, states):
             P -= T
             r0, r1 = P * Bs, (P + T) * Bs
             last = i == ns - 1
+            # end of the positions whose delta a fused attention-backward launch of this slice takes itself
+            own_end = min(L, P + sum(runner.seq_slices[i:i + max(len(lanes), 1)]))
             if runner.slice_timing is not None:
                 runner.slice_timing["bwd"].append(_timing_event(main))
             if bufs.position_indexed:
@@ -333,9 +336,14 @@ def _backward_body(runner, ws, act, bufs, states):
                         sync = None
                         if lanes:
                             # the one-pass dK/dV of (slice i, layer l) reads dO and delta of every later
-                            # slice at layer l: after its own dQ kernel (which leaves its delta; its dO is
-                            # older) the slice waits for the next slice's event of that layer, then records
-                            # its own
+                            # slice at layer l.  Two launches: after its own dQ kernel (which leaves its
+                            # delta; its dO is older) the slice waits for the next slice's event of that
+                            # layer, then records its own.  One fused launch: the same wait and record come
+                            # BEFORE the launch (the slice's dO is there, its delta is not), and the launch
+                            # takes the delta of its own positions and of the next len(lanes) - 1 slices --
+                            # whose fused launches may still be running -- itself; slice i + len(lanes) is an
+                            # earlier piece of work of this same stream, and the slices after it are earlier
+                            # work of the streams whose events this one has waited for
                             def sync(l=l, st_i=st_i, later=later_done, done=done):
                                 if later is not None:
                                     _wait_event(st_i, later[l])
@@ -347,7 +355,9 @@ def _backward_body(runner, ws, act, bufs, states):
                         core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), H, None, None,
                                        None, False, None, False, False, False, activation=act[l], buf=bf,
                                        suffix=dict(q_all=pb["q"][l], d_o_all=pb["d_o"][l], lse_all=pb["lse"][l],
-                                                   delta_all=pb["delta"][l], q_end=L))
+                                                   delta_all=pb["delta"][l], q_end=L,
+                                                   o_all=pb["o"][l].view(L, Bs, E) if bufs.fused_attn_bwd else None,
+                                                   own_end=own_end))
                         if lanes:
                             # end of (slice, layer): what the parameter gradients of the layer wait for
                             fin = torch.cuda.Event()
@@ -577,6 +587,9 @@ class TeraPipe(nn.Module):
     positions (every later slice has run its backward by then) -- the same sum that the reference builds
     up through the cache gradients, without gradient caches and their read-modify-write per slice.  With
     False (and always in fp32) the gradient caches are used.
+    fused_attn_bwd (with suffix_dkdv): dQ of a slice and the one-pass dK/dV of its keys go out as one launch whose
+    two halves run side by side (the first streams the keys before the slice, the second the queries after it)
+    instead of two launches one after the other.  Same results.
     slice_streams (with suffix_dkdv, fp16 / bf16): slice i runs on stream i mod slice_streams.  The attention
     kernel of a layer waits (by event) for the in_proj GEMMs of the earlier slices at that layer, the one-pass
     dK/dV kernel for the dQ kernels of the later slices; nothing else orders slices, so consecutive slices
@@ -597,7 +610,8 @@ class TeraPipe(nn.Module):
     """
 
     def __init__(self, layers, batch_size, seq_len, batch_slices, seq_slices, batch_dim=1, sequence_dim=0,
-                 fp32_grad_cache=True, use_hip_graph=False, suffix_dkdv=True, slice_streams=None, launch_replay=None):
+                 fp32_grad_cache=True, use_hip_graph=False, suffix_dkdv=True, slice_streams=None, launch_replay=None,
+                 fused_attn_bwd=True):
         super().__init__()
         assert sum(batch_slices) == batch_size and sum(seq_slices) == seq_len
         assert batch_dim == 1 and sequence_dim == 0, "layers take [seq, batch, embed] inputs"
@@ -608,6 +622,7 @@ class TeraPipe(nn.Module):
         self.fp32_grad_cache = fp32_grad_cache
         self.use_hip_graph = use_hip_graph
         self.suffix_dkdv = suffix_dkdv
+        self.fused_attn_bwd = bool(fused_attn_bwd)
         # defaults: three slice streams and launch replay; one stream and no replay under use_hip_graph
         self.slice_streams = int(slice_streams) if slice_streams is not None else (1 if use_hip_graph else 3)
         self.launch_replay = bool(launch_replay) if launch_replay is not None else not use_hip_graph
@@ -641,6 +656,7 @@ class TeraPipe(nn.Module):
         ptrs = [t.data_ptr() for w in ws for t in w.values()]
         if (self._sbufs is None or self._sbufs.dtype != dtype or self._sbufs.device != device
                 or self._sbufs.slice_streams != self.slice_streams
+                or self._sbufs.fused_attn_bwd != self.fused_attn_bwd
                 or self._sbufs.param_ptrs != ptrs):     # recorded graphs / launches hold the parameter addresses
             self._sbufs = _StackBuffers(self, dtype, device, ws)
         return self._sbufs

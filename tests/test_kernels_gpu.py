@@ -501,6 +501,45 @@ def test_attn_position_indexed_and_suffix_dkdv(dtype, B, H, Dh, L, slices):
     assert_close(dq, q64.grad * 0.5, dtype, "dq")
     assert_close(dk, k64.grad, dtype, "dk over all later queries")
     assert_close(dv, v64.grad, dtype, "dv over all later queries")
+    # the two launches of a slice as one (tp_attn_bwd_fused): its dK/dV half takes delta of the slice's own
+    # positions from dO and O itself instead of waiting for the dQ half -- same arithmetic, same bits
+    # (window: how many slices' delta the dK/dV half takes itself -- its own, or also that of the next two, whose
+    # entries in the delta array it then must not read: they are poisoned here)
+    for window in (1, 3):
+        dqkv_fused = torch.zeros(Ltot * B, 3 * E, dtype=dtype, device=DEV)
+        delta_fused = torch.full((BH, L), 321.0, dtype=torch.float32, device=DEV)
+        for i in reversed(range(len(slices))):
+            T, P = slices[i], sum(slices[:i])
+            own_end = sum(slices[:i + window])
+            seen = delta_fused.clone()
+            seen[:, P:own_end] = float("nan")
+            ops.attn_bwd_fused(qd[:, P:], kd, vd, o_all[P:P + T], lse_all[:, P:], dod[P:P + T], dqkv_fused[P * B:(P + T) * B],
+                               B, H, Dh, T, P, 0.5, delta_fused[:, P:], qd, dod, lse_all, seen, o_all, Ltot,
+                               own_delta_end=own_end, q_bh_rows=L, stat_bh_rows=L)
+        assert torch.equal(delta_fused, delta_all), "delta, fused launch, window %d" % window
+        assert torch.equal(dqkv_fused, dqkv_all), "dqkv, fused launch, window %d" % window
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("T,B,H,Dh,P,ns", [(32, 2, 3, 128, 480, 2), (40, 1, 2, 64, 200, 3), (128, 1, 4, 128, 896, 5),
+                                           (7, 1, 1, 64, 5, 4), (160, 1, 2, 128, 100, 16), (32, 2, 48, 128, 992, 2)])
+def test_attn_fwd_keys_shared_by_workgroups(dtype, T, B, H, Dh, P, ns):
+    """The 16-bit forward with the key range of every query block forced onto `ns` workgroups whose fp32 partials
+    the merge launch weighs together -- what the plan does by itself for calls with few blocks and long key ranges
+    (BASELINE config 5's later slices in ATTN_CASES).  Shares that come out empty (more workgroups than tiles) and
+    ragged last tiles are part of the cases.  Checked against the fp64 attention."""
+    ops = _ops()
+    S, E, BH = P + T, H * Dh, B * H
+    g = torch.Generator().manual_seed(T * 5 + P + ns)
+    q = _rnd((BH, T, Dh), dtype, g, 1.0)
+    kc, vc = _rnd((BH, S, Dh), dtype, g, Dh ** -0.25), _rnd((BH, S, Dh), dtype, g)
+    q64, k64, v64 = q.double(), kc.double(), vc.double()
+    oref = _attn_ref(q64, k64, v64, B, H, T, P)
+    lse_ref = torch.logsumexp(torch.bmm(q64, k64.transpose(1, 2)) + oracle.causal_prefix_mask(T, P, torch.float64), -1)
+    for variant in (2, 4):
+        o, lse = ops.attn_prefix_fwd(q.to(DEV), kc.to(DEV), vc.to(DEV), B, H, Dh, T, P, 1.0, nsplit=ns, variant=variant)
+        assert_close(o, oref, dtype, "o, keys over %d workgroups, variant %d" % (ns, variant))
+        assert_close(lse, lse_ref, torch.float32, "lse, keys over %d workgroups, variant %d" % (ns, variant), 1e3)
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)

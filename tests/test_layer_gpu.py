@@ -617,6 +617,30 @@ def test_slice_streams_match_single_stream(dtype):
                 assert_close(a, b, dtype, "parameter gradient with %d lanes" % n, 1.0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_fused_attention_backward_matches_two_launches(dtype):
+    """The runner with dQ and the one-pass dK/dV of a slice as one launch (the default) against the same runner with
+    the two launches one after the other, on one stream and on three (where the launch sits between the wait for
+    the later slice's event and the record of the slice's own): outputs and input gradients bit-identical."""
+    ta = _mods()
+    n_layers, E, H, Fd, L, B = 3, 512, 4, 2048, 512, 2
+    ss = [128, 32, 96, 40, 88, 128]
+    ps = make_params(n_layers, E, Fd, dtype, seed=19)
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    g = torch.Generator().manual_seed(15)
+    x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
+    _, y1, dx1 = _run_terapipe(ta, layers, x, dy, B, L, [B], ss, fused_attn_bwd=False)
+    g1 = [p.grad.clone() for p in layers.parameters()]
+    for n in (1, 3):
+        for rep in range(2):
+            _, y2, dx2 = _run_terapipe(ta, layers, x, dy, B, L, [B], ss, slice_streams=n, fused_attn_bwd=True)
+            torch.cuda.synchronize()
+            assert torch.equal(y2, y1), "y, fused backward, %d streams" % n
+            assert torch.equal(dx2, dx1), "dx, fused backward, %d streams" % n
+            for a, b in zip([p.grad for p in layers.parameters()], g1):
+                assert_close(a, b, dtype, "parameter gradient, fused backward, %d streams" % n, 1.0)
+
+
 def test_latency_measurement_feeds_the_planner():
     """measure_layer_latency -> fit_latency_grid -> best_plan on a small stack: every requested point is
     measured, latencies are positive, and the plan covers the sequence (at this size the times are launch
