@@ -192,7 +192,7 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
                             st.cache_len, float(Dh) ** -0.5, accumulate_prefix, has_incoming, zero_slice_rows,
                             colsum_dqkv_acc=sa.get("attn.in_proj.bias"), delta=buf.delta,
                             q_bh_rows=st.q_bh_rows, stat_bh_rows=st.stat_bh_rows)
-    elif suffix.get("o_all") is not None and suffix["own_end"] - st.cache_len <= ops.FUSED_BWD_MAX_OWN:
+    elif suffix.get("o_all") is not None and suffix["own_end"] - st.cache_len <= ops.FUSED_BWD_WINDOW:
         # dQ of the slice and dK / dV of its keys over all later positions as one launch.  The dK/dV half takes delta
         # of the positions up to own_end itself, so what it needs of the later slices is their dO (and, past own_end,
         # their delta): the slice waits for the next slice's event and records its own BEFORE the launch

@@ -589,7 +589,8 @@ class TeraPipe(nn.Module):
     False (and always in fp32) the gradient caches are used.
     fused_attn_bwd (with suffix_dkdv): dQ of a slice and the one-pass dK/dV of its keys go out as one launch whose
     two halves run side by side (the first streams the keys before the slice, the second the queries after it)
-    instead of two launches one after the other.  Same results.
+    instead of two launches one after the other, whenever the slice and the slice_streams - 1 slices after it are
+    at most ops.FUSED_BWD_WINDOW positions together (the launch recomputes their delta).  Same results.
     slice_streams (with suffix_dkdv, fp16 / bf16): slice i runs on stream i mod slice_streams.  The attention
     kernel of a layer waits (by event) for the in_proj GEMMs of the earlier slices at that layer, the one-pass
     dK/dV kernel for the dQ kernels of the later slices; nothing else orders slices, so consecutive slices
