@@ -765,18 +765,32 @@ def test_replay_survives_a_larger_workspace_on_the_same_stream():
     assert_close(C, A.float() @ Bm.float().t(), dtype, "the large product itself")
 
 
-def test_default_runner_matches_single_stream_at_c2_shape():
+@pytest.mark.parametrize("n_layers,steps", [(2, 5), (24, 4)])
+def test_default_runner_matches_single_stream_at_c2_shape(n_layers, steps):
     """BASELINE config 2's geometry (hidden 2048, 16 heads, FFN 8192, sequence 2048 as 8 x 256, fp16) on two
-    layers: the constructor's defaults (three slice streams, launch replay) against one stream launched
-    from Python, five steps -- the first as written, the second recorded, the rest re-issued.  Same kernels
-    on the same data: outputs and input gradients are bit-identical; the parameter gradients (fp32 atomics
-    for the vector parameters) agree to rounding."""
+    layers and on all 24: the constructor's defaults (three slice streams, launch replay) against one stream
+    launched from Python, several steps -- the first as written, the second recorded, the rest re-issued.  Same
+    kernels on the same data: outputs and input gradients are bit-identical; the parameter gradients (fp32
+    atomics for the vector parameters) agree to rounding."""
     ta = _mods()
     dtype = torch.float16
-    n_layers, E, H, Fd, L, B = 2, 2048, 16, 8192, 2048, 1
+    E, H, Fd, L, B = 2048, 16, 8192, 2048, 1
     ss = [256] * 8
-    ps = make_params(n_layers, E, Fd, dtype, seed=21)
-    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    print("C2 geometry, %d layers, %d steps" % (n_layers, steps), flush=True)
+    if n_layers <= 2:
+        ps = make_params(n_layers, E, Fd, dtype, seed=21)
+        layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    else:
+        # (the full stack's parameters are drawn on the device: 1.2 G values)
+        layers = ta.TransformerLayers(n_layers, E, Fd, H, dtype=dtype, device=DEV)
+        gd = torch.Generator(device=DEV).manual_seed(21)
+        with torch.no_grad():
+            for layer in layers.layers:
+                for name, t in layer.param_dict().items():
+                    if name.endswith("ln.weight"):
+                        t.copy_(1.0 + 0.2 * torch.randn(t.shape, generator=gd, device=DEV))
+                    else:
+                        t.copy_(torch.randn(t.shape, generator=gd, device=DEV) * (0.1 if name.endswith("bias") else 0.02))
     fast = ta.TeraPipe(layers, B, L, [B], ss)
     plain = ta.TeraPipe(layers, B, L, [B], ss, slice_streams=1, launch_replay=False)
     assert fast.slice_streams == 3 and fast.launch_replay
@@ -789,7 +803,7 @@ def test_default_runner_matches_single_stream_at_c2_shape():
         (y * dy).sum().backward()
         return y.detach().clone(), xd.grad.clone(), [p.grad.clone() for p in layers.parameters()]
 
-    for seed in range(5):
+    for seed in range(steps):
         g = torch.Generator().manual_seed(700 + seed)
         x = torch.randn(L, B, E, generator=g).to(dtype).to(DEV)
         dy = (torch.randn(L, B, E, generator=g) * 0.1).to(dtype).to(DEV)
