@@ -152,6 +152,9 @@ typedef struct tp_gemm_desc {
 
 /* number of k splits the plan uses for this product (1 = none; 0 = invalid descriptor) */
 int tp_gemm_splits(const tp_gemm_desc* d);
+/* The plan tp_gemm would run the product with: the tile configuration's number (the kernel and tile shape, as listed
+ * in csrc/gemm.hip) and the number of k splits.  Host code only; for tuning, tests and logs. */
+int tp_gemm_plan(const tp_gemm_desc* d, int* tile_cfg, int* nsplit);
 size_t tp_gemm_workspace_bytes(const tp_gemm_desc* d);
 int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_bytes, void* stream);
 /* n independent products as if by n tp_gemm calls in order on the stream (the four weight gradients of a layer,

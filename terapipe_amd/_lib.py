@@ -107,6 +107,7 @@ SYMBOLS = {
     "tp_layernorm_bwd_partials": (c_int, [c_void_p, c_int] + [c_void_p] * 11 + [c_int, c_int, c_int, c_void_p]),
     "tp_vec_param_grads": (c_int, [ctypes.POINTER(VecGradDesc), c_int, c_int, c_void_p]),
     "tp_gemm_splits": (c_int, [ctypes.POINTER(GemmDesc)]),
+    "tp_gemm_plan": (c_int, [ctypes.POINTER(GemmDesc), ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "tp_gemm_workspace_bytes": (c_size_t, [ctypes.POINTER(GemmDesc)]),
     "tp_gemm": (c_int, [ctypes.POINTER(GemmDesc), c_void_p, c_size_t, c_void_p]),
     "tp_gemm_static_ws_capacity": (c_size_t, []),

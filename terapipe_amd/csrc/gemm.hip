@@ -648,29 +648,53 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     // bits 8-15 force the number of k splits.  For tuning and tests.
     int forced_cfg = (d->reserved & 0xff) - 1;
     int forced_split = (d->reserved >> 8) & 0xff;
-    // Measured on MI355X: the 128 x 128 x 64 two-stage tile (two workgroups per CU) wins whenever its
-    // tile count comes near the CU count, 64 x 64 x 64 otherwise; k is split to reach about two
-    // workgroups per CU as long as every split keeps at least 2048 (small tiles) / 1024 (large) of k.
     const long t128 = (long)((d->M + 127) / 128) * ((d->N + 127) / 128);
     const long t64 = (long)((d->M + 63) / 64) * ((d->N + 63) / 64);
     int cfg, ns = 1;
     const long t256n = (d->N + 255) / 256;
     const long t256 = (long)((d->M + 255) / 256) * t256n;
-    if (d->M <= 64 && (long)d->N * d->K >= (64L << 20)) {
-        // a short activation against a large weight: 64 x 256 x 64 tiles stream the weight with a quarter
-        // of the activation re-reads of 64-wide tiles; k is split to about 200 workgroups
-        cfg = 11;
-        ns = (int)((208 + t256n / 2) / t256n);
-        int maxs = d->K / 1536;
-        if (ns > maxs) ns = maxs;
-        if (ns > 8) ns = 8;
-    } else if (d->M > 64 && d->M <= 128 && t128 >= 64 && d->K >= 4096) {
-        // one row of 128 x 256 x 64 tiles (eight waves) streaming the weight once
-        cfg = 3;
-        ns = t256n >= 176 ? 1 : (t256n >= 96 ? 3 : (int)((192 + t256n - 1) / t256n));
-        int maxs = d->K / 2048;
-        if (ns > maxs) ns = maxs;
-        if (ns > 8) ns = 8;
+    // k splits that bring `tiles` workgroups as near to one per CU as they get without exceeding it (a second, partly
+    // filled round costs more than the idle CUs) while every split keeps at least min_k of k
+    auto splits_for = [&](long tiles, int min_k) {
+        int v = (int)(kNumCU / tiles);
+        const int maxs = d->K / min_k;
+        if (v > maxs) v = maxs;
+        if (v > 8) v = 8;
+        return v < 1 ? 1 : v;
+    };
+    if (d->op != TP_GEMM_TN && d->M <= 512) {
+        // A slice's linears, forward (NT) and data gradient (NN): up to 512 rows against a weight.  The rules are the
+        // common ground of sweeps over every tile configuration and split on layer geometries that have no entry in
+        // the measured table (hidden 3072 to 10240, 64 to 512 rows): about one workgroup per CU is the target -- fewer
+        // leave CUs without a share of the weight stream, every extra split adds a round of fp32 partial sums and
+        // does not pay below 1536-2048 of k per split -- and the tile grows with the slice so that the activation,
+        // which every column tile re-reads, stays the smaller part of what a CU has to fill.
+        const long t3 = (long)((d->M + 127) / 128) * t256n;          // 128 x 256 tiles
+        const bool small_weight = (long)d->N * d->K <= (16L << 20);  // 4096 x 4096 and below
+        if (d->M <= 64) {
+            // one row of tiles: 64 x 64 until they come to more than two per CU, then 64 x 256
+            if (t64 >= 2 * kNumCU) { cfg = 11; ns = splits_for(t256n, 2048); }
+            else { cfg = 8; ns = splits_for(t64, 2048); }
+        } else if (small_weight) {
+            // 64 x 64 tiles reach the CU count without splitting k
+            cfg = (d->M <= 256 && d->K % 128 == 0) ? 12 : 8;
+            ns = t64 >= 96 ? 1 : splits_for(t64, 2048);
+        } else if (d->M <= 128) {
+            const int ns13 = splits_for(t128, 1536);
+            if (t128 > kNumCU) { cfg = 3; ns = splits_for(t3, 2048); }                      // many column tiles: 128 x 256
+            else if (t128 * ns13 < 192 && t64 >= 192 && t64 <= 2 * kNumCU) { cfg = 8; }     // too few 128 x 128 tiles for the chip
+            else { cfg = 13; ns = ns13; }
+        } else if (d->M > 448 && d->K % 64 == 0 && t256 >= 160) {
+            cfg = 19;               // two full rows of 256 x 256 tiles for most of the CUs
+        } else if (d->M > 256 && d->M <= 384 && d->K % 64 == 0 && t3 > kNumCU) {
+            cfg = 33;               // two row tiles of 192 x 256 (the weight-streaming kernel) where 128 x 256 tiles are too many
+            ns = splits_for(2 * t256n, 2048);
+        } else {
+            // 128 x 256 tiles when a split still keeps 4096 of k, to amortise the larger tile's prologue; else 128 x 128
+            const int ns3 = splits_for(t3, 2048);
+            if (d->K / ns3 >= 4096 || t128 > kNumCU) { cfg = 3; ns = ns3; }
+            else { cfg = 13; ns = splits_for(t128, 2048); }
+        }
     } else if ((d->op == TP_GEMM_TN || d->M >= 512) && d->K % 64 == 0 && t256 >= 192) {
         // parameter gradients of a whole step, and any product of 512 rows or more with that many tiles (the LM
         // head): 256 x 256 tiles by eight waves (half the bytes per flop of a 128 x 128 tile through the
@@ -823,6 +847,15 @@ static int validate_gemm(const tp_gemm_desc* d) {
 extern "C" int tp_gemm_splits(const tp_gemm_desc* d) {
     if (tp::validate_gemm(d) != TP_OK) return 0;
     return tp::plan_gemm(d).nsplit;
+}
+
+extern "C" int tp_gemm_plan(const tp_gemm_desc* d, int* tile_cfg, int* nsplit) {
+    int rc = tp::validate_gemm(d);
+    if (rc != TP_OK) return rc;
+    tp::GemmPlan p = tp::plan_gemm(d);
+    if (tile_cfg) *tile_cfg = p.cfg;
+    if (nsplit) *nsplit = p.nsplit;
+    return TP_OK;
 }
 
 extern "C" size_t tp_gemm_workspace_bytes(const tp_gemm_desc* d) {

@@ -82,7 +82,9 @@ class Workspace:
     """A grow-only scratch tensor per device and stream (torch-owned), handed to calls that need
     workspace: kernels of different streams may run at the same time and must not share partial sums.
     A buffer that is outgrown is kept for the life of the process, never returned to torch's allocator:
-    recorded launches and captured HIP graphs hold its raw address and may run again at any time."""
+    recorded launches and captured HIP graphs hold its raw address and may run again at any time.  A new
+    buffer is at least half as large again as the one it replaces, so that the outgrown ones of a stream
+    add up to no more than twice its current buffer however the requests creep up."""
     _bufs = {}
     _superseded = []
 
@@ -94,9 +96,11 @@ class Workspace:
         key = (device.type, device.index, stream)
         buf = cls._bufs.get(key)
         if buf is None or buf.numel() < nbytes:
+            size = max(int(nbytes), 1 << 20)
             if buf is not None:
                 cls._superseded.append(buf)
-            buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+                size = max(size, buf.numel() + buf.numel() // 2)
+            buf = torch.empty(size, dtype=torch.uint8, device=device)
             cls._bufs[key] = buf
         return buf
 

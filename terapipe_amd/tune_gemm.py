@@ -39,10 +39,15 @@ SPLITS = [1, 2, 3, 4, 6, 8]
 OPS = {"NT": _lib.TP_GEMM_NT, "NN": _lib.TP_GEMM_NN, "TN": _lib.TP_GEMM_TN}
 
 
+_PAIR_STREAMS = []
+
+
 def _time_pair_us(fn, n=6):
     """Two chains of the same call on two streams inside one graph: time per call when a neighbour shares the GPU
     (the runner overlaps consecutive slices on two streams)."""
-    s0, s1 = torch.cuda.Stream(), torch.cuda.Stream()
+    while len(_PAIR_STREAMS) < 2:
+        _PAIR_STREAMS.append(torch.cuda.Stream())
+    s0, s1 = _PAIR_STREAMS
     fn(0, 0)
     fn(1, 1)
     torch.cuda.synchronize()
@@ -72,10 +77,16 @@ def _time_pair_us(fn, n=6):
     return e0.elapsed_time(e1) / (4 * n) * 1e3
 
 
+_WARMUP_STREAM = []
+
+
 def _time_us(fn, n=6):
     fn(0)
     torch.cuda.synchronize()
-    side = torch.cuda.Stream()
+    # one side stream for every call: the library's workspaces are per stream and never shrink
+    if not _WARMUP_STREAM:
+        _WARMUP_STREAM.append(torch.cuda.Stream())
+    side = _WARMUP_STREAM[0]
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         fn(1)
