@@ -154,7 +154,7 @@ def cpu_baseline(w, sample_layers=None):
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
     flops_layer = gemm_flops_per_step(w) / w["n_layers"]
-    sample_layers = sample_layers or max(1, min(w["n_layers"], int(0.8e13 // flops_layer)))
+    sample_layers = sample_layers or max(1, min(w["n_layers"], int(1.3e13 // flops_layer)))
     ps = oracle.init_stack_params(sample_layers, w["E"], w["F"], w["std"], torch.float32, seed=0)
     for p in ps:
         for v in p.values():
