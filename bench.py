@@ -83,8 +83,9 @@ def gemm_shape_name(meta):
 
 
 def pmc_traffic(workload):
-    """HBM bytes per GEMM launch of a step, from the committed summary of the two rocprofv3 --pmc runs
-    (FETCH_SIZE, WRITE_SIZE) over one step of this workload; None when no such summary is in the tree."""
+    """Bytes per GEMM launch of a step between L2 and the fabric, from the committed summary of the two rocprofv3 --pmc
+    runs (FETCH_SIZE, WRITE_SIZE, each scaled by its reading on kernels of known size) over one step of this workload;
+    None when no such summary is in the tree."""
     path = os.path.join(ROOT, "profiles", "bench_%s_gemm_hbm_traffic.pmc.txt" % workload)
     try:
         m = re.search(r"traffic_bytes_per_gemm_launch:\s*([0-9.eE+]+)", open(path).read())
@@ -284,6 +285,10 @@ def measure_workload(name, args, device, detail):
                   "split-K reduce included)",
         "bound": "mfma", "achieved": achieved / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
         "frac": achieved / peak, "traffic": pmc_traffic(name),
+        "traffic_note": "bytes per launch that L2 exchanges with the fabric (the memory-side cache serves part of them): rocprofv3 "
+                        "FETCH_SIZE / 0.500 + WRITE_SIZE / 1.000, the factors read off a plain copy and a fill of known size in "
+                        "the same counter runs; from the committed profiles/ summary of one eager step",
+        "algorithmic_bytes_per_launch": sum(b for _f, b in work) / max(len(gemm_calls), 1),
         "launches": len(gemm_calls), "avg_launch_us": g_ms * 1e3 / max(len(gemm_calls), 1),
         "algorithmic_flops_per_step": flops, "kernel_ms_per_step": g_ms,
         "attainable": attainable / 1e12, "attainable_frac": attainable / peak,
