@@ -186,7 +186,7 @@ int tp_gemm_static_ws(const tp_gemm_desc* d, void* stream);
  */
 typedef struct tp_attn_desc {
     int32_t dtype;
-    int32_t batch, heads, head_dim;     /* head_dim must be 64 or 128 */
+    int32_t batch, heads, head_dim;     /* 16, 32, 64, 80, 96 or 128 */
     int32_t T;                          /* slice length */
     int32_t cache_len;                  /* P: rows of the caches filled by earlier slices */
     int64_t cache_rows;                 /* L_max */
@@ -236,7 +236,7 @@ int tp_attn_prefix_bwd(const tp_attn_desc* d, void* workspace, size_t workspace_
  * Query position t in [key_begin, q_end) sees key position s <= t.  Writes the k and v parts of dqkv. */
 typedef struct tp_attn_suffix_desc {
     int32_t dtype;                      /* TP_F16 or TP_BF16 */
-    int32_t batch, heads, head_dim;
+    int32_t batch, heads, head_dim;     /* head_dim 64 or 128 */
     int32_t key_begin, key_count;       /* P, T of the slice whose keys these are */
     int32_t q_end;                      /* queries [key_begin, q_end) take part */
     int32_t reserved;

@@ -86,8 +86,9 @@ __device__ __forceinline__ void mfma_acc_as_b(float16v* acc, const T* tile, int 
 template <typename T, int DH, int NW, int BN>
 __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs a) {
     typedef Elem<T> E;
-    typedef TileLayout<T, DH> L;
-    constexpr int NT = NW * 64, NKB = BN / 32, NDB = DH / 32, NKS = DH / E::KSTEP;
+    constexpr int DP = (DH + 31) / 32 * 32;   // LDS tiles and accumulators are padded to whole 32-column blocks
+    typedef TileLayout<T, DP> L;
+    constexpr int NT = NW * 64, NKB = BN / 32, NDB = DP / 32, NKS = DH / E::KSTEP;
     __shared__ __attribute__((aligned(16))) T sK[L::size(BN)];
     __shared__ __attribute__((aligned(16))) T sV[L::size(BN)];
 
@@ -114,7 +115,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs a) {
 
     const T* Kb = reinterpret_cast<const T*>(a.kc) + (long)bh * a.cache_rows * DH;
     const T* Vb = reinterpret_cast<const T*>(a.vc) + (long)bh * a.cache_rows * DH;
-    TileCopy<T, BN, DH, NT> ck, cv;
+    TileCopy<T, BN, DP, NT> ck, cv;
     if (t_beg < t_end) {
         ck.load(Kb, DH, t_beg * BN, 0, S, DH, tid);
         cv.load(Vb, DH, t_beg * BN, 0, S, DH, tid);
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs a) {
                 for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
 #pragma unroll
                 for (int ks = 0; ks < NKS; ++ks) {
-                    typename E::opnd_t kop = fetch_km<T, DH>(sK, kb * 32 + li, ks * E::KSTEP, lane);
+                    typename E::opnd_t kop = fetch_km<T, DP>(sK, kb * 32 + li, ks * E::KSTEP, lane);
                     sacc[kb] = E::mfma(kop, qreg[ks], sacc[kb]);
                 }
             }
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
 #pragma unroll
-            for (int kb = 0; kb < NKB; ++kb) mfma_acc_as_b<T, DH>(oacc, sV, kb * 32, sacc[kb], lane);
+            for (int kb = 0; kb < NKB; ++kb) mfma_acc_as_b<T, DP>(oacc, sV, kb * 32, sacc[kb], lane);
         }
         __syncthreads();
         if (t + 1 < t_end) {
@@ -191,6 +192,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
                 for (int jq = 0; jq < 4; ++jq) {
                     int dh = db * 32 + 8 * jq + 4 * g;
+                    if (DP != DH && dh >= DH) continue;
                     store4<T>(O + dh, oacc[db][4 * jq] * inv, oacc[db][4 * jq + 1] * inv,
                               oacc[db][4 * jq + 2] * inv, oacc[db][4 * jq + 3] * inv);
                 }
@@ -203,6 +205,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
                 for (int jq = 0; jq < 4; ++jq) {
                     int dh = db * 32 + 8 * jq + 4 * g;
+                    if (DP != DH && dh >= DH) continue;
                     *reinterpret_cast<float4*>(PO + dh) =
                         make_float4(oacc[db][4 * jq] * inv, oacc[db][4 * jq + 1] * inv,
                                     oacc[db][4 * jq + 2] * inv, oacc[db][4 * jq + 3] * inv);
@@ -224,21 +227,24 @@ __global__ __launch_bounds__(256) void attn_fwd_merge_kernel(AttnArgs a) {
     float mx = -INFINITY;
     for (int z = 0; z < a.nsplit; ++z) mx = fmaxf(mx, a.part_lse[(long)z * BH * a.T + row]);
     float wsum = 0.f;
-    float acc[DH / 64];
+    constexpr int NC = (DH + 63) / 64;
+    float acc[NC];
 #pragma unroll
-    for (int i = 0; i < DH / 64; ++i) acc[i] = 0.f;
+    for (int i = 0; i < NC; ++i) acc[i] = 0.f;
     for (int z = 0; z < a.nsplit; ++z) {
         float l = a.part_lse[(long)z * BH * a.T + row];
         float w = l == -INFINITY ? 0.f : exp2f((l - mx) * kLog2e);
         wsum += w;
         const float* PO = a.part_o + ((long)z * BH * a.T + row) * DH;
 #pragma unroll
-        for (int i = 0; i < DH / 64; ++i) acc[i] += w * PO[lane + 64 * i];
+        for (int i = 0; i < NC; ++i)
+            if (DH % 64 == 0 || lane + 64 * i < DH) acc[i] += w * PO[lane + 64 * i];
     }
     T* O = reinterpret_cast<T*>(a.o) + ((long)t * a.B + b) * ((long)a.H * DH) + (long)h * DH;
     const float inv = 1.0f / wsum;
 #pragma unroll
-    for (int i = 0; i < DH / 64; ++i) O[lane + 64 * i] = Elem<T>::from_float(acc[i] * inv);
+    for (int i = 0; i < NC; ++i)
+        if (DH % 64 == 0 || lane + 64 * i < DH) O[lane + 64 * i] = Elem<T>::from_float(acc[i] * inv);
     if (lane == 0) a.lse[(long)bh * a.st_bhs + t] = mx + logf(wsum);
 }
 
@@ -260,8 +266,9 @@ __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(AttnArgs a) {
     const T* dO = reinterpret_cast<const T*>(a.d_o) + off;
     float s = 0.f;
 #pragma unroll
-    for (int i = 0; i < DH / 64; ++i)
-        s += Elem<T>::to_float(O[lane + 64 * i]) * Elem<T>::to_float(dO[lane + 64 * i]);
+    for (int i = 0; i < (DH + 63) / 64; ++i)
+        if (DH % 64 == 0 || lane + 64 * i < DH)
+            s += Elem<T>::to_float(O[lane + 64 * i]) * Elem<T>::to_float(dO[lane + 64 * i]);
     s = wave_sum(s);
     if (lane == 0) a.delta[((long)b * a.H + h) * a.st_bhs + t] = s;
 }
@@ -270,8 +277,9 @@ __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(AttnArgs a) {
 template <typename T, typename GT, int DH, int NW>
 __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_kernel(AttnArgs a) {
     typedef Elem<T> E;
-    typedef TileLayout<T, DH> L;
-    constexpr int NT = NW * 64, NDB = DH / 32, NKS = DH / E::KSTEP;
+    constexpr int DP = (DH + 31) / 32 * 32;
+    typedef TileLayout<T, DP> L;
+    constexpr int NT = NW * 64, NDB = DP / 32, NKS = DH / E::KSTEP;
     __shared__ __attribute__((aligned(16))) T sQ[L::size(32)];
     __shared__ __attribute__((aligned(16))) T sdO[L::size(32)];
     __shared__ __attribute__((aligned(16))) float sLse[32];
@@ -299,7 +307,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_kernel(AttnArgs a) {
     const T* dOb = reinterpret_cast<const T*>(a.d_o) + (long)b * EE + (long)h * DH;  // row t at stride B*E
     const int nqb = (T_ + 31) / 32;
     const int qb_start = key0wg > P ? (key0wg - P) / 32 : 0;
-    TileCopy<T, 32, DH, NT> cq, cdo;
+    TileCopy<T, 32, DP, NT> cq, cdo;
     for (int qb = qb_start; qb < nqb; ++qb) {
         cq.load(Qb, DH, qb * 32, 0, T_, DH, tid);
         cdo.load(dOb, (long)a.B * EE, qb * 32, 0, T_, DH, tid);
@@ -318,9 +326,9 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_kernel(AttnArgs a) {
             for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; pacc[r] = 0.f; }
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) {
-                typename E::opnd_t qop = fetch_km<T, DH>(sQ, li, ks * E::KSTEP, lane);
+                typename E::opnd_t qop = fetch_km<T, DP>(sQ, li, ks * E::KSTEP, lane);
                 sacc = E::mfma(qop, kreg[ks], sacc);
-                typename E::opnd_t doop = fetch_km<T, DH>(sdO, li, ks * E::KSTEP, lane);
+                typename E::opnd_t doop = fetch_km<T, DP>(sdO, li, ks * E::KSTEP, lane);
                 pacc = E::mfma(doop, vreg[ks], pacc);
             }
 #pragma unroll
@@ -340,8 +348,8 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_kernel(AttnArgs a) {
                     pacc[j] = ds;
                 }
             }
-            mfma_acc_as_b<T, DH>(dv, sdO, 0, sacc, lane);
-            mfma_acc_as_b<T, DH>(dk, sQ, 0, pacc, lane);
+            mfma_acc_as_b<T, DP>(dv, sdO, 0, sacc, lane);
+            mfma_acc_as_b<T, DP>(dk, sQ, 0, pacc, lane);
         }
     }
 
@@ -354,6 +362,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_kernel(AttnArgs a) {
 #pragma unroll
                 for (int jq = 0; jq < 4; ++jq) {
                     int dh = db * 32 + 8 * jq + 4 * g;
+                    if (DP != DH && dh >= DH) continue;
                     float ok[4] = {0.f, 0.f, 0.f, 0.f}, ov[4] = {0.f, 0.f, 0.f, 0.f};
                     if (a.accumulate_prefix) { load4<GT>(gK + dh, ok); load4<GT>(gV + dh, ov); }
                     store4<GT>(gK + dh, ok[0] + dk[db][4 * jq], ok[1] + dk[db][4 * jq + 1],
@@ -369,6 +378,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_kernel(AttnArgs a) {
 #pragma unroll
                 for (int jq = 0; jq < 4; ++jq) {
                     int dh = db * 32 + 8 * jq + 4 * g;
+                    if (DP != DH && dh >= DH) continue;
                     float ok[4] = {0.f, 0.f, 0.f, 0.f}, ov[4] = {0.f, 0.f, 0.f, 0.f};
                     if (a.has_incoming) { load4<GT>(gK + dh, ok); load4<GT>(gV + dh, ov); }
                     store4<T>(dst + DH + dh, ok[0] + dk[db][4 * jq], ok[1] + dk[db][4 * jq + 1],
@@ -388,8 +398,9 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dkdv_kernel(AttnArgs a) {
 template <typename T, int DH, int NW, int BN>
 __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_kernel(AttnArgs a) {
     typedef Elem<T> E;
-    typedef TileLayout<T, DH> L;
-    constexpr int NT = NW * 64, NKB = BN / 32, NDB = DH / 32, NKS = DH / E::KSTEP;
+    constexpr int DP = (DH + 31) / 32 * 32;   // LDS tiles and accumulators are padded to whole 32-column blocks
+    typedef TileLayout<T, DP> L;
+    constexpr int NT = NW * 64, NKB = BN / 32, NDB = DP / 32, NKS = DH / E::KSTEP;
     __shared__ __attribute__((aligned(16))) T sK[L::size(BN)];
     __shared__ __attribute__((aligned(16))) T sV[L::size(BN)];
 
@@ -417,7 +428,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_kernel(AttnArgs a) {
 
     const T* Kb = reinterpret_cast<const T*>(a.kc) + (long)bh * a.cache_rows * DH;
     const T* Vb = reinterpret_cast<const T*>(a.vc) + (long)bh * a.cache_rows * DH;
-    TileCopy<T, BN, DH, NT> ck, cv;
+    TileCopy<T, BN, DP, NT> ck, cv;
     if (ntiles > 0) {
         ck.load(Kb, DH, 0, 0, S, DH, tid);
         cv.load(Vb, DH, 0, 0, S, DH, tid);
@@ -439,9 +450,9 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_kernel(AttnArgs a) {
                 for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; pacc[r] = 0.f; }
 #pragma unroll
                 for (int ks = 0; ks < NKS; ++ks) {
-                    typename E::opnd_t kop = fetch_km<T, DH>(sK, kb * 32 + li, ks * E::KSTEP, lane);
+                    typename E::opnd_t kop = fetch_km<T, DP>(sK, kb * 32 + li, ks * E::KSTEP, lane);
                     sacc = E::mfma(kop, qreg[ks], sacc);
-                    typename E::opnd_t vop = fetch_km<T, DH>(sV, kb * 32 + li, ks * E::KSTEP, lane);
+                    typename E::opnd_t vop = fetch_km<T, DP>(sV, kb * 32 + li, ks * E::KSTEP, lane);
                     pacc = E::mfma(vop, doreg[ks], pacc);
                 }
 #pragma unroll
@@ -450,7 +461,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_kernel(AttnArgs a) {
                     float p = key > P + tq ? 0.f : exp2f((sacc[j] - lse_q) * kLog2e);
                     pacc[j] = p * (pacc[j] - delta_q);
                 }
-                mfma_acc_as_b<T, DH>(dq, sK, kb * 32, pacc, lane);
+                mfma_acc_as_b<T, DP>(dq, sK, kb * 32, pacc, lane);
             }
         }
         __syncthreads();
@@ -467,6 +478,7 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_kernel(AttnArgs a) {
 #pragma unroll
             for (int jq = 0; jq < 4; ++jq) {
                 int dh = db * 32 + 8 * jq + 4 * g;
+                if (DP != DH && dh >= DH) continue;
                 store4<T>(dst + dh, dq[db][4 * jq] * a.qscale, dq[db][4 * jq + 1] * a.qscale,
                           dq[db][4 * jq + 2] * a.qscale, dq[db][4 * jq + 3] * a.qscale);
             }
@@ -1554,11 +1566,28 @@ __global__ __launch_bounds__(256) void attn_bwd_fused_kernel(AttnArgs a, SuffixA
 // ------------------------------------------------------------------------------------------------
 static constexpr int kNumCU = 256;
 
+// head dimensions of the 16-bit kernels with direct global->LDS loads; the others run, in every dtype, on the
+// register-staged kernels, whose LDS tiles pad the head dimension to whole 32-column blocks
+static inline bool tiled16(int head_dim) { return head_dim == 64 || head_dim == 128; }
+static inline bool known_head_dim(int hd) { return hd == 16 || hd == 32 || hd == 64 || hd == 80 || hd == 96 || hd == 128; }
+
+// calls f(std::integral_constant<int, hd>) for a known head dimension
+template <typename F> static void for_head_dim(int hd, F&& f) {
+    switch (hd) {
+    case 16: f(std::integral_constant<int, 16>()); break;
+    case 32: f(std::integral_constant<int, 32>()); break;
+    case 64: f(std::integral_constant<int, 64>()); break;
+    case 80: f(std::integral_constant<int, 80>()); break;
+    case 96: f(std::integral_constant<int, 96>()); break;
+    default: f(std::integral_constant<int, 128>()); break;
+    }
+}
+
 static int validate_attn(const tp_attn_desc* d, bool bwd) {
     const char* who = bwd ? "tp_attn_prefix_bwd" : "tp_attn_prefix_fwd";
     if (!d) { set_error("%s: null descriptor", who); return TP_ERR_ARG; }
     if (d->dtype < TP_F32 || d->dtype > TP_BF16) { set_error("%s: bad dtype %d", who, d->dtype); return TP_ERR_ARG; }
-    if (d->head_dim != 64 && d->head_dim != 128) { set_error("%s: head_dim %d not supported (64 or 128)", who, d->head_dim); return TP_ERR_UNSUPPORTED; }
+    if (!known_head_dim(d->head_dim)) { set_error("%s: head_dim %d not supported (16, 32, 64, 80, 96 or 128)", who, d->head_dim); return TP_ERR_UNSUPPORTED; }
     if (d->batch <= 0 || d->heads <= 0 || d->T <= 0 || d->cache_len < 0) { set_error("%s: bad geometry B=%d H=%d T=%d P=%d", who, d->batch, d->heads, d->T, d->cache_len); return TP_ERR_ARG; }
     if ((long)d->cache_len + d->T > d->cache_rows) { set_error("%s: slice [%d, %d) does not fit a cache of %ld rows", who, d->cache_len, d->cache_len + d->T, (long)d->cache_rows); return TP_ERR_ARG; }
     if (!d->q || !d->k_cache || !d->v_cache || !d->o || !d->lse) { set_error("%s: null tensor", who); return TP_ERR_ARG; }
@@ -1576,7 +1605,7 @@ struct FwdPlan { int nw, bn, nsplit, qblocks; };
 
 static FwdPlan plan_fwd(const tp_attn_desc* d) {
     FwdPlan p;
-    if (d->dtype != TP_F32) {
+    if (d->dtype != TP_F32 && tiled16(d->head_dim)) {
         // 16-bit: one workgroup per 32 queries whose four waves split the key range and merge in LDS
         p.nw = 0; p.bn = 32; p.nsplit = 1; p.qblocks = (d->T + 31) / 32;
         // A call with so few query blocks that over half of the CUs would get no workgroup, and a key range long
@@ -1636,7 +1665,7 @@ static AttnArgs make_args(const tp_attn_desc* d) {
 template <typename T, int DH>
 static void launch_fwd(const FwdPlan& p, const AttnArgs& a, hipStream_t s) {
     dim3 grid(p.qblocks, a.B * a.H, p.nsplit);
-    if constexpr (sizeof(T) == 2) {
+    if constexpr (sizeof(T) == 2 && (DH == 64 || DH == 128)) {
         const dim3 g2(xcd_grid(a.B * a.H, (a.T + 31) / 32), p.nsplit);
         if (p.bn == 8) attn_fwd2_kernel<T, DH, 8, 1><<<g2, 512, 0, s>>>(a);
         else attn_fwd2_kernel<T, DH, 4><<<g2, 256, 0, s>>>(a);
@@ -1655,7 +1684,8 @@ template <typename T, typename GT, int DH>
 static void launch_bwd(const AttnArgs& a, hipStream_t s) {
     const int S = a.P + a.T;
     long rows = (long)a.T * a.B * a.H;
-    if constexpr (sizeof(T) == 2) {
+    constexpr bool kTiled16 = sizeof(T) == 2 && (DH == 64 || DH == 128);
+    if constexpr (kTiled16) {
         // dQ first: it also leaves delta for the dK/dV kernel
         attn_bwd_dq2_kernel<T, DH, 4><<<xcd_grid(a.B * a.H, (a.T + 31) / 32), 256, 0, s>>>(a);
     } else {
@@ -1668,8 +1698,8 @@ static void launch_bwd(const AttnArgs& a, hipStream_t s) {
         if (((S + 127) / 128) * bh < 2L * kNumCU) nw = 2;
         if (((S + 63) / 64) * bh < 2L * kNumCU) nw = 1;
         dim3 grid((S + 32 * nw - 1) / (32 * nw), (unsigned)bh);
-        if (sizeof(T) == 2 && a.T <= kMaxTLds) {
-            if constexpr (sizeof(T) == 2) {
+        if (kTiled16 && a.T <= kMaxTLds) {
+            if constexpr (kTiled16) {
                 const size_t dyn = (size_t)2 * ((a.T + 31) / 32) * 32 * sizeof(float);
                 const unsigned g2 = xcd_grid((int)bh, (int)grid.x);
                 if (nw == 4) attn_bwd_dkdv2_kernel<T, GT, DH, 4, 3><<<g2, 256, dyn, s>>>(a);
@@ -1682,7 +1712,7 @@ static void launch_bwd(const AttnArgs& a, hipStream_t s) {
             else attn_bwd_dkdv_kernel<T, GT, DH, 1><<<grid, 64, 0, s>>>(a);
         }
     }
-    if constexpr (sizeof(T) == 4) {
+    if constexpr (!kTiled16) {
         int nw = a.T > 64 ? 4 : (a.T > 32 ? 2 : 1);
         if (nw == 4 && (long)((a.T + 127) / 128) * a.B * a.H < kNumCU / 2) nw = 2;
         dim3 grid((a.T + 32 * nw - 1) / (32 * nw), a.B * a.H);
@@ -1696,24 +1726,13 @@ static void launch_bwd(const AttnArgs& a, hipStream_t s) {
 
 template <typename T>
 static void dispatch_fwd(int hd, const FwdPlan& p, const AttnArgs& a, hipStream_t s) {
-    if (hd == 64) launch_fwd<T, 64>(p, a, s);
-    else launch_fwd<T, 128>(p, a, s);
+    for_head_dim(hd, [&](auto dh) { launch_fwd<T, decltype(dh)::value>(p, a, s); });
 }
 
 template <typename T>
 static void dispatch_bwd(int hd, bool f32grad, const AttnArgs& a, hipStream_t s) {
-    if constexpr (sizeof(T) == 4) {
-        if (hd == 64) launch_bwd<T, float, 64>(a, s);
-        else launch_bwd<T, float, 128>(a, s);
-    } else {
-        if (f32grad) {
-            if (hd == 64) launch_bwd<T, float, 64>(a, s);
-            else launch_bwd<T, float, 128>(a, s);
-        } else {
-            if (hd == 64) launch_bwd<T, T, 64>(a, s);
-            else launch_bwd<T, T, 128>(a, s);
-        }
-    }
+    if (sizeof(T) == 4 || f32grad) for_head_dim(hd, [&](auto dh) { launch_bwd<T, float, decltype(dh)::value>(a, s); });
+    else for_head_dim(hd, [&](auto dh) { launch_bwd<T, T, decltype(dh)::value>(a, s); });
 }
 
 }  // namespace tp

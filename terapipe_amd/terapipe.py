@@ -82,7 +82,8 @@ class _StackBuffers:
         nl, E, F, H = layers.n_layers, layers.embedding_dim, layers.ffn_embedding_dim, layers.num_attention_heads
         L, Dh = runner.seq_len, layers.embedding_dim // layers.num_attention_heads
         self.dtype, self.device = dtype, device
-        self.position_indexed = runner.suffix_dkdv and dtype != torch.float32     # the one-pass kernel is 16-bit
+        # the one-pass dK/dV kernel is 16-bit and has head dimensions 64 and 128; other runs keep gradient caches
+        self.position_indexed = runner.suffix_dkdv and dtype != torch.float32 and Dh in (64, 128)
         self.fused_attn_bwd = runner.fused_attn_bwd
         gdt = torch.float32 if runner.fp32_grad_cache else dtype
         kw = dict(dtype=dtype, device=device)

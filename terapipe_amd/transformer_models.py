@@ -4,7 +4,7 @@ with the arithmetic done by the HIP kernels of libterapipe_hip.so.
 
 Differences that are deliberate: no ``mpu`` / ``torch.distributed`` process group is needed (tensor-
 parallel size is 1, mpu/mappings.py:26-28 of the reference makes every collective an identity there);
-head dimension must be 64 or 128; the K/V caches are written by the QKV GEMM's epilogue rather than by
+the head dimension is one of 16, 32, 64, 80, 96, 128 (every entry of MODEL_CONFIGS); the K/V caches are written by the QKV GEMM's epilogue rather than by
 a separate _AssignCache op, with the same in-place, alias-returning semantics and the same gradient
 contract (reference transformer_models.py:177-193).
 """

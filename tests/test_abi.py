@@ -78,11 +78,33 @@ def test_argument_errors_without_gpu(lib):
     assert lib.tp_gemm(ctypes.byref(d), None, 0, None) == 2          # TP_ERR_UNSUPPORTED
     assert lib.tp_gemm_workspace_bytes(ctypes.byref(d)) == 0
     a = _lib.AttnDesc()
-    a.head_dim = 96
+    a.head_dim = 72
     assert lib.tp_attn_prefix_fwd(ctypes.byref(a), None, 0, None) != 0
     assert b"head_dim" in lib.tp_last_error()
     assert lib.tp_layernorm_fwd(None, None, None, None, None, None, 4, 64, 1e-5, 0, None) == 1
     assert lib.tp_zero_words(None, 4, None) == 1
+
+
+def test_every_head_dimension_of_the_model_table_is_accepted(lib):
+    """The attention entry points take the head dimension of every entry of MODEL_CONFIGS (reference
+    transformer_models.py:17-59): a descriptor that is otherwise empty gets past the head-dimension check and is
+    refused for its geometry instead."""
+    from terapipe_amd import _lib, transformer_models as tm
+    dims = sorted({e // h for (_, e, _, h) in tm.MODEL_CONFIGS.values()})
+    assert dims == [16, 64, 80, 96, 128]
+    for hd in dims + [32]:
+        a = _lib.AttnDesc()
+        a.head_dim = hd
+        assert lib.tp_attn_prefix_fwd(ctypes.byref(a), None, 0, None) == 1      # TP_ERR_ARG
+        assert b"geometry" in lib.tp_last_error()
+    for hd in (8, 48, 72, 112, 256):
+        a = _lib.AttnDesc()
+        a.head_dim = hd
+        assert lib.tp_attn_prefix_bwd(ctypes.byref(a), None, 0, None) == 2      # TP_ERR_UNSUPPORTED
+    s = _lib.AttnSuffixDesc()
+    s.dtype, s.head_dim = _lib.TP_F16, 96
+    assert lib.tp_attn_suffix_dkdv(ctypes.byref(s), None) == 2                  # the one-pass kernel: 64 and 128 only
+    assert b"head_dim" in lib.tp_last_error()
 
 
 def test_failed_replayed_launch_raises_the_library_error():

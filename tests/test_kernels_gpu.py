@@ -337,7 +337,8 @@ def test_gemm_epilogues(dtype, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
-@pytest.mark.parametrize("T,B,H,Dh,P,L", [(16, 2, 4, 64, 32, 128), (32, 1, 2, 128, 0, 64), (5, 3, 2, 64, 3, 16)])
+@pytest.mark.parametrize("T,B,H,Dh,P,L", [(16, 2, 4, 64, 32, 128), (32, 1, 2, 128, 0, 64), (5, 3, 2, 64, 3, 16),
+                                           (16, 2, 4, 80, 32, 128), (40, 1, 3, 96, 7, 64), (24, 2, 5, 16, 9, 40)])
 def test_gemm_qkv_scatter(dtype, T, B, H, Dh, P, L):
     ops = _ops()
     from terapipe_amd import _lib as Lb
@@ -381,6 +382,19 @@ ATTN_CASES = [
     (32, 2, 48, 128, 2016, 2048),  # BASELINE config 5's last slice: 96 (batch, head) pairs, 32 queries, 2048 keys
     (128, 1, 96, 128, 1920, 2048), # config 4's last slice
     (160, 1, 40, 128, 1888, 2048), # config 3's last slice
+    # head dimensions other than 64 and 128 (the reference's model table has 80, 96 and 16, transformer_models.py:33-49):
+    # the register-staged kernels with the head dimension padded to whole 32-column blocks in LDS, in every dtype
+    (16, 2, 4, 80, 112, 128),
+    (64, 1, 2, 96, 0, 64),         # no prefix: also pinned against SDPA
+    (32, 2, 3, 80, 480, 512),      # split over keys, merged
+    (128, 1, 4, 96, 896, 1024),
+    (160, 1, 2, 96, 100, 300),     # ragged
+    (7, 1, 1, 80, 5, 12),
+    (96, 2, 32, 80, 416, 512),     # 64 (batch, head) pairs, several query blocks
+    (16, 2, 4, 16, 112, 128),      # head dimension 16: gpt3-175b-megatron's 6144 / 384 (transformer_models.py:49)
+    (100, 1, 5, 16, 300, 512),
+    (40, 1, 3, 32, 7, 64),
+    (128, 2, 2, 32, 896, 1024),
 ]
 
 
@@ -717,9 +731,9 @@ def test_error_paths():
     w = torch.zeros(20, dtype=torch.float16, device=DEV)
     with pytest.raises(L.TeraPipeHipError):
         ops.layernorm_fwd(x, w, w)
-    q = torch.zeros(2, 4, 96, dtype=torch.float16, device=DEV)  # head_dim 96 unsupported
-    kc = torch.zeros(2, 8, 96, dtype=torch.float16, device=DEV)
-    with pytest.raises(L.TeraPipeHipError):
-        ops.attn_prefix_fwd(q, kc, kc, 1, 2, 96, 4, 0, 1.0)
+    q = torch.zeros(2, 4, 72, dtype=torch.float16, device=DEV)  # head_dim 72 unsupported
+    kc = torch.zeros(2, 8, 72, dtype=torch.float16, device=DEV)
+    with pytest.raises(L.TeraPipeHipError, match="head_dim"):
+        ops.attn_prefix_fwd(q, kc, kc, 1, 2, 72, 4, 0, 1.0)
     with pytest.raises(L.TeraPipeHipError):
         ops.layernorm_fwd(torch.zeros(4, 64), torch.zeros(64), torch.zeros(64))  # CPU tensors

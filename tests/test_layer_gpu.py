@@ -428,6 +428,35 @@ def test_terapipe_16bit_reduced_shapes(dtype, case):
         _check_param_grads(_param_grads(layers), go, dtype, tag)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("Dh", [16, 32, 80, 96])
+def test_terapipe_other_head_dims(dtype, Dh):
+    """Head dimensions of the reference's model table other than 64 and 128 (transformer_models.py:33-49: 96 for
+    megatron-* and gpt3-7hm, 80 for gpt3-2b, 16 for gpt3-175b-megatron), and 32: the runner keeps gradient caches
+    there, whatever suffix_dkdv says, and matches the oracle like the other widths."""
+    ta = _mods()
+    H = 3
+    E, Fd = H * Dh, 4 * H * Dh
+    n_layers, L, B, bs, ss = 2, 320, 2, [1, 1], [96, 64, 32, 80, 48]
+    ps = make_params(n_layers, E, Fd, dtype, seed=4, rand_small=True)
+    g = torch.Generator().manual_seed(23)
+    x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps)
+    for kw in (dict(), dict(fp32_grad_cache=False)):
+        runner, y, dx = _run_terapipe(ta, layers, x, dy, B, L, bs, ss, keep_states=True, **kw)
+        masks = None if dtype == torch.float32 else _relu_masks_from_states(runner.last_states)
+        leaf = [{k: v.clone().requires_grad_(True) for k, v in p.items()} for p in ps]
+        yo, dxo, fco = oracle.terapipe_forward_backward(leaf, x.float(), dy.float(), H, bs, ss, relu_masks=masks)
+        go = [{k: v.grad for k, v in p.items()} for p in leaf]
+        tag = "Dh=%d %s" % (Dh, kw)
+        assert_close(y, yo, dtype, tag + " y")
+        assert_close(dx, dxo, dtype, tag + " dx")
+        for b in range(len(bs)):
+            for j in range(2 * n_layers):
+                assert_close(runner.last_caches[b][j], fco[b][j], dtype, tag + " final cache")
+        _check_param_grads(_param_grads(layers), go, dtype, tag)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
 def test_slicing_invariance_full_width(dtype):
     """Size-independent property at a BASELINE width (hidden 2048, 16 heads, seq 2048): gradients with 8
