@@ -177,6 +177,26 @@ def test_host_side_surface_mirrors_reference_names():
         ta.TeraPipe(None, 2, 16, [2], [8, 4])                 # slices must sum to the sequence length
 
 
+def test_slicers_and_loss_on_cpu_tensors():
+    """uniform_slice_x, grid_slice_batch_and_sequence and loss_func are plain tensor code: checked on CPU tensors
+    against index arithmetic (reference transformer_models.py:368-377, :393-409, terapipe.py:48-49)."""
+    import terapipe_amd as ta
+    x = torch.arange(11 * 4 * 3, dtype=torch.float32).view(11, 4, 3)
+    parts = ta.uniform_slice_x(x, 4)                           # 11 = 3 + 3 + 3 + 2: the first 11 % 4 slices get one more
+    assert [p.size(0) for p in parts] == [3, 3, 3, 2] == ta.uniform_slice(11, 4)
+    assert torch.equal(torch.cat(parts), x)
+    assert parts[1].data_ptr() == x[3:].data_ptr()             # views, as in the reference
+    g = ta.grid_slice_batch_and_sequence(x, [1, 3], [5, 2, 4], requires_grad=True)
+    assert g.shape == (2, 3) and g.dtype == object
+    assert torch.equal(g[1, 2], x[7:11, 1:4]) and g[1, 2].is_contiguous() and g[1, 2].requires_grad and g[1, 2].is_leaf
+    assert torch.equal(g[0, 1], x[5:7, 0:1])
+    with pytest.raises(AssertionError):
+        ta.grid_slice_batch_and_sequence(x, [1, 3], [5, 2])    # slices must cover the sequence
+    with pytest.raises(AssertionError):
+        ta.grid_slice_batch_and_sequence(x, [1, 2], [5, 2, 4])
+    assert ta.loss_func(x).item() == pytest.approx(x.mean().item())
+
+
 def test_adam_table_validation_without_gpu(lib):
     from terapipe_amd import _lib
     t = (_lib.AdamTensor * 2)()
