@@ -190,6 +190,18 @@ __device__ __forceinline__ void tr_offsets(int krow0, int col0, int lane, int& o
     o0 = L::off(r0, col);
     o1 = L::off(r0 + (INTERLEAVED ? 8 : 4), col);
 }
+// the transposed fetch of a 16x16x32 operand: k-slot e of the lane's group q = lane >> 4 is row krow0 + 8 * q + e,
+// the lane's row / column of the block is col0 + (lane & 15)
+template <typename T, int COLS>
+__device__ __forceinline__ void tr_offsets16(int krow0, int col0, int lane, int& o0, int& o1) {
+    static_assert(sizeof(T) == 2, "16-bit tiles");
+    typedef TileLayout<T, COLS> L;
+    const int q = lane >> 4, p = lane & 15;
+    const int col = col0 + 4 * (p & 3);
+    const int r0 = krow0 + 8 * q + (p >> 2);
+    o0 = L::off(r0, col);
+    o1 = L::off(r0 + 4, col);
+}
 template <typename T> __device__ __forceinline__ uint4 load_km(const T* p) {
     return *reinterpret_cast<const uint4*>(p);
 }
@@ -377,6 +389,12 @@ template <typename T, int ROWS, int COLS, int NT, bool ALONG_COLS> struct ClampT
             dma16_saddr_lds(off[i], o, lds_bytes + (unsigned)((i * (NT / 64) + wave_uniform) * 512 * (int)sizeof(T)));
         origin += step;
     }
+    // the same, one load at a time (for loops that spread a tile's loads between other instructions): load i of
+    // the tile at `origin`; `advance` moves on to the next tile
+    __device__ __forceinline__ void issue_one(int i, unsigned lds_bytes, int wave_uniform) const {
+        dma16_saddr_lds(off[i], uniform_ptr(origin), lds_bytes + (unsigned)((i * (NT / 64) + wave_uniform) * 512 * (int)sizeof(T)));
+    }
+    __device__ __forceinline__ void advance() { origin += step; }
 };
 
 // error plumbing shared by the host-side entry points

@@ -24,6 +24,20 @@ struct GemmArgs {
     float* partial;  // [nsplit][M][N] fp32 when nsplit > 1
 };
 
+// v_mfma_f32_16x16x32: lane l feeds row / column (l & 15) with the 8 consecutive k values 8 * (l >> 4) .. + 7; the
+// 16x16 fp32 result leaves column (l & 15), rows 4 * (l >> 4) + r in register r.
+template <typename T> struct Mfma16x16x32;
+template <> struct Mfma16x16x32<f16> {
+    static __device__ __forceinline__ float4v run(uint4 a, uint4 b, float4v c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mfma16x16x32<bf16> {
+    static __device__ __forceinline__ float4v run(uint4 a, uint4 b, float4v c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+};
+
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
 __device__ __forceinline__ float gelu_erf_grad(float z) {
     float cdf = 0.5f * (1.0f + erff(z * 0.70710678118654752f));

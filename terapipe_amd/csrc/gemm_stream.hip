@@ -17,20 +17,6 @@
 
 namespace tp {
 
-template <typename T> struct Mfma16x16x32;
-template <> struct Mfma16x16x32<f16> {
-    static __device__ __forceinline__ float4v run(uint4 a, uint4 b, float4v c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
-    }
-};
-template <> struct Mfma16x16x32<bf16> {
-    static __device__ __forceinline__ float4v run(uint4 a, uint4 b, float4v c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-    }
-};
-
-// Operand layout of the 16x16x32 MFMA: lane l feeds row / column (l & 15) with the 8 consecutive k values
-// 8 * (l >> 4) .. + 7; the 16x16 fp32 result leaves column (l & 15), rows 4 * (l >> 4) + r in register r.
 template <typename T, bool BKM, int RB, int CB, int WN, int AS, int BS>
 __global__ __launch_bounds__(256 * WN) void gemm_stream_kernel(GemmArgs a) {
     static_assert(sizeof(T) == 2, "16-bit only");
