@@ -279,7 +279,10 @@ __device__ __forceinline__ void xcd_tile(int t, int tx, int ty, int& tile_x, int
     tile_y = band * 4 + within % hb;
 }
 
-template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN, int STAGES, bool GROUPED = false>
+// MI16: 16 x 16 x 32 MFMA blocks and ONE set of operand registers per wave (two waves share a SIMD: one computes
+// while the other fetches; two sets of the twice as many operand registers do not fit beside the accumulators).
+template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN, int STAGES, bool GROUPED = false,
+          bool MI16 = false>
 __global__ __launch_bounds__(WM * WN * 64)
 void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs>::type args) {
     // which problem and which of its tiles (wave-uniform)
@@ -308,7 +311,10 @@ void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     typedef Elem<T> E;
     static_assert(sizeof(T) == 2, "16-bit only");
     constexpr int NT = WM * WN * 64;
-    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int BLK = MI16 ? 16 : 32;                  // rows / columns of an MFMA block
+    constexpr int KS = MI16 ? 32 : E::KSTEP;             // k of one MFMA
+    static_assert(!MI16 || WM * WN == 8, "the 16 x 16 blocks are written for two waves per SIMD");
+    constexpr int TM = BM / WM / BLK, TN = BN / WN / BLK;
     constexpr int AR = AKM ? BM : BK, AC = AKM ? BK : BM;
     constexpr int BR = BKM ? BN : BK, BC = BKM ? BK : BN;
     constexpr int A_ELEMS = AR * AC, B_ELEMS = BR * BC;
@@ -340,36 +346,44 @@ void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
         db.issue(sA + (unsigned)(A_ELEMS * (int)sizeof(T)), wave_u);
     };
 
-    float16v acc[TM][TN];
+    typedef typename std::conditional<MI16, float4v, float16v>::type acc_t;
+    acc_t acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            for (int r = 0; r < (MI16 ? 4 : 16); ++r) acc[i][j][r] = 0.f;
 
-    constexpr int NKSTEP = BK / E::KSTEP;
+    constexpr int NKSTEP = BK / KS;
     constexpr int NPA = AKM ? 1 : 2, NPB = BKM ? 1 : 2;
     // lane's fetch offsets for k-step 0 of stage 0; k-steps and stages are compile-time byte offsets for
-    // k-major operands (a k-step is two chunks further along the row)
+    // k-major operands (a k-step is two (four) chunks further along the row)
     int oa[NKSTEP][TM][NPA], ob[NKSTEP][TN][NPB];
+    auto operand_offsets = [&](auto km_c, auto cols_c, int row0, int k0, int& o0, int& o1) {
+        constexpr bool KM = decltype(km_c)::value;
+        constexpr int COLS = decltype(cols_c)::value;
+        if constexpr (MI16) {
+            if constexpr (KM) o0 = o1 = TileLayout<T, COLS>::off(row0 + (lane & 15), k0 + 8 * (lane >> 4));
+            else tr_offsets16<T, COLS>(k0, row0, lane, o0, o1);
+        } else {
+            if constexpr (KM) o0 = o1 = km_offset<T, COLS>(row0 + (lane & 31), k0, lane);
+            else tr_offsets<T, COLS, false>(k0, row0, lane, o0, o1);
+        }
+    };
 #pragma unroll
     for (int ks = 0; ks < NKSTEP; ++ks) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int mb = (wm * TM + i) * 32;
-            if constexpr (AKM) oa[ks][i][0] = km_offset<T, AC>(mb + (lane & 31), ks * E::KSTEP, lane);
-            else tr_offsets<T, AC, false>(ks * E::KSTEP, mb, lane, oa[ks][i][0], oa[ks][i][NPA - 1]);
-        }
+        for (int i = 0; i < TM; ++i)
+            operand_offsets(std::integral_constant<bool, AKM>{}, std::integral_constant<int, AC>{}, (wm * TM + i) * BLK,
+                            ks * KS, oa[ks][i][0], oa[ks][i][NPA - 1]);
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const int nb = (wn * TN + j) * 32;
-            if constexpr (BKM) ob[ks][j][0] = A_ELEMS + km_offset<T, BC>(nb + (lane & 31), ks * E::KSTEP, lane);
-            else {
-                tr_offsets<T, BC, false>(ks * E::KSTEP, nb, lane, ob[ks][j][0], ob[ks][j][NPB - 1]);
-                ob[ks][j][0] += A_ELEMS;
-                ob[ks][j][NPB - 1] += A_ELEMS;
-            }
+            int o0, o1;
+            operand_offsets(std::integral_constant<bool, BKM>{}, std::integral_constant<int, BC>{}, (wn * TN + j) * BLK,
+                            ks * KS, o0, o1);
+            ob[ks][j][0] = A_ELEMS + o0;
+            ob[ks][j][NPB - 1] = A_ELEMS + o1;
         }
     }
 
@@ -378,7 +392,8 @@ void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     for (int s = 0; s < STAGES - 1; ++s)
         if (s < nk) issue(s);
 
-    typename E::opnd_t fa[2][TM], fb[2][TN];
+    constexpr int NSET = MI16 ? 1 : 2;
+    typename E::opnd_t fa[NSET][TM], fb[NSET][TN];
     auto fetch = [&](auto ksc, auto sc, int buf) {
         constexpr int ks = decltype(ksc)::value, s = decltype(sc)::value;
         const T* st = tiles + s * STAGE_ELEMS;
@@ -407,12 +422,21 @@ void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
         if (more) issue((s + STAGES - 1) % STAGES);   // issued while the fetch above is in flight
         auto step = [&](auto ksc) {
             constexpr int ks = decltype(ksc)::value;
-            if constexpr (ks + 1 < NKSTEP) fetch(std::integral_constant<int, ks + 1>{}, sc, (ks + 1) & 1);
+            constexpr int set = MI16 ? 0 : (ks & 1);
+            if constexpr (MI16) {
+                if constexpr (ks > 0) fetch(ksc, sc, 0);
+            } else if constexpr (ks + 1 < NKSTEP) {
+                fetch(std::integral_constant<int, ks + 1>{}, sc, (ks + 1) & 1);
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = E::mfma(fa[ks & 1][i], fb[ks & 1][j], acc[i][j]);
+                for (int j = 0; j < TN; ++j) {
+                    if constexpr (MI16) acc[i][j] = Mfma16x16x32<T>::run(fa[set][i], fb[set][j], acc[i][j]);
+                    else acc[i][j] = E::mfma(fa[set][i], fb[set][j], acc[i][j]);
+                }
+            if constexpr (MI16) __builtin_amdgcn_sched_barrier(0);
         };
         step(std::integral_constant<int, 0>{});
         if constexpr (NKSTEP > 1) step(std::integral_constant<int, 1>{});
@@ -431,7 +455,8 @@ void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
+    if constexpr (MI16) gemm_epilogue16<T, TM / 2, TN / 2, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
+    else gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -786,6 +811,7 @@ static bool tile_cfg(int id, TileCfg& c) {
     case 12: c = {64, 64, 128, 4}; return true;
     case 13: c = {128, 128, 64, 3}; return true;
     // gemm_tall_kernel: 256-row tiles
+    case 2: c = {256, 256, 32, 4}; return true;    // gemm_tall_kernel, 20 on 16 x 16 x 32 MFMA blocks
     // gemm_pipe_kernel: four waves, 16 x 16 x 32 MFMA blocks, software-pipelined k-loop
     case 14: c = {192, 128, 64, 3}; return true;   // 2 x 2 waves of 96 x 64
     case 15: c = {256, 128, 64, 3}; return true;   // 4 x 1 waves of 64 x 128
@@ -930,8 +956,9 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     } else if ((d->op == TP_GEMM_TN || d->M >= 512) && d->K % 64 == 0 && t256 >= 192) {
         // parameter gradients of a whole step, and any product of 512 rows or more with that many tiles (the LM
         // head): 256 x 256 tiles by eight waves (half the bytes per flop of a 128 x 128 tile through the
-        // 64 B/clk vector-memory path into LDS)
-        cfg = 19;
+        // 64 B/clk vector-memory path into LDS); the parameter gradients on 16 x 16 x 32 blocks with the 32-wide
+        // k-tile in four stages (timed inside steps of four geometries: 1 to 5 % under the 32 x 32 blocks)
+        cfg = d->op == TP_GEMM_TN ? 2 : 19;
     } else if (d->op != TP_GEMM_TN && d->M >= 512 && d->K % 64 == 0 && t256 >= 48 && d->K >= 8192) {
         // the same tiles on a long k with too few of them for the chip (the LM head's data gradient, k =
         // vocabulary): k is split to about one workgroup per CU
@@ -965,7 +992,7 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     if (forced_split) ns = forced_split;
     // the tall tiles load whole k-tiles only, and the 160 / 192 wide ones exist for the k-major weight (NT)
     // (a token-major tile 160 or 192 wide has no XOR swizzle: the chunk index would leave the row)
-    if (cfg >= 14 && cfg <= 20 && (d->K % 64 || (cfg == 17 && d->op != TP_GEMM_NT) || (cfg == 14 && d->op == TP_GEMM_TN))) cfg = 5;
+    if (((cfg >= 14 && cfg <= 20) || cfg == 2) && (d->K % 64 || (cfg == 17 && d->op != TP_GEMM_NT) || (cfg == 14 && d->op == TP_GEMM_TN))) cfg = 5;
     // the streaming kernel: NT and NN only; tiles whose width is not a power of two need the k-major weight (NT)
     if (cfg >= kFirstStreamCfg && (d->op == TP_GEMM_TN || ((cfg == 24 || cfg == 25) && d->op != TP_GEMM_NT))) cfg = 5;
     p.cfg = cfg;
@@ -983,6 +1010,7 @@ static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
         gemm_kernel<T, AKM, BKM, 64, 64, 16, 2, 2><<<grid, 256, 0, s>>>(a);
     } else {
         switch (p.cfg) {
+        case 2: gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4, false, true><<<grid, 512, 0, s>>>(a); break;
         case 3: gemm_dma_kernel<T, AKM, BKM, 128, 256, 64, 2, 4, 3><<<grid, 512, 0, s>>>(a); break;
         case 5: gemm_dma_kernel<T, AKM, BKM, 128, 128, 64, 2, 2, 2><<<grid, 256, 0, s>>>(a); break;
         case 8: gemm_dma_kernel<T, AKM, BKM, 64, 64, 64, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
@@ -1135,7 +1163,7 @@ static int group_cfg(const tp_gemm_desc* descs, int n) {
         if ((double)d.M * d.N > (double)descs[big].M * descs[big].N) big = i;
     }
     const GemmPlan pb = plan_gemm(&descs[big]);
-    return ((pb.cfg == 15 || pb.cfg == 19 || pb.cfg == 20) && pb.nsplit == 1) ? pb.cfg : 0;
+    return ((pb.cfg == 2 || pb.cfg == 15 || pb.cfg == 19 || pb.cfg == 20) && pb.nsplit == 1) ? pb.cfg : 0;
 }
 
 template <typename T>
@@ -1159,7 +1187,8 @@ static void launch_group(const tp_gemm_desc* descs, int n, int cfg, hipStream_t 
     }
     for (int i = n; i < kGroupMax; ++i) { ga.g[i] = ga.g[0]; ga.first_tile[i] = tiles; ga.tiles_x[i] = 1; ga.tiles_y[i] = 1; }
     ga.n = n;
-    if (cfg == 15) gemm_pipe_kernel<T, AKM, BKM, 256, 128, 4, 1, 3, true><<<dim3(tiles), 256, 0, s>>>(ga);
+    if (cfg == 2) gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4, true, true><<<dim3(tiles), 512, 0, s>>>(ga);
+    else if (cfg == 15) gemm_pipe_kernel<T, AKM, BKM, 256, 128, 4, 1, 3, true><<<dim3(tiles), 256, 0, s>>>(ga);
     else if (cfg == 19) gemm_tall_kernel<T, AKM, BKM, 256, 256, 64, 4, 2, 2, true><<<dim3(tiles), 512, 0, s>>>(ga);
     else gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4, true><<<dim3(tiles), 512, 0, s>>>(ga);
 }

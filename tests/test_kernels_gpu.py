@@ -112,7 +112,7 @@ def test_gemm_nt_nn_tn(dtype, M, N, K):
         assert_close(W, 2 * ref, dtype, "TN accumulate")
 
 
-TILE_CFGS = [0, 3, 5, 8, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20] + list(range(21, 41))
+TILE_CFGS = [0, 2, 3, 5, 8, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20] + list(range(21, 41))
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
@@ -211,7 +211,7 @@ def test_gemm_grouped_single_launch_matches_member_by_member(dtype):
               (L.TP_GEMM_TN, rnd(192, 3000, 0.1), rnd(192, 4504), 3000, 4504, 192)]
     for tag, items in (("layer", layer), ("ragged", ragged)):
         cfg = _group_cfg(L, items, dtype)
-        assert cfg in (19, 20), "%s: the group should run as one launch (got %d)" % (tag, cfg)
+        assert cfg in (2, 19, 20), "%s: the group should run as one launch (got %d)" % (tag, cfg)
         got, want = _group(ops, L, items, dtype, force_cfg=cfg)
         for i, (a, b) in enumerate(zip(got, want)):
             assert torch.equal(a, b), "%s member %d differs from the product launched alone" % (tag, i)
@@ -246,7 +246,7 @@ def test_gemm_grouped_falls_back_member_by_member():
     # accumulate epilogue through the grouped launch: C += product
     items = [(L.TP_GEMM_TN, rnd(128, 4096, 0.1), rnd(128, 4096), 4096, 4096, 128),
              (L.TP_GEMM_TN, rnd(128, 512, 0.1), rnd(128, 768), 512, 768, 128)]
-    assert _group_cfg(L, items, dtype) in (19, 20)
+    assert _group_cfg(L, items, dtype) in (2, 19, 20)
     Cs = [torch.ones(M, N, dtype=dtype, device=DEV) for (_, _, _, M, N, K) in items]
     ops.gemm_grouped([(op, A, B, M, N, K, C, L.TP_EPI_ACCUMULATE) for (op, A, B, M, N, K), C in zip(items, Cs)])
     for (op, A, B, M, N, K), C in zip(items, Cs):
