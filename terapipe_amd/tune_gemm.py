@@ -155,7 +155,7 @@ def shapes_of(geometry):
     return out
 
 
-def in_step(spec, dtype=torch.float16, log=sys.stderr):
+def in_step(spec, dtype=torch.float16, log=sys.stderr, only_rows=None):
     """Coordinate descent over the plans of the slice GEMMs (NT forward, NN data gradient) of one geometry,
     timing whole steps.  Returns [(op, M, N, K, cfg, nsplit)] for the shapes whose plan changed."""
     import time
@@ -197,7 +197,8 @@ def in_step(spec, dtype=torch.float16, log=sys.stderr):
     shapes = []
     for N, K in ((3 * E, E), (E, E), (F, E), (E, F)):
         for M in sorted({t * B for t in slices}):
-            shapes += [("NT", M, N, K), ("NN", M, K, N)]
+            if only_rows is None or M in only_rows:
+                shapes += [("NT", M, N, K), ("NN", M, K, N)]
     chosen = {}
     for op, M, N, K in shapes:
         key = (OPS[op], M, N, K)
@@ -238,6 +239,9 @@ def main():
     ap.add_argument("--in-step", metavar="SPEC",
                     help="hidden:ffn:heads:layers:batch:slice_tokens,... -- search the slice GEMM plans by timing "
                          "whole steps; prints the table entries to change")
+    ap.add_argument("--only-rows", metavar="M,M,...",
+                    help="with --in-step: search only the slice GEMMs of these row counts (a whole geometry can take "
+                         "longer than one sitting)")
     ap.add_argument("--pair", action="store_true",
                     help="time two concurrent chains of each GEMM on two streams (per-call time with a neighbour) "
                          "instead of one chain alone")
@@ -247,7 +251,8 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("tune_gemm: needs the GPU")
     if args.in_step:
-        for op, M, N, K, cfg, ns, ms in in_step(args.in_step):
+        rows = {int(v) for v in args.only_rows.split(",")} if args.only_rows else None
+        for op, M, N, K, cfg, ns, ms in in_step(args.in_step, only_rows=rows):
             print("{TP_GEMM_%s, %d, %d, %d, %d, %d},  // in-step search: step %.2f ms" % (op, M, N, K, cfg, ns, ms))
         return
     device = torch.device("cuda:0")
