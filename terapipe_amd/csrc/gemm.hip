@@ -23,10 +23,12 @@ struct GemmGroupArgs {
 // through its own LDS staging block so that a lane ends up with 8 consecutive columns of a row: 16-byte
 // stores and a vector epilogue.  Lane -> (row = lane / 4 + 16 * pass, columns 8 * (lane % 4) .. + 7).
 // `stage_base` must hold 32 * 36 floats per wave and must no longer be read as tile data by any wave.
-// `write_block(ic, jc, stage)` puts the wave's 32x32 block (ic, jc) into `stage` (row pitch 36 floats).
-template <typename T, int TM, int TN, int WM, int WN, typename WriteBlock>
+// `write_block(ic, jc, stage)` puts the wave's 32x32 block (ic, jc) into `stage` (row pitch 36 floats).  A wave's tile
+// is WROWS x WCOLS (multiples of 16): its last block row / column may be half a block.
+template <typename T, int TM, int TN, int WM, int WN, int WROWS, int WCOLS, typename WriteBlock>
 __device__ __forceinline__ void gemm_epilogue_blocks(const GemmArgs& a, WriteBlock&& write_block, float* stage_base,
                                                      int m0, int n0) {
+    static_assert(WROWS <= TM * 32 && WROWS > TM * 32 - 32 && WCOLS <= TN * 32 && WCOLS > TN * 32 - 32, "block counts");
     constexpr int SPITCH = 36;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave % WM, wn = wave / WM;
@@ -34,7 +36,8 @@ __device__ __forceinline__ void gemm_epilogue_blocks(const GemmArgs& a, WriteBlo
     const int er = lane >> 2, ec = (lane & 3) * 8;
     static_for<TN>([&](auto jc) __attribute__((always_inline)) {
         constexpr int j = decltype(jc)::value;
-        const int col0 = n0 + (wn * TN + j) * 32 + ec;
+        const int col0 = n0 + wn * WCOLS + j * 32 + ec;
+        const bool col_in = (j + 1) * 32 <= WCOLS || ec < WCOLS - j * 32;      // compile-time true for whole blocks
         float csum[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) csum[e] = 0.f;
@@ -47,13 +50,14 @@ __device__ __forceinline__ void gemm_epilogue_blocks(const GemmArgs& a, WriteBlo
 #pragma unroll
             for (int pass = 0; pass < 2; ++pass) {
                 const int rr = er + 16 * pass;
-                const int row = m0 + (wm * TM + i) * 32 + rr;
+                const int row = m0 + wm * WROWS + i * 32 + rr;
+                const bool row_in = (i + 1) * 32 <= WROWS || rr < WROWS - i * 32;
                 float v[8];
                 float4 v0 = *reinterpret_cast<const float4*>(stage + rr * SPITCH + ec);
                 float4 v1 = *reinterpret_cast<const float4*>(stage + rr * SPITCH + ec + 4);
                 v[0] = v0.x; v[1] = v0.y; v[2] = v0.z; v[3] = v0.w;
                 v[4] = v1.x; v[5] = v1.y; v[6] = v1.z; v[7] = v1.w;
-                if (row < a.M && col0 < a.N) {
+                if (row < a.M && col0 < a.N && row_in && col_in) {
                     if (a.nsplit > 1) {
                         float* dst = a.partial + ((long)blockIdx.z * a.M + row) * a.N + col0;
                         *reinterpret_cast<float4*>(dst) = v0;
@@ -67,7 +71,7 @@ __device__ __forceinline__ void gemm_epilogue_blocks(const GemmArgs& a, WriteBlo
             }
             __builtin_amdgcn_wave_barrier();
         });
-        if (a.nsplit == 1 && a.colsum) {
+        if (a.nsplit == 1 && a.colsum && col_in) {
             // lanes with equal (lane & 3) hold the same columns
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -91,28 +95,30 @@ template <typename T, int TM, int TN, int WM, int WN>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, float16v (&acc)[TM][TN], float* stage_base,
                                               int m0, int n0) {
     const int lane = threadIdx.x & 63, g = lane >> 5, li = lane & 31;
-    gemm_epilogue_blocks<T, TM, TN, WM, WN>(a, [&](auto ic, auto jc, float* stage) __attribute__((always_inline)) {
+    gemm_epilogue_blocks<T, TM, TN, WM, WN, TM * 32, TN * 32>(a, [&](auto ic, auto jc, float* stage) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
 #pragma unroll
         for (int r = 0; r < 16; ++r) stage[acc_row(r, g) * 36 + li] = acc[i][j][r];
     }, stage_base, m0, n0);
 }
 
-// accumulators of 16x16 MFMA blocks (TM, TN count 32x32 blocks: the array is [2 TM][2 TN]): register r of a block is
-// row 4 * (lane >> 4) + r, column lane & 15
+// accumulators of 16x16 MFMA blocks (TM x TN of them, either may be odd): register r of a block is row
+// 4 * (lane >> 4) + r, column lane & 15
 template <typename T, int TM, int TN, int WM, int WN>
-__device__ __forceinline__ void gemm_epilogue16(const GemmArgs& a, float4v (&acc)[2 * TM][2 * TN], float* stage_base,
+__device__ __forceinline__ void gemm_epilogue16(const GemmArgs& a, float4v (&acc)[TM][TN], float* stage_base,
                                                 int m0, int n0) {
     const int lane = threadIdx.x & 63, q = lane >> 4, c = lane & 15;
-    gemm_epilogue_blocks<T, TM, TN, WM, WN>(a, [&](auto ic, auto jc, float* stage) __attribute__((always_inline)) {
+    gemm_epilogue_blocks<T, (TM + 1) / 2, (TN + 1) / 2, WM, WN, TM * 16, TN * 16>(
+        a, [&](auto ic, auto jc, float* stage) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
-#pragma unroll
-        for (int di = 0; di < 2; ++di)
-#pragma unroll
-            for (int dj = 0; dj < 2; ++dj)
+        static_for<4>([&](auto dc) __attribute__((always_inline)) {
+            constexpr int di = decltype(dc)::value >> 1, dj = decltype(dc)::value & 1;
+            if constexpr (2 * i + di < TM && 2 * j + dj < TN) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
                     stage[(16 * di + 4 * q + r) * 36 + 16 * dj + c] = acc[2 * i + di][2 * j + dj][r];
+            }
+        });
     }, stage_base, m0, n0);
 }
 
@@ -455,7 +461,7 @@ void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if constexpr (MI16) gemm_epilogue16<T, TM / 2, TN / 2, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
+    if constexpr (MI16) gemm_epilogue16<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
     else gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
 }
 
@@ -501,7 +507,7 @@ void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     static_assert(WM * WN == 4, "one wave per SIMD");
     constexpr int NT = WM * WN * 64, BK = 64, KS = 32;
     constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
-    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "a wave's tile is whole 32 x 32 blocks");
+    static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "a wave's tile is whole 16 x 16 blocks");
     constexpr int NF = TM + TN, NM = TM * TN;
     constexpr int AR = AKM ? BM : BK, AC = AKM ? BK : BM;
     constexpr int BR = BKM ? BN : BK, BC = BKM ? BK : BN;
@@ -655,7 +661,7 @@ void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    gemm_epilogue16<T, TM / 2, TN / 2, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
+    gemm_epilogue16<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
 }
 
 template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN>
@@ -813,6 +819,8 @@ static bool tile_cfg(int id, TileCfg& c) {
     // gemm_tall_kernel: 256-row tiles
     case 2: c = {256, 256, 32, 4}; return true;    // gemm_tall_kernel, 20 on 16 x 16 x 32 MFMA blocks
     // gemm_pipe_kernel: four waves, 16 x 16 x 32 MFMA blocks, software-pipelined k-loop
+    case 6: c = {192, 160, 64, 3}; return true;    // 2 x 2 waves of 96 x 80 (NT only, like 7)
+    case 7: c = {160, 160, 64, 3}; return true;    // 2 x 2 waves of 80 x 80
     case 14: c = {192, 128, 64, 3}; return true;   // 2 x 2 waves of 96 x 64
     case 15: c = {256, 128, 64, 3}; return true;   // 4 x 1 waves of 64 x 128
     case 16: c = {128, 128, 64, 3}; return true;   // 2 x 2 waves of 64 x 64
@@ -992,6 +1000,7 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     if (forced_split) ns = forced_split;
     // the tall tiles load whole k-tiles only, and the 160 / 192 wide ones exist for the k-major weight (NT)
     // (a token-major tile 160 or 192 wide has no XOR swizzle: the chunk index would leave the row)
+    if ((cfg == 6 || cfg == 7) && (d->K % 64 || d->op != TP_GEMM_NT)) cfg = 5;
     if (((cfg >= 14 && cfg <= 20) || cfg == 2) && (d->K % 64 || (cfg == 17 && d->op != TP_GEMM_NT) || (cfg == 14 && d->op == TP_GEMM_TN))) cfg = 5;
     // the streaming kernel: NT and NN only; tiles whose width is not a power of two need the k-major weight (NT)
     if (cfg >= kFirstStreamCfg && (d->op == TP_GEMM_TN || ((cfg == 24 || cfg == 25) && d->op != TP_GEMM_NT))) cfg = 5;
@@ -1018,6 +1027,8 @@ static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
         case 10: gemm_dma_kernel<T, AKM, BKM, 128, 128, 32, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
         case 12: gemm_dma_kernel<T, AKM, BKM, 64, 64, 128, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
         case 13: gemm_dma_kernel<T, AKM, BKM, 128, 128, 64, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
+        case 6: if constexpr (AKM && BKM) gemm_pipe_kernel<T, AKM, BKM, 192, 160, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
+        case 7: if constexpr (AKM && BKM) gemm_pipe_kernel<T, AKM, BKM, 160, 160, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
         case 14: if constexpr (AKM) gemm_pipe_kernel<T, AKM, BKM, 192, 128, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
         case 15: gemm_pipe_kernel<T, AKM, BKM, 256, 128, 4, 1, 3><<<grid, 256, 0, s>>>(a); break;
         case 16: gemm_pipe_kernel<T, AKM, BKM, 128, 128, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;

@@ -31,7 +31,7 @@ DEFAULT_GEOMETRIES = [
     "12288:49152:128:2048",                                 # 175B shape, 128-token slices
     "6144:24576:64:4096",                                   # 44B shape, 32-token slices x batch 2
 ]
-DMA_CFGS = [2, 3, 5, 8, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20]
+DMA_CFGS = [2, 3, 5, 6, 7, 8, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20]
 # the weight-streaming kernel's configurations (NT and NN only; 24 and 25 NT only): cfg -> rows of its row tile
 STREAM_CFGS = {21: 192, 22: 256, 24: 192, 25: 256, 26: 128, 29: 256, 30: 192, 31: 192, 32: 256, 33: 192, 34: 256,
                35: 128, 36: 64, 37: 128, 38: 64}
@@ -126,7 +126,8 @@ def sweep(op, M, N, K, dtype, device, log, pair=False):
         for ns in SPLITS:
             if K // ns < 512 or (17 <= cfg <= 20 and (M < 192 or K % 64)) or (cfg == 17 and op != "NT"):
                 continue
-            if cfg in (2, 14, 15, 16) and (K % 64 or (cfg == 14 and op == "TN") or (cfg in (2, 14, 15) and M < 128)):
+            if cfg in (2, 6, 7, 14, 15, 16) and (K % 64 or (cfg == 14 and op == "TN") or (cfg in (6, 7) and op != "NT") or
+                                                 (cfg in (2, 6, 7, 14, 15) and M < 128)):
                 continue
             if cfg in STREAM_CFGS and ((cfg in (24, 25) and op != "NT") or STREAM_CFGS[cfg] < M // 2 or
                                        STREAM_CFGS[cfg] >= 2 * M):
@@ -207,7 +208,8 @@ def in_step(spec, dtype=torch.float16, log=sys.stderr, only_rows=None):
             for ns in (1, 2, 3, 4):
                 if K // ns < 512 or (cfg >= 17 and (M < 192 or K % 64)) or (cfg == 17 and op != "NT"):
                     continue
-                if cfg in (2, 14, 15, 16) and (K % 64 or (cfg in (2, 14, 15) and M < 128)):
+                if cfg in (2, 6, 7, 14, 15, 16) and (K % 64 or (cfg in (6, 7) and op != "NT") or
+                                                     (cfg in (2, 6, 7, 14, 15) and M < 128)):
                     continue
                 ops.GEMM_PLAN_OVERRIDE[key] = (cfg, ns)
                 try:

@@ -12,7 +12,7 @@ from terapipe_amd import _lib
 
 OPS = {"NT": _lib.TP_GEMM_NT, "NN": _lib.TP_GEMM_NN, "TN": _lib.TP_GEMM_TN}
 # tile configuration -> (rows, columns, workgroups that fit a CU)
-TILES = {0: (64, 64, 2), 2: (256, 256, 1), 3: (128, 256, 1), 5: (128, 128, 2), 8: (64, 64, 2), 10: (128, 128, 2), 11: (64, 256, 1),
+TILES = {0: (64, 64, 2), 2: (256, 256, 1), 6: (192, 160, 1), 7: (160, 160, 1), 3: (128, 256, 1), 5: (128, 128, 2), 8: (64, 64, 2), 10: (128, 128, 2), 11: (64, 256, 1),
          12: (64, 64, 2), 13: (128, 128, 1), 14: (192, 128, 1), 15: (256, 128, 1), 16: (128, 128, 1), 17: (256, 160, 1), 18: (256, 128, 1), 19: (256, 256, 1), 20: (256, 256, 1),
          31: (192, 128, 1), 33: (192, 256, 1)}
 
