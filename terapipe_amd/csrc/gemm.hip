@@ -992,6 +992,24 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
             if (ns > maxs) ns = maxs;
         }
     }
+    // The pipelined 16 x 16 x 32 tiles in place of the 32 x 32 ones the rules above name, where a sweep over other
+    // geometries (hidden 3072, 4096, 8192; 128 to 512 rows; 144 slice products) has them ahead: 128 x 128 for
+    // 128 x 128 (0.94 to 0.99 of the time), 192 x 128 for 128 x 256 at 129 to 192 rows and at 257 to 384 (0.83 to 0.91),
+    // 256 x 128 above 384 rows (0.92); a k-split stays within one round of workgroups of the new tile.
+    if (d->op != TP_GEMM_TN && d->K % 64 == 0 && (cfg == 13 || cfg == 3)) {
+        int bm = 128, bn = 128, to = 16;
+        if (cfg == 3) {
+            if ((d->M > 128 && d->M <= 192) || (d->M > 256 && d->M <= 384)) { to = 14; bm = 192; }
+            else if (d->M > 384) { to = 15; bm = 256; }
+            else to = 3;
+        }
+        if (to != 3) {
+            cfg = to;
+            const long tiles = (long)((d->M + bm - 1) / bm) * ((d->N + bn - 1) / bn);
+            const int cap = (int)(kNumCU / tiles);
+            if (ns > 1 && ns > cap) ns = cap < 1 ? 1 : cap;
+        }
+    }
     if (const TunedPlan* t = find_tuned(d)) { cfg = t->cfg; ns = t->nsplit; }
     if (ns < 1) ns = 1;
     if (ns > 16) ns = 16;

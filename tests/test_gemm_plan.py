@@ -84,12 +84,13 @@ def test_rule_examples():
     assert plan("NT", 64, 16384, 4096) == (8, 1)           # 256 tiles of 64 x 64
     assert plan("NN", 64, 4096, 16384) == (8, 4)           # 64 tiles, k split to 256 workgroups
     assert plan("NT", 128, 4096, 4096) == (12, 1)          # small weight: 64 x 64 x 128 tiles, unsplit
-    assert plan("NN", 128, 4096, 12288) == (13, 8)         # 32 tiles of 128 x 128
+    assert plan("NN", 128, 4096, 12288) == (16, 8)         # 32 tiles of 128 x 128 (the pipelined tile)
     assert plan("NT", 256, 32768, 8192) == (3, 1)          # 256 tiles of 128 x 256
     assert plan("NN", 256, 8192, 32768) == (3, 4)          # 64 of them on a long k
-    assert plan("NT", 256, 12288, 4096) == (13, 1)         # 192 tiles of 128 x 128, k too short to split
+    assert plan("NT", 256, 12288, 4096) == (16, 1)         # 192 tiles of 128 x 128, k too short to split
     assert plan("NT", 320, 30720, 10240) == (33, 1)        # two row tiles of 192: the weight-streaming kernel
     assert plan("NT", 512, 20480, 4096) == (19, 1)         # two rows of 256 x 256 tiles
-    assert plan("NN", 512, 4096, 16384) == (3, 4)
+    assert plan("NN", 512, 4096, 16384) == (15, 4)         # 2 x 32 pipelined tiles of 256 x 128 on a long k
+    assert plan("NT", 384, 16384, 4096) == (14, 1)         # two row tiles of 192 x 128
     # fp32 keeps its own plan (64 x 64 register-staged tiles)
     assert plan("NT", 128, 4096, 4096, _lib.TP_F32)[0] == 0
