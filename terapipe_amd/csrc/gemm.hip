@@ -652,7 +652,34 @@ void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
             substep(I1{}, No{}, sc, I0{}, No{}, sc);
         }
     };
-    for (int kt0 = 0; kt0 < nk; kt0 += STAGES) {
+    // a tile in the steady state: the next tile exists and the one STAGES ahead is loaded into this tile's buffer
+    auto tile_steady = [&](auto sc) __attribute__((always_inline)) {
+        constexpr int s = decltype(sc)::value, sn = (s + 1) % STAGES;
+        typedef std::integral_constant<int, 0> I0;
+        typedef std::integral_constant<int, 1> I1;
+        typedef std::integral_constant<bool, true> Yes;
+        typedef std::integral_constant<bool, false> No;
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_sched_barrier(0);
+        substep(I0{}, Yes{}, sc, I1{}, No{}, sc);
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        wait_vmcnt<NLOAD * (STAGES - 2)>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        substep(I1{}, Yes{}, std::integral_constant<int, sn>{}, I0{}, Yes{}, sc);
+        da.advance();
+        db.advance();
+    };
+    // one straight-line loop body of STAGES tiles while every one of them refills its buffer (no branches and no
+    // copies of accumulators between its tiles), then the last tiles one by one
+    int kt0 = 0;
+    for (; kt0 + 2 * STAGES <= nk; kt0 += STAGES) {
+        tile_steady(std::integral_constant<int, 0>{});
+        if constexpr (STAGES > 1) tile_steady(std::integral_constant<int, 1>{});
+        if constexpr (STAGES > 2) tile_steady(std::integral_constant<int, 2>{});
+    }
+    for (; kt0 < nk; kt0 += STAGES) {
         if (kt0 + 0 < nk) tile(std::integral_constant<int, 0>{}, kt0);
         if constexpr (STAGES > 1) { if (kt0 + 1 < nk) tile(std::integral_constant<int, 1>{}, kt0 + 1); }
         if constexpr (STAGES > 2) { if (kt0 + 2 < nk) tile(std::integral_constant<int, 2>{}, kt0 + 2); }
