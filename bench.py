@@ -281,7 +281,7 @@ def measure_workload(name, args, device, detail):
     bound_s = sum(max(f / peak, b / PEAK_HBM) for f, b in work)
     attainable = sum(f for f, _ in work) / bound_s
     roof = {
-        "kernel": "tp::gemm_dma_kernel / tp::gemm_tall_kernel / tp::gemm_stream_kernel (all NT/NN/TN launches of one step, "
+        "kernel": "tp::gemm_pipe_kernel / tp::gemm_tall_kernel / tp::gemm_dma_kernel / tp::gemm_stream_kernel (all NT/NN/TN launches of one step, "
                   "split-K reduce included)",
         "bound": "mfma", "achieved": achieved / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
         "frac": achieved / peak, "traffic": pmc_traffic(name),
