@@ -516,7 +516,7 @@ void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     typedef ClampTileDma<T, AR, AC, NT, AKM> DA;
     typedef ClampTileDma<T, BR, BC, NT, BKM> DB;
     constexpr int NLOAD = DA::N + DB::N;
-    static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
+    static_assert(NLOAD * STAGES <= 63, "too many loads in flight for vmcnt (every buffer has a tile under way)");
     constexpr int TILE_BYTES = STAGES * STAGE_ELEMS * 2;
     constexpr int EPI_BYTES = WM * WN * 32 * 36 * 4;
     constexpr int SMEM_BYTES = TILE_BYTES > EPI_BYTES ? TILE_BYTES : EPI_BYTES;
