@@ -240,13 +240,22 @@ def measure_workload(name, args, device, detail):
     for _ in range(warmup):
         one_step(layers, runner, x, R)
     torch.cuda.synchronize()
+    # an event behind every step (recorded without waiting): the spread of the steps, as the reference's loop prints
+    # mean and standard deviation (terapipe.py:290-315); the figure itself is the host clock around all K steps
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(steps):
+    marks[0].record()
+    for i in range(steps):
         one_step(layers, runner, x, R)
+        marks[i + 1].record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    per_step = [marks[i].elapsed_time(marks[i + 1]) for i in range(steps)]
+    mean = sum(per_step) / steps
     res = {"workload": "%s: %s" % (name, w["desc"]), "dtype": w["dtype"], "steps": steps, "warmup": warmup,
-           "ms_per_step": elapsed * 1e3 / steps, "tokens_per_s": w["L"] * w["B"] * steps / elapsed}
+           "ms_per_step": elapsed * 1e3 / steps, "tokens_per_s": w["L"] * w["B"] * steps / elapsed,
+           "ms_per_step_std": (sum((t - mean) ** 2 for t in per_step) / steps) ** 0.5,
+           "ms_per_step_min": min(per_step), "ms_per_step_max": max(per_step)}
     if args.no_roofline:
         return res, (layers, runner, x, R)
 
@@ -565,6 +574,8 @@ def main():
         "metric": "sliced-layer fwd+bwd tokens/s on 1 MI355X; % MFMA peak (GEMM), % HBM BW (attn)",
         "value": res["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step_std": res["ms_per_step_std"], "ms_per_step_min": res["ms_per_step_min"],
+        "ms_per_step_max": res["ms_per_step_max"],
         "dtype": w["dtype"], "data": "synthetic",
         "config": {"workload": res["workload"],
                    "loss": "sum(y * R), R ~ N(0,1) fixed", "optimizer_step": "outside the timed step (--optimizer times it separately)",
