@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libterapipe_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["misc.hip", "layernorm.hip", "gemm.hip", "gemm_stream.hip", "attention.hip", "vocab.hip", "planner.hip", "optimizer.hip"]
+SOURCES = ["misc.hip", "layernorm.hip", "gemm.hip", "gemm_pipe.hip", "gemm_stream.hip", "attention.hip", "vocab.hip", "planner.hip", "optimizer.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -34,7 +34,7 @@ def _stale(src_path, obj):
     """True unless obj is newer than its source and every header the sources share."""
     if not os.path.exists(obj):
         return True
-    deps = [src_path, os.path.join(CSRC, "common.h"), os.path.join(CSRC, "gemm_args.h"), os.path.join(CSRC, "gemm_tuned.inc"),
+    deps = [src_path, os.path.join(CSRC, "common.h"), os.path.join(CSRC, "gemm_args.h"), os.path.join(CSRC, "gemm_epilogue.h"), os.path.join(CSRC, "gemm_tuned.inc"),
             os.path.join(os.path.dirname(HERE), "include", "terapipe_hip.h")]
     t = os.path.getmtime(obj)
     return any(os.path.getmtime(d) > t for d in deps if os.path.exists(d))

@@ -2,125 +2,11 @@
 // size 1.  One templated kernel covers the three operand layouts and the three dtypes: an operand is
 // either "k-major" (k contiguous in memory: fetched from LDS with ds_read_b128) or "mn-major"
 // (k is the slow dimension: fetched with the gfx950 LDS transpose read), see common.h.
-#include "gemm_args.h"
+#include "gemm_epilogue.h"
 
 #include <mutex>
 
 namespace tp {
-
-// Several GEMMs of one tile configuration in one launch (unsplit k): workgroup w works on one of the
-// tiles_x[p] x tiles_y[p] tiles of problem p, the last p whose first_tile is <= w.
-constexpr int kGroupMax = 4;
-struct GemmGroupArgs {
-    GemmArgs g[kGroupMax];
-    int first_tile[kGroupMax];
-    int tiles_x[kGroupMax];
-    int tiles_y[kGroupMax];
-    int n;
-};
-
-// Epilogue shared by the GEMM kernels.  Each wave transposes one 32x32 accumulator block at a time
-// through its own LDS staging block so that a lane ends up with 8 consecutive columns of a row: 16-byte
-// stores and a vector epilogue.  Lane -> (row = lane / 4 + 16 * pass, columns 8 * (lane % 4) .. + 7).
-// `stage_base` must hold 32 * 36 floats per wave and must no longer be read as tile data by any wave.
-// `write_block(ic, jc, stage)` puts the wave's 32x32 block (ic, jc) into `stage` (row pitch 36 floats).  A wave's tile
-// is WROWS x WCOLS (multiples of 16): its last block row / column may be half a block.
-template <typename T, int TM, int TN, int WM, int WN, int WROWS, int WCOLS, typename WriteBlock>
-__device__ __forceinline__ void gemm_epilogue_blocks(const GemmArgs& a, WriteBlock&& write_block, float* stage_base,
-                                                     int m0, int n0) {
-    static_assert(WROWS <= TM * 32 && WROWS > TM * 32 - 32 && WCOLS <= TN * 32 && WCOLS > TN * 32 - 32, "block counts");
-    constexpr int SPITCH = 36;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave % WM, wn = wave / WM;
-    float* stage = stage_base + wave * 32 * SPITCH;
-    const int er = lane >> 2, ec = (lane & 3) * 8;
-    static_for<TN>([&](auto jc) __attribute__((always_inline)) {
-        constexpr int j = decltype(jc)::value;
-        const int col0 = n0 + wn * WCOLS + j * 32 + ec;
-        const bool col_in = (j + 1) * 32 <= WCOLS || ec < WCOLS - j * 32;      // compile-time true for whole blocks
-        float csum[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) csum[e] = 0.f;
-        static_for<TM>([&](auto ic) __attribute__((always_inline)) {
-            constexpr int i = decltype(ic)::value;
-            write_block(ic, jc, stage);
-            // the block is private to the wave: LDS operations of one wave complete in order
-            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int pass = 0; pass < 2; ++pass) {
-                const int rr = er + 16 * pass;
-                const int row = m0 + wm * WROWS + i * 32 + rr;
-                const bool row_in = (i + 1) * 32 <= WROWS || rr < WROWS - i * 32;
-                float v[8];
-                float4 v0 = *reinterpret_cast<const float4*>(stage + rr * SPITCH + ec);
-                float4 v1 = *reinterpret_cast<const float4*>(stage + rr * SPITCH + ec + 4);
-                v[0] = v0.x; v[1] = v0.y; v[2] = v0.z; v[3] = v0.w;
-                v[4] = v1.x; v[5] = v1.y; v[6] = v1.z; v[7] = v1.w;
-                if (row < a.M && col0 < a.N && row_in && col_in) {
-                    if (a.nsplit > 1) {
-                        float* dst = a.partial + ((long)blockIdx.z * a.M + row) * a.N + col0;
-                        *reinterpret_cast<float4*>(dst) = v0;
-                        *reinterpret_cast<float4*>(dst + 4) = v1;
-                    } else {
-                        epilogue_vec8<T>(a, row, col0, v);
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) csum[e] += v[e];
-                    }
-                }
-            }
-            __builtin_amdgcn_wave_barrier();
-        });
-        if (a.nsplit == 1 && a.colsum && col_in) {
-            // lanes with equal (lane & 3) hold the same columns
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float s = csum[e];
-                s += __shfl_xor(s, 4, 64);
-                s += __shfl_xor(s, 8, 64);
-                s += __shfl_xor(s, 16, 64);
-                s += __shfl_xor(s, 32, 64);
-                csum[e] = s;
-            }
-            if (lane < 4 && col0 < a.N) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) atomicAdd(a.colsum + col0 + e, csum[e]);
-            }
-        }
-    });
-}
-
-// accumulators of 32x32 MFMA blocks: register r of block (i, j) is row acc_row(r, lane >> 5), column lane & 31
-template <typename T, int TM, int TN, int WM, int WN>
-__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, float16v (&acc)[TM][TN], float* stage_base,
-                                              int m0, int n0) {
-    const int lane = threadIdx.x & 63, g = lane >> 5, li = lane & 31;
-    gemm_epilogue_blocks<T, TM, TN, WM, WN, TM * 32, TN * 32>(a, [&](auto ic, auto jc, float* stage) __attribute__((always_inline)) {
-        constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) stage[acc_row(r, g) * 36 + li] = acc[i][j][r];
-    }, stage_base, m0, n0);
-}
-
-// accumulators of 16x16 MFMA blocks (TM x TN of them, either may be odd): register r of a block is row
-// 4 * (lane >> 4) + r, column lane & 15
-template <typename T, int TM, int TN, int WM, int WN>
-__device__ __forceinline__ void gemm_epilogue16(const GemmArgs& a, float4v (&acc)[TM][TN], float* stage_base,
-                                                int m0, int n0) {
-    const int lane = threadIdx.x & 63, q = lane >> 4, c = lane & 15;
-    gemm_epilogue_blocks<T, (TM + 1) / 2, (TN + 1) / 2, WM, WN, TM * 16, TN * 16>(
-        a, [&](auto ic, auto jc, float* stage) __attribute__((always_inline)) {
-        constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
-        static_for<4>([&](auto dc) __attribute__((always_inline)) {
-            constexpr int di = decltype(dc)::value >> 1, dj = decltype(dc)::value & 1;
-            if constexpr (2 * i + di < TM && 2 * j + dj < TN) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    stage[(16 * di + 4 * q + r) * 36 + 16 * dj + c] = acc[2 * i + di][2 * j + dj][r];
-            }
-        });
-    }, stage_base, m0, n0);
-}
 
 // ---------------------------------------------------------------------------------------------
 // 16-bit kernel with direct global->LDS loads (global_load_lds_dwordx4) and a STAGES-deep ring of
@@ -268,23 +154,6 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_dma_kernel(GemmArgs a) {
 // the tile count can be matched to the 256 CUs (N = 20480: BN = 160 gives exactly 256 tiles for M = 512).
 // Tiles are loaded with ClampTileDma (whole k-tiles only) and the operand fetches of k-step s+1 are issued
 // before the MFMAs of k-step s.
-// ---------------------------------------------------------------------------------------------
-// Which tile of a tx x ty tile grid the t-th workgroup of a launch (or of a problem of a grouped launch) takes.
-// Workgroups go to the eight XCDs in turn, and each XCD has its own L2.  The tiles are laid out as a sequence
-// that sweeps bands of four tile rows column by column, and XCD slot j = t mod 8 takes the j-th eighth of that
-// sequence in order: the 32 tiles an XCD works on at a time form a 4 x 8 block that shares 12 operand slabs per
-// k-tile, whatever the tile grid's width (with tiles numbered row by row a grid eight tiles wide gives an XCD one
-// column: 33 slabs for 32 tiles).  A bijection of [0, tx * ty); every slot gets its share of the tiles to within one.
-__device__ __forceinline__ void xcd_tile(int t, int tx, int ty, int& tile_x, int& tile_y) {
-    const int n = tx * ty;
-    const int j = t & 7, q = n >> 3, r = n & 7;
-    const int seq = j * q + min(j, r) + (t >> 3);
-    const int band = seq / (4 * tx), within = seq - band * 4 * tx;
-    const int hb = min(4, ty - band * 4);
-    tile_x = within / hb;
-    tile_y = band * 4 + within % hb;
-}
-
 // MI16: 16 x 16 x 32 MFMA blocks and ONE set of operand registers per wave (two waves share a SIMD: one computes
 // while the other fetches; two sets of the twice as many operand registers do not fit beside the accumulators).
 template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN, int STAGES, bool GROUPED = false,
@@ -463,232 +332,6 @@ void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     asm volatile("" ::: "memory");
     if constexpr (MI16) gemm_epilogue16<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
     else gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
-}
-
-// ---------------------------------------------------------------------------------------------
-// Software-pipelined tall tile on 16 x 16 x 32 MFMA blocks, one wave per SIMD (four waves, accumulators in AGPRs).
-// A k-tile of 64 is two sub-steps of 32.  While the MFMAs of a sub-step run, the operand fragments of the NEXT
-// sub-step are fetched from LDS into the other register set, one fetch between every few MFMAs, front-loaded so
-// that they have landed when the sub-step ends; the workgroup barrier sits in the MIDDLE of a k-tile: by then
-// every wave has read the tile's second half into registers, so its buffer is free and the loads of the tile
-// STAGES ahead are issued into it, spread over the second sub-step's MFMAs, and the next tile (which the barrier
-// also proves landed) is fetched from during that sub-step.  No LDS or barrier latency stands between two MFMAs
-// of a wave except the barrier itself.
-// The blocks are 16 x 16 x 32 rather than 32 x 32 x 16: the same flops per cycle and, for a wave's tile, the same
-// operand bytes from LDS per flop, but on operands with random bits the chip sustains more of them -- a loop of
-// nothing but MFMAs runs at 2.0 against 1.6 PFLOP/s (2.4 for both on zeros).  They also cut a tile at 16 rows
-// (192 = 2 x 96 rows).  Measured on the 13B slice shapes: 4 to 12 % under the 32 x 32 tiles' times.
-// ---------------------------------------------------------------------------------------------
-template <typename T, bool AKM, bool BKM, int BM, int BN, int WM, int WN, int STAGES, bool GROUPED = false>
-__global__ __launch_bounds__(WM * WN * 64)
-void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs>::type args) {
-    int prob = 0, tile_x = blockIdx.x, tile_y = blockIdx.y;
-    if constexpr (GROUPED) {
-        static_assert(kGroupMax == 4, "the selects below are written out for four problems");
-        int first = 0, tx = args.tiles_x[0], ty = args.tiles_y[0];
-        if (1 < args.n && (int)blockIdx.x >= args.first_tile[1]) { prob = 1; first = args.first_tile[1]; tx = args.tiles_x[1]; ty = args.tiles_y[1]; }
-        if (2 < args.n && (int)blockIdx.x >= args.first_tile[2]) { prob = 2; first = args.first_tile[2]; tx = args.tiles_x[2]; ty = args.tiles_y[2]; }
-        if (3 < args.n && (int)blockIdx.x >= args.first_tile[3]) { prob = 3; first = args.first_tile[3]; tx = args.tiles_x[3]; ty = args.tiles_y[3]; }
-        xcd_tile((int)blockIdx.x - first, tx, ty, tile_x, tile_y);
-    } else if (gridDim.z == 1) {
-        xcd_tile((int)(blockIdx.y * gridDim.x + blockIdx.x), (int)gridDim.x, (int)gridDim.y, tile_x, tile_y);
-    }
-    const GemmArgs a = [&]() -> GemmArgs {
-        if constexpr (GROUPED) {
-            if (prob == 1) return args.g[1];
-            if (prob == 2) return args.g[2];
-            if (prob == 3) return args.g[3];
-            return args.g[0];
-        } else {
-            return args;
-        }
-    }();
-    static_assert(sizeof(T) == 2, "16-bit only");
-    static_assert(WM * WN == 4, "one wave per SIMD");
-    constexpr int NT = WM * WN * 64, BK = 64, KS = 32;
-    constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
-    static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0, "a wave's tile is whole 16 x 16 blocks");
-    constexpr int NF = TM + TN, NM = TM * TN;
-    constexpr int AR = AKM ? BM : BK, AC = AKM ? BK : BM;
-    constexpr int BR = BKM ? BN : BK, BC = BKM ? BK : BN;
-    constexpr int A_ELEMS = AR * AC, B_ELEMS = BR * BC;
-    constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
-    typedef ClampTileDma<T, AR, AC, NT, AKM> DA;
-    typedef ClampTileDma<T, BR, BC, NT, BKM> DB;
-    constexpr int NLOAD = DA::N + DB::N;
-    static_assert(NLOAD * STAGES <= 63, "too many loads in flight for vmcnt (every buffer has a tile under way)");
-    constexpr int TILE_BYTES = STAGES * STAGE_ELEMS * 2;
-    constexpr int EPI_BYTES = WM * WN * 32 * 36 * 4;
-    constexpr int SMEM_BYTES = TILE_BYTES > EPI_BYTES ? TILE_BYTES : EPI_BYTES;
-    static_assert(SMEM_BYTES <= 160 * 1024, "LDS");
-    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
-    T* tiles = reinterpret_cast<T*>(smem);
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave % WM, wn = wave / WM;
-    const int m0 = tile_y * BM, n0 = tile_x * BN;
-    const int kbeg = blockIdx.z * a.kper;
-    const int kend = min(a.K, kbeg + a.kper);
-    const int nk = (kend - kbeg) / BK;          // whole tiles only (the plan guarantees it)
-    DA da;
-    DB db;
-    da.init(reinterpret_cast<const T*>(a.A), a.lda, m0, a.M, kbeg, BK, tid);
-    db.init(reinterpret_cast<const T*>(a.B), a.ldb, n0, a.N, kbeg, BK, tid);
-    const unsigned lds0 = lds_addr(smem);
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-
-    float4v acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
-
-    constexpr int NPA = AKM ? 1 : 2, NPB = BKM ? 1 : 2;
-    int oa[2][TM][NPA], ob[2][TN][NPB];        // [sub-step][block][piece]: element offsets inside stage 0
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int mb = (wm * TM + i) * 16;
-            if constexpr (AKM) oa[ks][i][0] = TileLayout<T, AC>::off(mb + (lane & 15), ks * KS + 8 * (lane >> 4));
-            else tr_offsets16<T, AC>(ks * KS, mb, lane, oa[ks][i][0], oa[ks][i][NPA - 1]);
-        }
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int nb = (wn * TN + j) * 16;
-            if constexpr (BKM) ob[ks][j][0] = A_ELEMS + TileLayout<T, BC>::off(nb + (lane & 15), ks * KS + 8 * (lane >> 4));
-            else {
-                tr_offsets16<T, BC>(ks * KS, nb, lane, ob[ks][j][0], ob[ks][j][NPB - 1]);
-                ob[ks][j][0] += A_ELEMS;
-                ob[ks][j][NPB - 1] += A_ELEMS;
-            }
-        }
-    }
-
-    uint4 fa[2][TM], fb[2][TN];
-    // fetch number f of sub-step `sub` of the tile in stage s, into register set `set`
-    auto fetch_one = [&](auto fc, auto subc, auto sc, auto setc) __attribute__((always_inline)) {
-        constexpr int f = decltype(fc)::value, sub = decltype(subc)::value, s = decltype(sc)::value, set = decltype(setc)::value;
-        const T* st = tiles + s * STAGE_ELEMS;
-        if constexpr (f < TM) {
-            if constexpr (AKM) fa[set][f] = load_km<T>(st + oa[sub][f][0]);
-            else fa[set][f] = load_tr<T>(st + oa[sub][f][0], st + oa[sub][f][NPA - 1]);
-        } else {
-            constexpr int j = f - TM;
-            if constexpr (BKM) fb[set][j] = load_km<T>(st + ob[sub][j][0]);
-            else fb[set][j] = load_tr<T>(st + ob[sub][j][0], st + ob[sub][j][NPB - 1]);
-        }
-    };
-    // One sub-step: the NM MFMAs on register set SET, with the NF fetches of (stage FS, sub-step FSUB) into the
-    // other set after MFMAs 0, RF, 2 RF, ... (the first three quarters of the sub-step) and, if DMA, the NLOAD tile loads into
-    // stage DS after MFMAs at an even spacing.
-    auto substep = [&](auto setc, auto fetchc, auto fsc, auto fsubc, auto dmac, auto dsc) __attribute__((always_inline)) {
-        constexpr int set = decltype(setc)::value;
-        constexpr bool FETCH = decltype(fetchc)::value, DMA = decltype(dmac)::value;
-        constexpr int fs = decltype(fsc)::value, fsub = decltype(fsubc)::value, ds = decltype(dsc)::value;
-        constexpr int RF = (NM - NM / 4) / NF > 0 ? (NM - NM / 4) / NF : 1;
-        constexpr int RD = NM / NLOAD > 0 ? NM / NLOAD : 1;
-        const unsigned sA = lds0 + (unsigned)(ds * STAGE_ELEMS * 2);
-        static_for<NM>([&](auto mc) __attribute__((always_inline)) {
-            constexpr int m = decltype(mc)::value;
-            constexpr int i = m / TN, j = m % TN;
-            acc[i][j] = Mfma16x16x32<T>::run(fa[set][i], fb[set][j], acc[i][j]);
-            if constexpr (FETCH && m % RF == 0 && m / RF < NF)
-                fetch_one(std::integral_constant<int, m / RF>{}, fsubc, fsc, std::integral_constant<int, set ^ 1>{});
-            if constexpr (DMA && m % RD == RD - 1 && m / RD < NLOAD) {
-                constexpr int d = m / RD;
-                if constexpr (d < DA::N) da.issue_one(d, sA, wave_u);
-                else db.issue_one(d - DA::N, sA + (unsigned)(A_ELEMS * 2), wave_u);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        });
-        (void)fs; (void)fsub; (void)ds;
-    };
-
-    // prologue: every buffer gets a tile; tile 0 is waited for and its first sub-step fetched
-#pragma unroll
-    for (int s = 0; s < STAGES; ++s)
-        if (s < nk) {
-            const unsigned sA = lds0 + (unsigned)(s * STAGE_ELEMS * 2);
-            da.issue(sA, wave_u);
-            db.issue(sA + (unsigned)(A_ELEMS * 2), wave_u);
-        }
-    if (nk >= STAGES) wait_vmcnt<NLOAD * (STAGES - 1)>();
-    else wait_vmcnt<0>();
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    static_for<NF>([&](auto fc) __attribute__((always_inline)) {
-        fetch_one(fc, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
-    });
-
-    auto tile = [&](auto sc, int kt) __attribute__((always_inline)) {
-        constexpr int s = decltype(sc)::value, sn = (s + 1) % STAGES;
-        typedef std::integral_constant<int, 0> I0;
-        typedef std::integral_constant<int, 1> I1;
-        typedef std::integral_constant<bool, true> Yes;
-        typedef std::integral_constant<bool, false> No;
-        // first half: its operands were asked for during the previous sub-step
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        __builtin_amdgcn_sched_barrier(0);
-        substep(I0{}, Yes{}, sc, I1{}, No{}, sc);
-        // middle: this wave has read all of the tile; the next tile has landed once every wave says so
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        const bool next = kt + 1 < nk;               // uniform
-        const bool refill = kt + STAGES < nk;        // uniform
-        if (next) {
-            if (kt + STAGES - 1 < nk) wait_vmcnt<NLOAD * (STAGES - 2)>();
-            else wait_vmcnt<0>();
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (refill) {
-            substep(I1{}, Yes{}, std::integral_constant<int, sn>{}, I0{}, Yes{}, sc);
-            da.advance();
-            db.advance();
-        } else if (next) {
-            substep(I1{}, Yes{}, std::integral_constant<int, sn>{}, I0{}, No{}, sc);
-        } else {
-            substep(I1{}, No{}, sc, I0{}, No{}, sc);
-        }
-    };
-    // a tile in the steady state: the next tile exists and the one STAGES ahead is loaded into this tile's buffer
-    auto tile_steady = [&](auto sc) __attribute__((always_inline)) {
-        constexpr int s = decltype(sc)::value, sn = (s + 1) % STAGES;
-        typedef std::integral_constant<int, 0> I0;
-        typedef std::integral_constant<int, 1> I1;
-        typedef std::integral_constant<bool, true> Yes;
-        typedef std::integral_constant<bool, false> No;
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        __builtin_amdgcn_sched_barrier(0);
-        substep(I0{}, Yes{}, sc, I1{}, No{}, sc);
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        wait_vmcnt<NLOAD * (STAGES - 2)>();
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-        substep(I1{}, Yes{}, std::integral_constant<int, sn>{}, I0{}, Yes{}, sc);
-        da.advance();
-        db.advance();
-    };
-    // one straight-line loop body of STAGES tiles while every one of them refills its buffer (no branches and no
-    // copies of accumulators between its tiles), then the last tiles one by one
-    int kt0 = 0;
-    for (; kt0 + 2 * STAGES <= nk; kt0 += STAGES) {
-        tile_steady(std::integral_constant<int, 0>{});
-        if constexpr (STAGES > 1) tile_steady(std::integral_constant<int, 1>{});
-        if constexpr (STAGES > 2) tile_steady(std::integral_constant<int, 2>{});
-    }
-    for (; kt0 < nk; kt0 += STAGES) {
-        if (kt0 + 0 < nk) tile(std::integral_constant<int, 0>{}, kt0);
-        if constexpr (STAGES > 1) { if (kt0 + 1 < nk) tile(std::integral_constant<int, 1>{}, kt0 + 1); }
-        if constexpr (STAGES > 2) { if (kt0 + 2 < nk) tile(std::integral_constant<int, 2>{}, kt0 + 2); }
-        static_assert(STAGES <= 3, "at most three stages");
-    }
-    wait_vmcnt<0>();
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    gemm_epilogue16<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
 }
 
 template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN>
@@ -1057,6 +700,9 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     return p;
 }
 
+// the tile configurations of gemm_pipe.hip
+static inline bool is_pipe_cfg(int cfg) { return cfg == 6 || cfg == 7 || (cfg >= 14 && cfg <= 16); }
+
 template <typename T, bool AKM, bool BKM>
 static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
     dim3 grid(p.gx, p.gy, p.nsplit);
@@ -1072,11 +718,6 @@ static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
         case 10: gemm_dma_kernel<T, AKM, BKM, 128, 128, 32, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
         case 12: gemm_dma_kernel<T, AKM, BKM, 64, 64, 128, 2, 2, 4><<<grid, 256, 0, s>>>(a); break;
         case 13: gemm_dma_kernel<T, AKM, BKM, 128, 128, 64, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
-        case 6: if constexpr (AKM && BKM) gemm_pipe_kernel<T, AKM, BKM, 192, 160, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
-        case 7: if constexpr (AKM && BKM) gemm_pipe_kernel<T, AKM, BKM, 160, 160, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
-        case 14: if constexpr (AKM) gemm_pipe_kernel<T, AKM, BKM, 192, 128, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
-        case 15: gemm_pipe_kernel<T, AKM, BKM, 256, 128, 4, 1, 3><<<grid, 256, 0, s>>>(a); break;
-        case 16: gemm_pipe_kernel<T, AKM, BKM, 128, 128, 2, 2, 3><<<grid, 256, 0, s>>>(a); break;
         case 17: if constexpr (BKM) gemm_tall_kernel<T, AKM, BKM, 256, 160, 64, 4, 1, 3><<<grid, 256, 0, s>>>(a); break;
         case 18: gemm_tall_kernel<T, AKM, BKM, 256, 128, 64, 4, 1, 3><<<grid, 256, 0, s>>>(a); break;
         case 19: gemm_tall_kernel<T, AKM, BKM, 256, 256, 64, 4, 2, 2><<<grid, 512, 0, s>>>(a); break;
@@ -1090,6 +731,8 @@ template <typename T>
 static void launch_gemm(const tp_gemm_desc* d, const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
     if (p.cfg >= kFirstStreamCfg) {
         launch_gemm_stream(p.cfg, d->op, d->dtype, dim3(p.gx, p.gy, p.nsplit), a, s);
+    } else if (is_pipe_cfg(p.cfg) && d->dtype != TP_F32) {
+        launch_gemm_pipe(p.cfg, d->op, d->dtype, dim3(p.gx, p.gy, p.nsplit), a, s);
     } else {
         switch (d->op) {
         case TP_GEMM_NT: launch_cfg<T, true, true>(p, a, s); break;
@@ -1244,7 +887,7 @@ static void launch_group(const tp_gemm_desc* descs, int n, int cfg, hipStream_t 
     for (int i = n; i < kGroupMax; ++i) { ga.g[i] = ga.g[0]; ga.first_tile[i] = tiles; ga.tiles_x[i] = 1; ga.tiles_y[i] = 1; }
     ga.n = n;
     if (cfg == 2) gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4, true, true><<<dim3(tiles), 512, 0, s>>>(ga);
-    else if (cfg == 15) gemm_pipe_kernel<T, AKM, BKM, 256, 128, 4, 1, 3, true><<<dim3(tiles), 256, 0, s>>>(ga);
+    else if (cfg == 15) launch_gemm_pipe_group(cfg, descs[0].dtype, tiles, ga, s);
     else if (cfg == 19) gemm_tall_kernel<T, AKM, BKM, 256, 256, 64, 4, 2, 2, true><<<dim3(tiles), 512, 0, s>>>(ga);
     else gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4, true><<<dim3(tiles), 512, 0, s>>>(ga);
 }
