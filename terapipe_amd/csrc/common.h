@@ -69,11 +69,18 @@ __device__ __forceinline__ int acc_row(int j, int g) { return 8 * (j >> 2) + 4 *
 // the MFMA operand fetches are free of avoidable bank conflicts:
 //   (a) "k-major" fetch: 16 consecutive rows, the same 16-byte chunk (ds_read_b128), and
 //   (b) "transposed" fetch: ds_read_b64_tr_b16 over 4 consecutive rows x 64 bytes.
+// KM16 selects the mask for tiles whose only fetch is the k-major one of the 16x16x32 blocks (16 rows x 4
+// chunks a read): the LDS serves a ds_read_b128 in four groups of lanes that the masks of (a) and (b) leave
+// two-way conflicted for that shape (SQ_LDS_BANK_CONFLICT / SQ_LDS_IDX_ACTIVE 0.49 against 0.00 with these).
 // fp32 tiles are padded by 4 floats per row instead.
 // ---------------------------------------------------------------------------------------------
-template <int COLS> __device__ __forceinline__ int swz16(int row) {
+template <int COLS, bool KM16 = false> __device__ __forceinline__ int swz16(int row) {
     // returns the chunk XOR mask for a 16-bit tile with COLS elements per row
-    if constexpr (COLS >= 128) {
+    if constexpr (KM16 && COLS == 64) {
+        return (row >> 1) & 7;
+    } else if constexpr (KM16 && COLS == 32) {
+        return (row >> 1) & 3;
+    } else if constexpr (COLS >= 128) {
         return ((row & 3) << 2) | ((row >> 2) & 3);
     } else if constexpr (COLS == 64) {
         return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
@@ -84,13 +91,13 @@ template <int COLS> __device__ __forceinline__ int swz16(int row) {
     }
 }
 
-template <typename T, int COLS> struct TileLayout {
+template <typename T, int COLS, bool KM16 = false> struct TileLayout {
     static constexpr bool kSwz = (sizeof(T) == 2);
     static constexpr int LD = kSwz ? COLS : COLS + 4;   // row pitch in elements
     // element offset of (row, col); for swizzled tiles col's 8-element chunk index is permuted
     static __device__ __forceinline__ int off(int row, int col) {
         if constexpr (kSwz) {
-            return row * LD + ((((col >> 3) ^ swz16<COLS>(row)) << 3) | (col & 7));
+            return row * LD + ((((col >> 3) ^ swz16<COLS, KM16>(row)) << 3) | (col & 7));
         } else {
             return row * LD + col;
         }
@@ -354,7 +361,7 @@ __device__ __forceinline__ void dma4(const void* gptr, unsigned lds_wave_base) {
 // tile origin that advances by a scalar step, so a tile costs one VGPR per load and no vector ALU work.
 // Coordinates of the fixed axis beyond the matrix are CLAMPED to the last valid row / chunk (the caller never
 // stores results that depend on them); the sliding axis must be a whole number of tiles.
-template <typename T, int ROWS, int COLS, int NT, bool ALONG_COLS> struct ClampTileDma {
+template <typename T, int ROWS, int COLS, int NT, bool ALONG_COLS, bool KM16 = false> struct ClampTileDma {
     static constexpr int CPR = COLS / 8;
     static constexpr int TOTAL = ROWS * CPR;
     static constexpr int N = TOTAL / NT;
@@ -370,7 +377,7 @@ template <typename T, int ROWS, int COLS, int NT, bool ALONG_COLS> struct ClampT
         for (int i = 0; i < N; ++i) {
             const int p = (i * (NT / 64) + wave) * 64 + lane;
             const int row = p / CPR, pc = p % CPR;
-            const int lc = pc ^ swz16<COLS>(row);
+            const int lc = pc ^ swz16<COLS, KM16>(row);
             int fx = ALONG_COLS ? row : lc * 8;
             const int sl = ALONG_COLS ? lc * 8 : row;
             const int last = fixed_max - (ALONG_COLS ? 1 : 8) - fixed0;

@@ -194,8 +194,8 @@ void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     constexpr int BR = BKM ? BN : BK, BC = BKM ? BK : BN;
     constexpr int A_ELEMS = AR * AC, B_ELEMS = BR * BC;
     constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
-    typedef ClampTileDma<T, AR, AC, NT, AKM> DA;
-    typedef ClampTileDma<T, BR, BC, NT, BKM> DB;
+    typedef ClampTileDma<T, AR, AC, NT, AKM, MI16 && AKM> DA;
+    typedef ClampTileDma<T, BR, BC, NT, BKM, MI16 && BKM> DB;
     constexpr int NLOAD = DA::N + DB::N;
     static_assert(NLOAD * (STAGES - 1) <= 63, "too many loads in flight for vmcnt");
     constexpr int TILE_BYTES = STAGES * STAGE_ELEMS * 2;
@@ -239,7 +239,7 @@ void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
         constexpr bool KM = decltype(km_c)::value;
         constexpr int COLS = decltype(cols_c)::value;
         if constexpr (MI16) {
-            if constexpr (KM) o0 = o1 = TileLayout<T, COLS>::off(row0 + (lane & 15), k0 + 8 * (lane >> 4));
+            if constexpr (KM) o0 = o1 = TileLayout<T, COLS, true>::off(row0 + (lane & 15), k0 + 8 * (lane >> 4));
             else tr_offsets16<T, COLS>(k0, row0, lane, o0, o1);
         } else {
             if constexpr (KM) o0 = o1 = km_offset<T, COLS>(row0 + (lane & 31), k0, lane);

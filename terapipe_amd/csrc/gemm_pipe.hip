@@ -52,8 +52,8 @@ void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     constexpr int BR = BKM ? BN : BK, BC = BKM ? BK : BN;
     constexpr int A_ELEMS = AR * AC, B_ELEMS = BR * BC;
     constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
-    typedef ClampTileDma<T, AR, AC, NT, AKM> DA;
-    typedef ClampTileDma<T, BR, BC, NT, BKM> DB;
+    typedef ClampTileDma<T, AR, AC, NT, AKM, AKM> DA;
+    typedef ClampTileDma<T, BR, BC, NT, BKM, BKM> DB;
     constexpr int NLOAD = DA::N + DB::N;
     static_assert(NLOAD * STAGES <= 63, "too many loads in flight for vmcnt (every buffer has a tile under way)");
     constexpr int TILE_BYTES = STAGES * STAGE_ELEMS * 2;
@@ -89,13 +89,13 @@ void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int mb = (wm * TM + i) * 16;
-            if constexpr (AKM) oa[ks][i][0] = TileLayout<T, AC>::off(mb + (lane & 15), ks * KS + 8 * (lane >> 4));
+            if constexpr (AKM) oa[ks][i][0] = TileLayout<T, AC, true>::off(mb + (lane & 15), ks * KS + 8 * (lane >> 4));
             else tr_offsets16<T, AC>(ks * KS, mb, lane, oa[ks][i][0], oa[ks][i][NPA - 1]);
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const int nb = (wn * TN + j) * 16;
-            if constexpr (BKM) ob[ks][j][0] = A_ELEMS + TileLayout<T, BC>::off(nb + (lane & 15), ks * KS + 8 * (lane >> 4));
+            if constexpr (BKM) ob[ks][j][0] = A_ELEMS + TileLayout<T, BC, true>::off(nb + (lane & 15), ks * KS + 8 * (lane >> 4));
             else {
                 tr_offsets16<T, BC>(ks * KS, nb, lane, ob[ks][j][0], ob[ks][j][NPB - 1]);
                 ob[ks][j][0] += A_ELEMS;
