@@ -27,8 +27,8 @@ __global__ __launch_bounds__(256 * WN) void gemm_stream_kernel(GemmArgs a) {
     constexpr int CBW = CB / WN, BNW = 16 * CBW;
     constexpr int A_ELEMS = BM * BK, B_ELEMS = BN * BK;
     constexpr int BR = BKM ? BN : BK, BC = BKM ? BK : BN;
-    typedef ClampTileDma<T, BM, BK, NLA * 64, true> DA;
-    typedef ClampTileDma<T, BR, BC, (NW - NLA) * 64, BKM> DB;
+    typedef ClampTileDma<T, BM, BK, NLA * 64, true, true> DA;
+    typedef ClampTileDma<T, BR, BC, (NW - NLA) * 64, BKM, BKM> DB;
     constexpr int NA = DA::N, NB = DB::N;
     static_assert(NA * (AS - 1) <= 63 && NB * (BS - 1) <= 63, "too many loads in flight for vmcnt");
     constexpr int TILE_BYTES = (AS * A_ELEMS + BS * B_ELEMS) * 2;
@@ -66,11 +66,11 @@ __global__ __launch_bounds__(256 * WN) void gemm_stream_kernel(GemmArgs a) {
     const int r16 = lane & 15, g4 = lane >> 4;
     int oa[2];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) oa[ks] = TileLayout<T, BK>::off(wm * RB * 16 + r16, ks * 32 + 8 * g4);
+    for (int ks = 0; ks < 2; ++ks) oa[ks] = TileLayout<T, BK, true>::off(wm * RB * 16 + r16, ks * 32 + 8 * g4);
     int ob[BKM ? 2 : 2 * CBW];
     if constexpr (BKM) {
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) ob[ks] = TileLayout<T, BK>::off(wn * BNW + r16, ks * 32 + 8 * g4);
+        for (int ks = 0; ks < 2; ++ks) ob[ks] = TileLayout<T, BK, true>::off(wn * BNW + r16, ks * 32 + 8 * g4);
     } else {
         // k runs down the rows of the weight tile: two transpose reads per fragment, rows 8 * g4 + (p >> 2) and
         // four below, the 16 lanes of a group covering 4 rows x 16 columns
