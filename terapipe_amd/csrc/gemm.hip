@@ -143,7 +143,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_dma_kernel(GemmArgs a) {
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
+    gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0, (int)blockIdx.z);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -330,8 +330,8 @@ void gemm_tall_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if constexpr (MI16) gemm_epilogue16<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
-    else gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
+    if constexpr (MI16) gemm_epilogue16<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0, (int)blockIdx.z);
+    else gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0, (int)blockIdx.z);
 }
 
 template <typename T, bool AKM, bool BKM, int BM, int BN, int BK, int WM, int WN>
@@ -416,7 +416,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(GemmArgs a) {
         __syncthreads();
     }
 
-    gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
+    gemm_epilogue<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0, (int)blockIdx.z);
 }
 
 // Sums the split-K partials and applies the epilogue.  A block of 256 threads covers 256 columns

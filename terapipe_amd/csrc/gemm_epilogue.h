@@ -24,7 +24,7 @@ struct GemmGroupArgs {
 // is WROWS x WCOLS (multiples of 16): its last block row / column may be half a block.
 template <typename T, int TM, int TN, int WM, int WN, int WROWS, int WCOLS, typename WriteBlock>
 __device__ __forceinline__ void gemm_epilogue_blocks(const GemmArgs& a, WriteBlock&& write_block, float* stage_base,
-                                                     int m0, int n0) {
+                                                     int m0, int n0, int zsplit) {
     static_assert(WROWS <= TM * 32 && WROWS > TM * 32 - 32 && WCOLS <= TN * 32 && WCOLS > TN * 32 - 32, "block counts");
     constexpr int SPITCH = 36;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -56,7 +56,7 @@ __device__ __forceinline__ void gemm_epilogue_blocks(const GemmArgs& a, WriteBlo
                 v[4] = v1.x; v[5] = v1.y; v[6] = v1.z; v[7] = v1.w;
                 if (row < a.M && col0 < a.N && row_in && col_in) {
                     if (a.nsplit > 1) {
-                        float* dst = a.partial + ((long)blockIdx.z * a.M + row) * a.N + col0;
+                        float* dst = a.partial + ((long)zsplit * a.M + row) * a.N + col0;
                         *reinterpret_cast<float4*>(dst) = v0;
                         *reinterpret_cast<float4*>(dst + 4) = v1;
                     } else {
@@ -90,20 +90,20 @@ __device__ __forceinline__ void gemm_epilogue_blocks(const GemmArgs& a, WriteBlo
 // accumulators of 32x32 MFMA blocks: register r of block (i, j) is row acc_row(r, lane >> 5), column lane & 31
 template <typename T, int TM, int TN, int WM, int WN>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, float16v (&acc)[TM][TN], float* stage_base,
-                                              int m0, int n0) {
+                                              int m0, int n0, int zsplit) {
     const int lane = threadIdx.x & 63, g = lane >> 5, li = lane & 31;
     gemm_epilogue_blocks<T, TM, TN, WM, WN, TM * 32, TN * 32>(a, [&](auto ic, auto jc, float* stage) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
 #pragma unroll
         for (int r = 0; r < 16; ++r) stage[acc_row(r, g) * 36 + li] = acc[i][j][r];
-    }, stage_base, m0, n0);
+    }, stage_base, m0, n0, zsplit);
 }
 
 // accumulators of 16x16 MFMA blocks (TM x TN of them, either may be odd): register r of a block is row
 // 4 * (lane >> 4) + r, column lane & 15
 template <typename T, int TM, int TN, int WM, int WN>
 __device__ __forceinline__ void gemm_epilogue16(const GemmArgs& a, float4v (&acc)[TM][TN], float* stage_base,
-                                                int m0, int n0) {
+                                                int m0, int n0, int zsplit) {
     const int lane = threadIdx.x & 63, q = lane >> 4, c = lane & 15;
     gemm_epilogue_blocks<T, (TM + 1) / 2, (TN + 1) / 2, WM, WN, TM * 16, TN * 16>(
         a, [&](auto ic, auto jc, float* stage) __attribute__((always_inline)) {
@@ -116,7 +116,7 @@ __device__ __forceinline__ void gemm_epilogue16(const GemmArgs& a, float4v (&acc
                     stage[(16 * di + 4 * q + r) * 36 + 16 * dj + c] = acc[2 * i + di][2 * j + dj][r];
             }
         });
-    }, stage_base, m0, n0);
+    }, stage_base, m0, n0, zsplit);
 }
 
 // Which tile of a tx x ty tile grid the t-th workgroup of a launch (or of a problem of a grouped launch) takes.
@@ -130,6 +130,20 @@ __device__ __forceinline__ void xcd_tile(int t, int tx, int ty, int& tile_x, int
     const int j = t & 7, q = n >> 3, r = n & 7;
     const int seq = j * q + min(j, r) + (t >> 3);
     const int band = seq / (4 * tx), within = seq - band * 4 * tx;
+    const int hb = min(4, ty - band * 4);
+    tile_x = within / hb;
+    tile_y = band * 4 + within % hb;
+}
+// The same over a launch with k splits (grid = tx x ty x tz, workgroup t = (z * ty + y) * tx + x): the sequence
+// runs split by split, so an XCD's workgroups of a moment share one or two k ranges of the operands and its L2
+// holds those, instead of every XCD reading every k range of the row operand.
+__device__ __forceinline__ void xcd_tile3(int t, int tx, int ty, int tz, int& tile_x, int& tile_y, int& tile_z) {
+    const int plane = tx * ty, n = plane * tz;
+    const int j = t & 7, q = n >> 3, r = n & 7;
+    const int seq = j * q + min(j, r) + (t >> 3);
+    tile_z = seq / plane;
+    const int in_plane = seq - tile_z * plane;
+    const int band = in_plane / (4 * tx), within = in_plane - band * 4 * tx;
     const int hb = min(4, ty - band * 4);
     tile_x = within / hb;
     tile_y = band * 4 + within % hb;

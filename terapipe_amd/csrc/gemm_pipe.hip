@@ -21,7 +21,7 @@ namespace tp {
 template <typename T, bool AKM, bool BKM, int BM, int BN, int WM, int WN, int STAGES, bool GROUPED = false>
 __global__ __launch_bounds__(WM * WN * 64)
 void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs>::type args) {
-    int prob = 0, tile_x = blockIdx.x, tile_y = blockIdx.y;
+    int prob = 0, tile_x = blockIdx.x, tile_y = blockIdx.y, tile_z = blockIdx.z;
     if constexpr (GROUPED) {
         static_assert(kGroupMax == 4, "the selects below are written out for four problems");
         int first = 0, tx = args.tiles_x[0], ty = args.tiles_y[0];
@@ -31,6 +31,9 @@ void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
         xcd_tile((int)blockIdx.x - first, tx, ty, tile_x, tile_y);
     } else if (gridDim.z == 1) {
         xcd_tile((int)(blockIdx.y * gridDim.x + blockIdx.x), (int)gridDim.x, (int)gridDim.y, tile_x, tile_y);
+    } else {
+        xcd_tile3((int)((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x), (int)gridDim.x, (int)gridDim.y,
+                  (int)gridDim.z, tile_x, tile_y, tile_z);
     }
     const GemmArgs a = [&]() -> GemmArgs {
         if constexpr (GROUPED) {
@@ -66,7 +69,7 @@ void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave % WM, wn = wave / WM;
     const int m0 = tile_y * BM, n0 = tile_x * BN;
-    const int kbeg = blockIdx.z * a.kper;
+    const int kbeg = tile_z * a.kper;
     const int kend = min(a.K, kbeg + a.kper);
     const int nk = (kend - kbeg) / BK;          // whole tiles only (the plan guarantees it)
     DA da;
@@ -227,7 +230,7 @@ void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    gemm_epilogue16<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0);
+    gemm_epilogue16<T, TM, TN, WM, WN>(a, acc, reinterpret_cast<float*>(smem), m0, n0, tile_z);
 }
 
 template <typename T, bool AKM, bool BKM>
