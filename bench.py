@@ -303,7 +303,10 @@ def measure_workload(name, args, device, detail):
         "attainable": attainable / 1e12, "attainable_frac": attainable / peak,
         "achieved_over_attainable": achieved / attainable,
         "attainable_note": "per launch min(MFMA peak, (A + B + C bytes) / 8 TB/s), summed over the step's launches",
-        "method": "graph replay of the step's GEMM calls between two HIP events",
+        "method": "graph replay of the step's GEMM calls between two HIP events, one after the other on one stream: each "
+                  "launch has the chip to itself, with the tile and k splits the step uses (several of those were "
+                  "chosen by timing whole steps on the slice streams and are not the fastest alone; shared_chip times "
+                  "the same launches as the step overlaps them)",
     }
     if detail:
         groups = {}
