@@ -36,7 +36,7 @@ DMA_CFGS = [2, 3, 5, 6, 7, 8, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20]
 STREAM_CFGS = {21: 192, 22: 256, 24: 192, 25: 256, 26: 128, 29: 256, 30: 192, 31: 192, 32: 256, 33: 192, 34: 256,
                35: 128, 36: 64, 37: 128, 38: 64}
 SPLITS = [1, 2, 3, 4, 6, 8]
-# k splits the in-step search tries (whole 64-wide k-tiles per split only).  Inside a step the slice streams share the
+# k splits the in-step search tries (the library deals whole k-tiles to the splits, evenly to within one).  Inside a step the slice streams share the
 # chip, and fewer splits than are fastest for a launch alone often win: fewer, larger workgroups and fewer partial sums.
 IN_STEP_SPLITS = (1, 2, 3, 4, 5, 6, 8)
 OPS = {"NT": _lib.TP_GEMM_NT, "NN": _lib.TP_GEMM_NN, "TN": _lib.TP_GEMM_TN}
@@ -209,7 +209,7 @@ def in_step(spec, dtype=torch.float16, log=sys.stderr, only_rows=None):
         trials = []
         for cfg in DMA_CFGS:
             for ns in IN_STEP_SPLITS:
-                if K // ns < 512 or K % (64 * ns) or (cfg >= 17 and (M < 192 or K % 64)) or (cfg == 17 and op != "NT"):
+                if K // ns < 512 or (cfg >= 17 and (M < 192 or K % 64)) or (cfg == 17 and op != "NT"):
                     continue
                 if cfg in (2, 6, 7, 14, 15, 16) and (K % 64 or (cfg in (6, 7) and op != "NT") or
                                                      (cfg in (2, 6, 7, 14, 15) and M < 128)):
