@@ -173,8 +173,10 @@ int tp_gemm_group_cfg(const tp_gemm_desc* descs, int n);
  * result bits as tp_gemm with a caller workspace.  A product whose plan needs more than the array holds is
  * refused with TP_ERR_WORKSPACE (tp_gemm_workspace_bytes(d) > tp_gemm_static_ws_capacity()), defer_reduce with
  * TP_ERR_ARG.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two
- * threads) race on the partial sums; nothing in it needs to start at zero.  The first call on a device looks up
- * the array's address on that device (the device must be current, as for every launch). */
+ * threads) race on the partial sums; nothing in it needs to start at zero.  The array's address on a device is
+ * looked up once, by the first call of either function with that device current (a module and symbol lookup):
+ * a caller that captures tp_gemm_static_ws into a HIP graph calls tp_gemm_static_ws_capacity() on the device
+ * BEFORE the capture opens. */
 #define TP_GEMM_STATIC_WS_BYTES (64u << 20)
 size_t tp_gemm_static_ws_capacity(void);
 int tp_gemm_static_ws(const tp_gemm_desc* d, void* stream);

@@ -161,13 +161,16 @@ def attention_forward(p: Dict[str, torch.Tensor], prefix: str, x, num_heads: int
 
 
 def layer_forward(p: Dict[str, torch.Tensor], x, num_heads: int, full_cache=None,
-                  cache_len: int = 0, prefix: str = "", activation: str = "relu", relu_mask=None):
+                  cache_len: int = 0, prefix: str = "", activation: str = "relu", relu_mask=None,
+                  preact_sink: Optional[list] = None):
     """TransformerLayer.forward, transformer_models.py:273-285 (pre-LN block, ReLU MLP).
 
     relu_mask (optional bool tensor shaped like the fc1 output) replaces ``z > 0`` as the ReLU's
     active set: a 16-bit run decides the sign of near-zero pre-activations by its own rounding, and a
     parity test that wants to measure arithmetic error rather than those sign flips hands the mask of
-    the run under test to the oracle.  The reference path is relu_mask=None."""
+    the run under test to the oracle.  The reference path is relu_mask=None.
+    preact_sink (optional list) receives a detached copy of the fc1 output before the activation, so that a
+    test can check the active set it hands in against the sign of the oracle's own pre-activations."""
     y = x
     h = layer_norm(x, p[prefix + "attn_ln.weight"], p[prefix + "attn_ln.bias"])       # :275
     h, new_cache = attention_forward(p, prefix + "attn.", h, num_heads, full_cache, cache_len)
@@ -175,6 +178,8 @@ def layer_forward(p: Dict[str, torch.Tensor], x, num_heads: int, full_cache=None
     y = h
     z = layer_norm(h, p[prefix + "fc_ln.weight"], p[prefix + "fc_ln.bias"])           # :280
     z = linear_col(z, p[prefix + "fc1.weight"], p[prefix + "fc1.bias"])
+    if preact_sink is not None:
+        preact_sink.append(z.detach().clone())
     if activation == "relu":
         z = torch.relu(z) if relu_mask is None else z * relu_mask.to(z.dtype)        # :282
     else:
@@ -184,14 +189,16 @@ def layer_forward(p: Dict[str, torch.Tensor], x, num_heads: int, full_cache=None
 
 
 def stack_forward(params: List[Dict[str, torch.Tensor]], x, num_heads: int, cache, cache_len: int,
-                  activation: str = "relu", relu_masks=None):
+                  activation: str = "relu", relu_masks=None, preact_sink: Optional[list] = None):
     """TransformerLayers.forward, terapipe.py:79-86; cache is the flat list [k0, v0, k1, v1, ...].
-    relu_masks: optional list (one per layer) passed to layer_forward."""
+    relu_masks: optional list (one per layer) passed to layer_forward; preact_sink: optional list that
+    receives every layer's fc1 pre-activation in layer order."""
     cache_outputs = []
     for i, p in enumerate(params):
         x, (ko, vo) = layer_forward(p, x, num_heads, (cache[2 * i], cache[2 * i + 1]), cache_len,
                                     activation=activation,
-                                    relu_mask=None if relu_masks is None else relu_masks[i])
+                                    relu_mask=None if relu_masks is None else relu_masks[i],
+                                    preact_sink=preact_sink)
         cache_outputs += [ko, vo]
     return x, cache_outputs
 
@@ -275,7 +282,8 @@ def grid_slice_batch_and_sequence(x, batch_slices, seq_slices, requires_grad=Fal
 
 def terapipe_forward_backward(params: List[Dict[str, torch.Tensor]], x, dy, num_heads: int,
                               batch_slices: Sequence[int], seq_slices: Sequence[int],
-                              return_cache_grads: bool = False, activation: str = "relu", relu_masks=None):
+                              return_cache_grads: bool = False, activation: str = "relu", relu_masks=None,
+                              preacts: Optional[dict] = None):
     """TeraPipe.forward (terapipe.py:238-271) followed by TeraPipeBackwardPassHook.backward
     (terapipe.py:167-201) on a single pipeline stage.
 
@@ -283,7 +291,8 @@ def terapipe_forward_backward(params: List[Dict[str, torch.Tensor]], x, dy, num_
     exactly as in the reference (autograd sum).  Returns (y, dx, final_caches[, cache_grads]) where
     final_caches[b] is the flat K/V list after the last slice of batch slice b and cache_grads[b][i]
     is the list of .grad tensors of the cache inputs of slice i.  relu_masks, if given, maps
-    (batch slice, sequence slice) to the per-layer list of ReLU active sets (see layer_forward).
+    (batch slice, sequence slice) to the per-layer list of ReLU active sets (see layer_forward);
+    preacts, if given, is filled with (batch slice, sequence slice) -> per-layer fc1 pre-activations.
     """
     L = x.size(0)
     E = x.size(2)
@@ -301,8 +310,11 @@ def terapipe_forward_backward(params: List[Dict[str, torch.Tensor]], x, dy, num_
         for i in range(ns):
             xi = inputs[b, i]
             cache = [c.detach().requires_grad_() for c in cache]                          # :257
+            sink = None
+            if preacts is not None:
+                sink = preacts[(b, i)] = []
             y, cache_out = stack_forward(params, xi, num_heads, cache, cache_len, activation,      # :258
-                                         None if relu_masks is None else relu_masks[(b, i)])
+                                         None if relu_masks is None else relu_masks[(b, i)], sink)
             cache_inputs[b, i] = cache
             cache_outputs[b, i] = cache_out
             cache = cache_out

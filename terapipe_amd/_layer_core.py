@@ -154,6 +154,7 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
     suffix: None, or dict(q_all, d_o_all, lse_all, delta_all, q_end) of position-indexed buffers that hold
     every slice processed so far (buf.d_o and buf.delta are then views of them at this slice): dK/dV of
     the slice's keys are computed in one pass over all later query positions and gk / gv are not used.
+    With suffix["fused"] (needs o_all and own_end) dQ and that pass go out as one launch.
     Returns dx [T, B, E].
     """
     T, B = st.T, st.B
@@ -192,10 +193,12 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
                             st.cache_len, float(Dh) ** -0.5, accumulate_prefix, has_incoming, zero_slice_rows,
                             colsum_dqkv_acc=sa.get("attn.in_proj.bias"), delta=buf.delta,
                             q_bh_rows=st.q_bh_rows, stat_bh_rows=st.stat_bh_rows)
-    elif suffix.get("o_all") is not None and suffix["own_end"] - st.cache_len <= ops.FUSED_BWD_WINDOW:
+    elif suffix.get("fused"):
         # dQ of the slice and dK / dV of its keys over all later positions as one launch.  The dK/dV half takes delta
         # of the positions up to own_end itself, so what it needs of the later slices is their dO (and, past own_end,
-        # their delta): the slice waits for the next slice's event and records its own BEFORE the launch
+        # their delta): the slice waits for the next slice's event and records its own BEFORE the launch.  (An event
+        # recorded there does not cover this launch's delta: the caller may only mix fused and two-launch slices
+        # on ONE stream, see terapipe.fused_backward_slices.)
         if buf.sync is not None:
             buf.sync()
         ops.attn_bwd_fused(st.q, st.k_cache, st.v_cache, st.o, st.lse, d_o, dqkv, B, heads, Dh, T, st.cache_len,

@@ -690,8 +690,9 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     // (a token-major tile 160 or 192 wide has no XOR swizzle: the chunk index would leave the row)
     if ((cfg == 6 || cfg == 7) && (d->K % 64 || d->op != TP_GEMM_NT)) cfg = 5;
     if (((cfg >= 14 && cfg <= 20) || cfg == 2) && (d->K % 64 || (cfg == 17 && d->op != TP_GEMM_NT) || (cfg == 14 && d->op == TP_GEMM_TN))) cfg = 5;
-    // the streaming kernel: NT and NN only; tiles whose width is not a power of two need the k-major weight (NT)
-    if (cfg >= kFirstStreamCfg && (d->op == TP_GEMM_TN || ((cfg == 24 || cfg == 25) && d->op != TP_GEMM_NT))) cfg = 5;
+    // the streaming kernel: NT and NN only, whole 64-wide k-tiles only; tiles whose width is not a power of two need
+    // the k-major weight (NT)
+    if (cfg >= kFirstStreamCfg && (d->op == TP_GEMM_TN || d->K % 64 || ((cfg == 24 || cfg == 25) && d->op != TP_GEMM_NT))) cfg = 5;
     p.cfg = cfg;
     tile_cfg(cfg, tc);
     p.gx = (d->N + tc.bn - 1) / tc.bn;
@@ -727,12 +728,13 @@ static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
     }
 }
 
+// false: the plan names a (tile configuration, op, dtype) that no kernel is built for -- nothing was launched
 template <typename T>
-static void launch_gemm(const tp_gemm_desc* d, const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
+static bool launch_gemm(const tp_gemm_desc* d, const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
     if (p.cfg >= kFirstStreamCfg) {
-        launch_gemm_stream(p.cfg, d->op, d->dtype, dim3(p.gx, p.gy, p.nsplit), a, s);
+        if (!launch_gemm_stream(p.cfg, d->op, d->dtype, dim3(p.gx, p.gy, p.nsplit), a, s)) return false;
     } else if (is_pipe_cfg(p.cfg) && d->dtype != TP_F32) {
-        launch_gemm_pipe(p.cfg, d->op, d->dtype, dim3(p.gx, p.gy, p.nsplit), a, s);
+        if (!launch_gemm_pipe(p.cfg, d->op, d->dtype, dim3(p.gx, p.gy, p.nsplit), a, s)) return false;
     } else {
         switch (d->op) {
         case TP_GEMM_NT: launch_cfg<T, true, true>(p, a, s); break;
@@ -744,6 +746,7 @@ static void launch_gemm(const tp_gemm_desc* d, const GemmPlan& p, const GemmArgs
         dim3 grid((d->N + 255) / 256, (d->M + 31) / 32);
         gemm_splitk_reduce_kernel<T><<<grid, 256, 0, s>>>(a);
     }
+    return true;
 }
 
 static int validate_gemm(const tp_gemm_desc* d) {
@@ -866,7 +869,7 @@ static int group_cfg(const tp_gemm_desc* descs, int n) {
 }
 
 template <typename T>
-static void launch_group(const tp_gemm_desc* descs, int n, int cfg, hipStream_t s) {
+static bool launch_group(const tp_gemm_desc* descs, int n, int cfg, hipStream_t s) {
     constexpr bool AKM = false, BKM = false;     // TN: both operands token-major
     GemmGroupArgs ga;
     int tiles = 0;
@@ -887,9 +890,10 @@ static void launch_group(const tp_gemm_desc* descs, int n, int cfg, hipStream_t 
     for (int i = n; i < kGroupMax; ++i) { ga.g[i] = ga.g[0]; ga.first_tile[i] = tiles; ga.tiles_x[i] = 1; ga.tiles_y[i] = 1; }
     ga.n = n;
     if (cfg == 2) gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4, true, true><<<dim3(tiles), 512, 0, s>>>(ga);
-    else if (cfg == 15) launch_gemm_pipe_group(cfg, descs[0].dtype, tiles, ga, s);
+    else if (cfg == 15) return launch_gemm_pipe_group(cfg, descs[0].dtype, tiles, ga, s);
     else if (cfg == 19) gemm_tall_kernel<T, AKM, BKM, 256, 256, 64, 4, 2, 2, true><<<dim3(tiles), 512, 0, s>>>(ga);
     else gemm_tall_kernel<T, AKM, BKM, 256, 256, 32, 4, 2, 4, true><<<dim3(tiles), 512, 0, s>>>(ga);
+    return true;
 }
 }  // namespace tp
 
@@ -927,7 +931,13 @@ static void* scratch_on_current_device() {
 }
 }  // namespace tp
 
-extern "C" size_t tp_gemm_static_ws_capacity(void) { return (size_t)TP_GEMM_STATIC_WS_BYTES; }
+// Also looks up the array's address on the current device (a module and symbol lookup that must not happen while a
+// stream capture is open): callers that capture tp_gemm_static_ws call this once per device beforehand.
+extern "C" size_t tp_gemm_static_ws_capacity(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) == hipSuccess && n > 0) (void)tp::scratch_on_current_device();
+    return (size_t)TP_GEMM_STATIC_WS_BYTES;
+}
 
 extern "C" int tp_gemm_static_ws(const tp_gemm_desc* d, void* stream) {
     int rc = tp::validate_gemm(d);
@@ -963,10 +973,15 @@ extern "C" int tp_gemm(const tp_gemm_desc* d, void* workspace, size_t workspace_
     }
     tp::GemmArgs a = tp::fill_args(d, p, workspace);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    bool launched;
     switch (d->dtype) {
-    case TP_F32: tp::launch_gemm<float>(d, p, a, s); break;
-    case TP_F16: tp::launch_gemm<tp::f16>(d, p, a, s); break;
-    default: tp::launch_gemm<tp::bf16>(d, p, a, s); break;
+    case TP_F32: launched = tp::launch_gemm<float>(d, p, a, s); break;
+    case TP_F16: launched = tp::launch_gemm<tp::f16>(d, p, a, s); break;
+    default: launched = tp::launch_gemm<tp::bf16>(d, p, a, s); break;
+    }
+    if (!launched) {
+        tp::set_error("tp_gemm: no kernel for tile configuration %d with op %d, dtype %d", p.cfg, d->op, d->dtype);
+        return TP_ERR_UNSUPPORTED;
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { tp::set_error("tp_gemm: launch failed: %s", hipGetErrorString(e)); return TP_ERR_LAUNCH; }
@@ -988,8 +1003,12 @@ extern "C" int tp_gemm_grouped(const tp_gemm_desc* descs, int n, void* workspace
     }
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (const int cfg = tp::group_cfg(descs, n)) {
-        if (descs[0].dtype == TP_F16) tp::launch_group<tp::f16>(descs, n, cfg, s);
-        else tp::launch_group<tp::bf16>(descs, n, cfg, s);
+        const bool launched = descs[0].dtype == TP_F16 ? tp::launch_group<tp::f16>(descs, n, cfg, s)
+                                                       : tp::launch_group<tp::bf16>(descs, n, cfg, s);
+        if (!launched) {
+            tp::set_error("tp_gemm_grouped: no kernel for tile configuration %d, dtype %d", cfg, descs[0].dtype);
+            return TP_ERR_UNSUPPORTED;
+        }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) { tp::set_error("tp_gemm_grouped: launch failed: %s", hipGetErrorString(e)); return TP_ERR_LAUNCH; }
         return TP_OK;

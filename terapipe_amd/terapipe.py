@@ -188,6 +188,32 @@ def _flat_views(flat, layout):
     return [{n: flat[o:o + int(np.prod(s))].view(s) for n, (o, s) in d.items()} for d in layout]
 
 
+def fused_backward_slices(seq_slices, n_lanes, window=None):
+    """[(own_end, fused)] per sequence slice: the end of the positions whose delta a fused attention-backward launch
+    of the slice takes itself (the slice and the n_lanes - 1 slices after it, whose launches may still be running),
+    and whether the slice's attention backward goes out as that one launch.
+
+    A fused slice records its event BEFORE its launch, so the event does not stand for the delta that the launch
+    writes; a two-launch slice reads delta of every later position from memory after waiting for the next slice's
+    event only.  With several lanes a two-launch slice may therefore have no fused slice after it -- and since the
+    windows shrink towards the end of the sequence, that means all slices fused or none: fused when every slice's
+    window is at most `window` positions (ops.FUSED_BWD_WINDOW).  On one stream launches complete in issue order
+    and every slice decides for itself."""
+    window = ops.FUSED_BWD_WINDOW if window is None else window
+    n = max(int(n_lanes), 1)
+    L = sum(seq_slices)
+    ends, P = [], 0
+    for i, T in enumerate(seq_slices):
+        ends.append(min(L, P + sum(seq_slices[i:i + n])))
+        P += T
+    starts = [e - w for e, w in zip(np.cumsum(seq_slices).tolist(), seq_slices)]
+    spans = [e - s for e, s in zip(ends, starts)]
+    if n == 1:
+        return [(e, sp <= window) for e, sp in zip(ends, spans)]
+    every = max(spans) <= window
+    return [(e, every) for e in ends]
+
+
 def _program():
     rec = ops.CallRecorder.active
     return rec.program if rec is not None else None
@@ -312,6 +338,7 @@ def _backward_body(runner, ws, act, bufs, states):
         _wait_stream(st, main)
     if early_dw:
         _wait_stream(bufs.dw_stream, main)
+    fusion = fused_backward_slices(runner.seq_slices, len(lanes))
     for b in reversed(range(nb)):
         Bs = runner.batch_slices[b]
         pb = bufs.per_batch[b]
@@ -323,8 +350,7 @@ def _backward_body(runner, ws, act, bufs, states):
             P -= T
             r0, r1 = P * Bs, (P + T) * Bs
             last = i == ns - 1
-            # end of the positions whose delta a fused attention-backward launch of this slice takes itself
-            own_end = min(L, P + sum(runner.seq_slices[i:i + max(len(lanes), 1)]))
+            own_end, fuse = fusion[i]
             if runner.slice_timing is not None:
                 runner.slice_timing["bwd"].append(_timing_event(main))
             if bufs.position_indexed:
@@ -358,7 +384,7 @@ def _backward_body(runner, ws, act, bufs, states):
                                        suffix=dict(q_all=pb["q"][l], d_o_all=pb["d_o"][l], lse_all=pb["lse"][l],
                                                    delta_all=pb["delta"][l], q_end=L,
                                                    o_all=pb["o"][l].view(L, Bs, E) if bufs.fused_attn_bwd else None,
-                                                   own_end=own_end))
+                                                   own_end=own_end, fused=bufs.fused_attn_bwd and fuse))
                         if lanes:
                             # end of (slice, layer): what the parameter gradients of the layer wait for
                             fin = torch.cuda.Event()
@@ -590,8 +616,10 @@ class TeraPipe(nn.Module):
     False (and always in fp32) the gradient caches are used.
     fused_attn_bwd (with suffix_dkdv): dQ of a slice and the one-pass dK/dV of its keys go out as one launch whose
     two halves run side by side (the first streams the keys before the slice, the second the queries after it)
-    instead of two launches one after the other, whenever the slice and the slice_streams - 1 slices after it are
-    at most ops.FUSED_BWD_WINDOW positions together (the launch recomputes their delta).  Same results.
+    instead of two launches one after the other.  The launch recomputes delta of the slice and of the
+    slice_streams - 1 slices after it (its window); on one stream a slice is fused when its window is at most
+    ops.FUSED_BWD_WINDOW positions, on several streams all slices are fused when every window is, and none otherwise
+    (fused_backward_slices says why).  Same results.
     slice_streams (with suffix_dkdv, fp16 / bf16): slice i runs on stream i mod slice_streams.  The attention
     kernel of a layer waits (by event) for the in_proj GEMMs of the earlier slices at that layer, the one-pass
     dK/dV kernel for the dQ kernels of the later slices; nothing else orders slices, so consecutive slices

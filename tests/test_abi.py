@@ -131,6 +131,63 @@ def test_hip_graph_with_slice_streams_is_refused():
     assert r.slice_streams == 3 and r.launch_replay
 
 
+def _delta_reads_are_ordered(seq_slices, n_lanes, plan):
+    """Happens-before check of one layer of the reverse-order backward as the runner issues it: slice i runs on
+    lane i mod n_lanes; a two-launch slice issues dQ (writes its delta), waits for slice i+1's event, records its own,
+    then issues the one-pass dK/dV (reads delta of every later position from memory); a fused slice waits, records,
+    then issues one launch that writes its delta and reads delta from its own_end on.  Returns the first
+    (reader, writer) pair that nothing orders, or None."""
+    ns = len(seq_slices)
+    n = max(n_lanes, 1)
+    ends = [sum(seq_slices[:i + 1]) for i in range(ns)]
+    before_lane = {l: set() for l in range(n)}      # launches that precede the lane's next operation
+    event = {}                                       # slice -> launches its event stands for
+    for i in reversed(range(ns)):
+        lane = i % n
+        own_end, fused = plan[i]
+        if not fused:
+            before_lane[lane] = before_lane[lane] | {("w", i)}            # dQ launch leaves delta_i
+        if i + 1 in event:
+            before_lane[lane] = before_lane[lane] | event[i + 1]
+        event[i] = set(before_lane[lane])
+        first_read = own_end if fused else ends[i]
+        for j in range(i + 1, ns):
+            if ends[j] > first_read and ("w", j) not in before_lane[lane]:
+                return (i, j)
+        if fused:
+            before_lane[lane] = before_lane[lane] | {("w", i)}
+    return None
+
+
+def test_fused_backward_plan_orders_every_delta_read():
+    """Several lanes: no two-launch slice may come before a fused one (the fused slice's event is recorded before
+    the launch that writes its delta).  The rule decides once per step there; on one stream per slice."""
+    from terapipe_amd import ops
+    from terapipe_amd.terapipe import fused_backward_slices
+    W = ops.FUSED_BWD_WINDOW
+    cases = [[128] * 16, [64] * 32, [32] * 64, [512, 384, 320, 256, 224, 192, 160], [256] * 8, [16] * 8,
+             [40, 200, 24, 64, 32, 16, 8], [128, 64, 32, 32], [32, 32, 200, 32, 32], [2048]]
+    for ss in cases:
+        for n in (1, 2, 3, 4):
+            plan = fused_backward_slices(ss, n)
+            assert len(plan) == len(ss)
+            assert _delta_reads_are_ordered(ss, n, plan) is None, (ss, n)
+            for i, (own_end, fused) in enumerate(plan):
+                assert own_end == min(sum(ss), sum(ss[:i]) + sum(ss[i:i + n]))
+                if fused:
+                    assert own_end - sum(ss[:i]) <= W
+    # uniform 32-token slices on three lanes stay fused (96 positions), 128-token ones are not (384)
+    assert all(f for _, f in fused_backward_slices([32] * 64, 3))
+    assert not any(f for _, f in fused_backward_slices([128] * 16, 3))
+    assert all(f for _, f in fused_backward_slices([128] * 16, 1))
+    # the check has teeth: deciding per slice on three lanes (windows shrink at the sequence end, so the last slice
+    # of a 128-token slicing would be fused and the one before it not) leaves a read unordered
+    L = 2048
+    per_slice = [(e, e - 128 * i <= W) for i, (e, _) in enumerate(fused_backward_slices([128] * 16, 3))]
+    assert per_slice[15][1] and not per_slice[14][1]
+    assert _delta_reads_are_ordered([128] * 16, 3, per_slice) == (14, 15)
+
+
 def test_ops_refuse_cpu_tensors():
     """There is no CPU fallback: host tensors raise instead of computing."""
     from terapipe_amd import _lib, ops

@@ -94,3 +94,29 @@ def test_rule_examples():
     assert plan("NT", 384, 16384, 4096) == (14, 1)         # two row tiles of 192 x 128
     # fp32 keeps its own plan (64 x 64 register-staged tiles)
     assert plan("NT", 128, 4096, 4096, _lib.TP_F32)[0] == 0
+
+
+def _forced_plan(op, M, N, K, cfg, nsplit=0):
+    d = _lib.GemmDesc()
+    d.op, d.dtype, d.epilogue, d.M, d.N, d.K = OPS[op], _lib.TP_F16, _lib.TP_EPI_STORE, M, N, K
+    d.A = d.B = d.C = 4096
+    d.lda = M if op == "TN" else K
+    d.ldb = K if op == "NT" else N
+    d.ldc = N
+    d.reserved = (cfg + 1) | (nsplit << 8)
+    c, n = ctypes.c_int(), ctypes.c_int()
+    assert _lib.load().tp_gemm_plan(ctypes.byref(d), ctypes.byref(c), ctypes.byref(n)) == 0
+    return c.value, n.value
+
+
+def test_forced_tiles_that_load_whole_k_tiles_fall_back_on_a_ragged_k():
+    """A tile configuration forced through the descriptor's reserved field is replaced by the 128 x 128 register-
+    free tile (5) when the kernel behind it cannot run the shape: the weight-streaming, pipelined and tall tiles
+    load whole 64-wide k-tiles only, the weight-streaming tiles have no TN form."""
+    for cfg in (21, 26, 33, 40, 14, 15, 16, 19, 2):
+        assert _forced_plan("NT", 128, 1024, 1024, cfg)[0] == cfg, cfg          # K % 64 == 0: taken as forced
+        assert _forced_plan("NT", 128, 1024, 72, cfg)[0] == 5, cfg              # K = 72: would drop the k tail
+        assert _forced_plan("NN", 128, 1024, 1096, cfg)[0] == 5, cfg
+    for cfg in (21, 33):
+        assert _forced_plan("TN", 1024, 1024, 1024, cfg)[0] == 5, cfg
+    assert _forced_plan("NN", 128, 1024, 1024, 24)[0] == 5                      # 80-wide tiles: NT only

@@ -30,6 +30,7 @@ def test_static_workspace_gemm_matches_caller_workspace(dtype):
     lib = L.load(build_if_missing=False)
     g = torch.Generator(device=DEV).manual_seed(5)
     stream = torch.cuda.current_stream().cuda_stream
+    assert lib.tp_gemm_static_ws_capacity() == 64 << 20      # also looks up the array's address on this device
     # (op, M, N, K, k splits, epilogue): a large k-split product, then a smaller one with a bias epilogue, then one
     # whose plan does not split k at all (no workspace)
     cases = [(L.TP_GEMM_NT, 256, 2048, 8192, 4, L.TP_EPI_STORE),
@@ -50,8 +51,13 @@ def test_static_workspace_gemm_matches_caller_workspace(dtype):
         ws = torch.empty(max(need, 16), dtype=torch.uint8, device=DEV)
         print("static ws case op=%d %dx%dx%d splits=%d %s need=%d" % (op, M, N, K, ks, dtype, need), flush=True)
         L.check(lib.tp_gemm(ctypes.byref(d0), ws.data_ptr(), ws.numel(), stream), "tp_gemm")
+        torch.cuda.synchronize()
+        # the call under test allocates nothing: neither through torch nor behind its back (hipMemGetInfo)
+        held, (free0, _) = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()
         L.check(lib.tp_gemm_static_ws(ctypes.byref(d1), stream), "tp_gemm_static_ws")
         torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() == held
+        assert torch.cuda.mem_get_info()[0] >= free0, "device memory shrank across tp_gemm_static_ws"
         assert torch.equal(C0, C1), "op %d %dx%dx%d" % (op, M, N, K)
         ref = A.double() @ (Bm.double().t() if op == L.TP_GEMM_NT else Bm.double())
         if epi == L.TP_EPI_BIAS:
