@@ -146,6 +146,92 @@ def optimizer_step(layers, runner, x, R, reps=5):
             "note": "includes the host's build and upload of the tensor table each call"}
 
 
+def timed_steps(step, warmup, steps):
+    """(ms per step, tokens-independent) of `step()` over `steps` calls after `warmup`, host clock between two
+    synchronisations."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def layer_surface_step(layers, x, R, w):
+    """One step through the layer-level surface under the reference's own loop (terapipe.py:249-264 forward,
+    :182-191 backward): per slice ``layers(x_i, cache, cache_len)`` with the caches detached and marked
+    requires_grad, then in reverse ``autograd.backward([y_i] + cache_out_i, [dy_i] + da_{i+1})`` with
+    ``da_i = cache_in_i.grad``.  Every slice is one autograd graph on the calling stream, one slice at a time --
+    what a pipeline stage fed by an upstream stage runs."""
+    import terapipe_amd as ta
+    for p in layers.parameters():
+        p.grad = None
+    ss, B = w["slices"], w["B"]
+    xs = ta.grid_slice_batch_and_sequence(x, [B], ss, requires_grad=True)
+    dys = ta.grid_slice_batch_and_sequence(R, [B], ss)
+    cache = layers.create_cache(B, w["L"])
+    cin, cout, outs = [], [], []
+    cache_len = 0
+    for i, T in enumerate(ss):
+        cache = [c.detach().requires_grad_() for c in cache]
+        y, cache_out = layers(xs[0, i], cache, cache_len)
+        cin.append(cache)
+        cout.append(cache_out)
+        outs.append(y)
+        cache = cache_out
+        cache_len += T
+    da = []
+    for i in reversed(range(len(ss))):
+        a = list(cout[i]) if i < len(ss) - 1 else []
+        torch.autograd.backward([outs[i]] + a, [dys[0, i]] + da)
+        da = [t.grad for t in cin[i]]
+
+
+def box_constants(device, dtype=torch.float16):
+    """What this box delivers on two plain kernels, beside the published peaks the rooflines are priced against:
+    a 1 GiB device-to-device copy (bytes read + written per second) and an 8192^3 product on N(0,1) operands (this
+    library's tp_gemm and the vendor library behind torch.matmul), each replayed from a HIP graph between two events."""
+    from terapipe_amd import ops, _lib
+    n = 1 << 29
+    src = torch.empty(n, dtype=torch.int16, device=device).random_(-9, 9)
+    dst = torch.empty_like(src)
+    ms = _graph_ms([lambda: dst.copy_(src)] * 4) / 4
+    copy_gbps = 2 * n * 2 / (ms * 1e-3) / 1e9
+    del src, dst
+    M = 8192
+    A = torch.randn(M, M, device=device).to(dtype)
+    Bs = [torch.randn(M, M, device=device).to(dtype) for _ in range(3)]
+    C = torch.empty(M, M, device=device, dtype=dtype)
+    ours = _graph_ms([(lambda B=B: ops.gemm(_lib.TP_GEMM_NT, A, B, M, M, M, C=C)) for B in Bs]) / len(Bs)
+    vend = _graph_ms([(lambda B=B: torch.matmul(A, B.t(), out=C)) for B in Bs]) / len(Bs)
+    fl = 2.0 * M ** 3
+    return {"copy_GBps": round(copy_gbps, 1), "copy_frac_of_hbm_peak": round(copy_gbps * 1e9 / PEAK_HBM, 4),
+            "gemm_8192_TFLOPs": round(fl / (ours * 1e-3) / 1e12, 1),
+            "gemm_8192_frac_of_mfma_peak": round(fl / (ours * 1e-3) / PEAK_MFMA_16BIT, 4),
+            "vendor_gemm_8192_TFLOPs": round(fl / (vend * 1e-3) / 1e12, 1),
+            "note": "measured on this box: 1 GiB device copy (read + write bytes); NT 8192^3 fp16 on N(0,1) operands, "
+                    "tp_gemm and torch.matmul"}
+
+
+def in_step_picks():
+    """{(op, M, N, K)} of the measured plan table's entries that were chosen by timing whole steps on the slice
+    streams rather than the launch alone (their comments in gemm_tuned.inc say so): alone on the chip, as the
+    per-GEMM roofline times them, they are not the fastest plan of their shape."""
+    path = os.path.join(ROOT, "terapipe_amd", "csrc", "gemm_tuned.inc")
+    ops_ = {"NT": 0, "NN": 1, "TN": 2}
+    out = set()
+    try:
+        for line in open(path):
+            m = re.match(r"\{TP_GEMM_(\w+), (\d+), (\d+), (\d+), (\d+), (\d+)\},\s*//(.*)", line)
+            if m and ("in-step" in m.group(7) or "inside the step" in m.group(7)):
+                out.add((ops_[m.group(1)], int(m.group(2)), int(m.group(3)), int(m.group(4))))
+    except OSError:
+        pass
+    return out
+
+
 def cpu_baseline(w, sample_layers=None):
     """The CPU oracle (fp32 restatement of the reference path) on this host's cores, on a bounded
     sample: the full sequence and slice list through `sample_layers` layers of the stack; the
@@ -256,6 +342,21 @@ def measure_workload(name, args, device, detail):
            "ms_per_step": elapsed * 1e3 / steps, "tokens_per_s": w["L"] * w["B"] * steps / elapsed,
            "ms_per_step_std": (sum((t - mean) ** 2 for t in per_step) / steps) ** 0.5,
            "ms_per_step_min": min(per_step), "ms_per_step_max": max(per_step)}
+    if args.slice_streams > 1 and not args.graph:
+        # the same step with ONE slice stream: slice i+1 starts when slice i has left the stack, as on a pipeline
+        # stage that receives its slices from an upstream stage (terapipe.py:249-264); recorded launches re-issued
+        runner.slice_streams = 1
+        ms1 = timed_steps(lambda: one_step(layers, runner, x, R), 3, 5)
+        res["ms_per_step_one_stream"] = ms1
+        res["tokens_per_s_one_stream"] = w["L"] * w["B"] / (ms1 * 1e-3)
+        runner.slice_streams = args.slice_streams
+    if detail and w["dtype"] != "f32" and not args.no_layer_surface:
+        msl = timed_steps(lambda: layer_surface_step(layers, x, R, w), 2, 4)
+        res["layer_surface"] = {
+            "ms_per_step": msl, "tokens_per_s": w["L"] * w["B"] / (msl * 1e-3),
+            "what": "ModelParallelTransformerLayer.forward per slice under the reference's own loop and autograd "
+                    "(terapipe.py:249-264, :182-191): per-slice parameter-gradient GEMMs, gradient caches, one stream, "
+                    "every launch issued from Python"}
     if args.no_roofline:
         return res, (layers, runner, x, R)
 
@@ -314,6 +415,7 @@ def measure_workload(name, args, device, detail):
             groups.setdefault(c[1], []).append(c[2])
         groups = dict(sorted(groups.items(), key=lambda kv: str(kv[0])))
         per = []
+        picks = in_step_picks()
         for meta, fns in groups.items():
             ms = _graph_ms(fns)
             f, b = gemm_shape_work(meta, es)
@@ -322,7 +424,9 @@ def measure_workload(name, args, device, detail):
             per.append({"gemm": gemm_shape_name(meta), "calls": len(fns), "avg_us": round(us, 2),
                         "tflops": round(f / us / 1e6, 1), "bound_us": round(bound_us, 2),
                         "bound": "mfma" if f / peak >= b / PEAK_HBM else "hbm",
-                        "frac_of_bound": round(bound_us / us, 3)})
+                        "frac_of_bound": round(bound_us / us, 3),
+                        # the plan of this shape was chosen by timing whole steps, not this launch alone
+                        "in_step_pick": (not isinstance(meta[0], tuple)) and tuple(meta) in picks})
         if not args.no_vendor_gemm:
             # context only: the vendor library (hipBLASLt / rocBLAS behind torch.matmul) on the same products, plain
             # (no fused epilogue), timed the same way over weights that rotate through more memory than the caches hold
@@ -336,6 +440,9 @@ def measure_workload(name, args, device, detail):
                                       "note": "torch.matmul on the same (op, M, N, K) list, plain products, context only"}
         per.sort(key=lambda r: -r["avg_us"] * r["calls"])
         roof["per_gemm"] = per
+        roof["per_gemm_note"] = ("avg_us is the launch alone on the chip with the plan the step uses; in_step_pick marks "
+                                 "the shapes whose plan was chosen by timing whole steps on the slice streams (fewer k "
+                                 "splits than the fastest plan alone), so vendor_us may be below avg_us there")
     if args.slice_streams > 1:
         # the same GEMM calls as the step issues them: spread over the slice streams, so that a launch
         # which fills part of the chip runs beside its neighbours'.  Launched from the host (closures
@@ -499,6 +606,9 @@ def _short(res):
     """The other workloads' figures in short."""
     s = {"workload": res["workload"], "ms_per_step": round(res["ms_per_step"], 3),
          "tokens_per_s": round(res["tokens_per_s"], 1)}
+    if "ms_per_step_one_stream" in res:
+        s["ms_per_step_one_stream"] = round(res["ms_per_step_one_stream"], 3)
+        s["tokens_per_s_one_stream"] = round(res["tokens_per_s_one_stream"], 1)
     if "roofline" in res:
         r = res["roofline"]
         s["gemm"] = {"kernel_ms_per_step": round(r["kernel_ms_per_step"], 3), "achieved_TFLOPs": round(r["achieved"], 1),
@@ -524,6 +634,10 @@ def main():
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="with the default workload C3 the line also carries the prefix-attention roofline measured on C5 "
                          "(32-token slices) and short figures for C2, C4 and C5; this leaves them out")
+    ap.add_argument("--no-layer-surface", action="store_true",
+                    help="leave out the timing of the layer-level surface under the reference's own slice loop")
+    ap.add_argument("--no-box-constants", action="store_true",
+                    help="leave out the measured copy bandwidth and 8192^3 GEMM rate of this box")
     ap.add_argument("--no-vendor-gemm", action="store_true",
                     help="leave out the vendor library's times on the same GEMM shapes (context beside the per-GEMM table)")
     ap.add_argument("--attention-grid", action="store_true",
@@ -587,9 +701,12 @@ def main():
                               "eager, recorded launches re-issued from the host"),
                    "slice_streams": args.slice_streams},
     }
-    for k in ("roofline", "kernel_time_ms_per_step"):
+    for k in ("ms_per_step_one_stream", "tokens_per_s_one_stream", "layer_surface", "roofline", "kernel_time_ms_per_step"):
         if k in res:
             out[k] = res[k]
+    if "ms_per_step_one_stream" in res:
+        out["one_stream_note"] = ("value / ms_per_step overlap three consecutive slices on three streams of the one GPU; "
+                                  "*_one_stream run one slice at a time, as a pipeline stage fed by an upstream stage does")
     if "roofline_attention" in res:
         out["roofline_attention"] = dict(res["roofline_attention"], workload=args.workload)
     if args.optimizer and w["dtype"] != "f32":
@@ -613,6 +730,8 @@ def main():
                 out["roofline_attention"] = dict(r["roofline_attention"], workload="C5")
         out["other_workloads"] = others
 
+    if not args.no_box_constants and w["dtype"] != "f32":
+        out["box"] = box_constants(device, TORCH_DTYPE[w["dtype"]])
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)
 
