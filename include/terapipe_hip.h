@@ -214,7 +214,8 @@ typedef struct tp_attn_desc {
     int32_t reserved;                   /* 0 = automatic; bits 0-7: number of workgroups (fp32: splits) that share the key
                                            range of a query block in the forward (tuning, tests) */
     int32_t reserved2;                  /* tuning, tests.  bit 1 / bit 2: force the eight-wave / the four-wave form of the
-                                           16-bit forward kernel */
+                                           16-bit forward kernel; bit 3 / bit 4: force its workgroups of 32 / of 64 queries
+                                           (64 needs T >= 64) */
     int64_t q_bh_rows;                  /* rows per (b,h) block of q: 0 = T; see tp_gemm_desc.q_bh_rows */
     int64_t stat_bh_rows;               /* entries per (b,h) block of lse and delta: 0 = T */
     int32_t dq_only;                    /* backward: 1 = compute delta and the q part of dqkv only; dK/dV of the

@@ -1172,24 +1172,30 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
             for (int j = 0; j < 16; ++j) { sv[j] = sacc[j]; mt = fmaxf(mt, sv[j]); }
         }
         mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-        const float m_new = fmaxf(m, mt);
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = fast_exp2((m - m_safe) * kLog2e);
-        const float mneg = -m_safe * kLog2e;
+        // m is the row's REFERENCE value of the exponentials, not its running maximum: a row keeps it while its
+        // scores stay below m + kSlack (exponentials up to e^kSlack = 148, well inside fp16 and the fp32 sums), so
+        // the accumulators are rescaled only when some row of the wave outgrows that -- on the first tile and hardly
+        // ever again, where a running maximum moves for some of 32 rows on most tiles of a 2048-key range.  The
+        // row's log-sum-exp is m + log(sum) either way.
+        constexpr float kSlack = 5.0f;
+        if (__builtin_amdgcn_ballot_w64(mt > m + kSlack) != 0) {   // wave-uniform
+            const float m_new = fmaxf(m, mt);
+            const float alpha = m_new == -INFINITY ? 1.0f : fast_exp2((m - m_new) * kLog2e);
+            m = m_new;
+            lsum *= alpha;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+        }
+        const float mneg = m == -INFINITY ? 0.f : -m * kLog2e;
         float psum = 0.f;
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
             sv[j] = fast_exp2(fmaf(sv[j], kLog2e, mneg));   // exp(s - m); -inf -> 0
             psum += sv[j];
         }
-        lsum = lsum * alpha + psum;
-        m = m_new;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {   // wave-uniform: some row's running maximum moved
-#pragma unroll
-            for (int db = 0; db < NDB; ++db)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
-        }
+        lsum += psum;
         uint4 pop[2];
         pop[0] = pack8<T>(sv);
         pop[1] = pack8<T>(sv + 8);
@@ -1259,6 +1265,299 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd2_kernel(AttnArgs a) {
             else store4<T>(dst + c, acc4.x, acc4.y, acc4.z, acc4.w);
         }
     }
+}
+
+// Forward for slices of 64 queries and more.  A workgroup owns 64 queries of one (batch, head) -- two blocks of 32 --
+// and, as in attn_fwd2_kernel, its NW waves split the key range, each streaming its own K / V tiles through a
+// private two-stage ring.  Every wave works on BOTH query blocks against each tile it has fetched: a K / V byte
+// enters LDS once per 64 queries instead of once per 32 (the global -> LDS path is what bounds the 32-query form
+// from 128-token slices on), the K and V^T operands are read from LDS once for two blocks, and the two blocks are
+// independent instruction chains.  The loop is software-pipelined so that one straight-line block holds the
+// exponentials of tile t, its output MFMAs and the score MFMAs of tile t + 1 -- vector ALU and MFMA work with no
+// dependency between them, for the scheduler to interleave (one wave per SIMD: two blocks' accumulators and query
+// operands take more than half of the register file).  What has to sit between two such blocks is short: the row
+// maxima of the new scores, and the rescaling of the accumulators on the rare tile that moves a row's maximum.
+// A pair whose second block lies beyond the slice computes it on zero queries and stores nothing of it.
+template <typename T, int DH, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_fwd3_kernel(AttnArgs a) {
+    typedef Elem<T> E;
+    static_assert(sizeof(T) == 2, "direct-to-LDS kernels are for fp16 / bf16");
+    constexpr int NDB = DH / 32, NKS = DH / 16;
+    constexpr int TILE = 32 * DH;
+    constexpr int CPR = DH / 8;
+    constexpr int NLD = 32 * CPR / 64;                   // loads per K or V tile and lane
+    static_assert(3 * NLD <= 63, "too many loads in flight for vmcnt");
+    constexpr int WAVE_RING = 2 * 2 * TILE * 2;          // bytes: two stages of K + V
+    constexpr int EPI_LD = DH + 4;
+    constexpr int STAT_FLOATS = 2 * NW * 32;
+    constexpr int EPI_BYTES = (STAT_FLOATS + NW * 32 * EPI_LD) * 4;
+    constexpr int SMEM = NW * WAVE_RING > EPI_BYTES ? NW * WAVE_RING : EPI_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM];
+
+    const int tid = threadIdx.x, lane = tid & 63, g = lane >> 5, li = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int bh, qblk;
+    if (!xcd_map(a.B * a.H, bh, qblk)) return;
+    const int b = bh / a.H, h = bh - b * a.H;
+    const int T_ = a.T, P = a.P, S = a.P + a.T;
+    const long EE = (long)a.H * DH;
+    const int q0 = ((T_ + 63) / 64 - 1 - qblk) * 64;     // the pairs with the longest key range start first
+    const bool two = q0 + 32 < T_;                       // workgroup-uniform: the pair's second block exists
+    const int tq0 = q0 + li, tq1 = q0 + 32 + li;
+    const bool qok0 = tq0 < T_, qok1 = tq1 < T_;
+    const int kv_end = P + min(T_, q0 + 64);
+    const int ntiles = (kv_end + 31) / 32;
+    int wg_beg = 0, wg_end = ntiles;
+    if (a.nsplit > 1) {
+        const int per = (ntiles + a.nsplit - 1) / a.nsplit;
+        wg_beg = min(ntiles, (int)blockIdx.y * per);
+        wg_end = min(ntiles, wg_beg + per);
+    }
+    const int tpw = (wg_end - wg_beg + NW - 1) / NW;
+    const int t_beg = wg_beg + wave * tpw, t_end = min(wg_end, t_beg + tpw);
+    const int nt = max(t_end - t_beg, 0);
+
+    T* ring = reinterpret_cast<T*>(smem) + wave * (WAVE_RING / 2);
+    const unsigned ring_lds = lds_addr(smem) + wave * WAVE_RING;
+
+    const T* pkm[NKS];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) pkm[ks] = ring + km_offset<T, DH>(li, ks * 16, lane);
+    const T* ptr0[NDB];
+    const T* ptr1[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+        int o0, o1;
+        tr_offsets<T, DH, true>(0, db * 32, lane, o0, o1);
+        ptr0[db] = ring + TILE + o0;          // inside the V tile
+        ptr1[db] = ring + TILE + o1;
+    }
+    unsigned koff[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int p = i * 64 + lane;
+        const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+        koff[i] = (unsigned)(r * DH * 2 + lc * 16);
+    }
+    const char* Kb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.kc) + (long)bh * a.cache_rows * DH));
+    const char* Vb = uniform_ptr(reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.vc) + (long)bh * a.cache_rows * DH));
+
+    // one tile (K: which = 0, V: which = 1) of 32 keys into its half of a stage; rows at or past S are clamped to
+    // row S - 1: finite data, and every such key is masked
+    auto issue = [&](int stage, int which, int tile) {
+        const unsigned dst = ring_lds + (unsigned)((stage * 2 + which) * TILE * 2);
+        const char* base = which ? Vb : Kb;
+        const int row0 = tile * 32;
+        if (row0 + 32 <= S) {
+            const char* sb = base + (long)row0 * (DH * 2);
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) dma16_saddr_lds(koff[i], sb, dst + i * 1024);
+        } else {
+            const int last = S - 1;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int p = i * 64 + lane;
+                const int r = p / CPR, lc = (p % CPR) ^ swz16<DH>(r);
+                const unsigned off = (unsigned)(min(row0 + r, last) * DH * 2 + lc * 16);
+                dma16_saddr_lds(off, base, dst + i * 1024);
+            }
+        }
+    };
+
+    float16v oacc0[NDB], oacc1[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { oacc0[db][r] = 0.f; oacc1[db][r] = 0.f; }
+    float m0 = -INFINITY, l0 = 0.f, m1 = -INFINITY, l1 = 0.f;
+
+    // loads go out in the order K(0) V(0) K(1) V(1), then per tile t: K(t + 2) when its body starts, V(t + 2) when
+    // it ends (vector-memory operations complete in issue order)
+    if (nt > 0) { issue(0, 0, t_beg); issue(0, 1, t_beg); }
+    if (nt > 1) { issue(1, 0, t_beg + 1); issue(1, 1, t_beg + 1); }
+    typename E::opnd_t qreg0[NKS], qreg1[NKS];
+    const T* qbase = reinterpret_cast<const T*>(a.q) + (long)bh * a.q_bhs;
+    load_row_operands<T, DH>(qreg0, qbase + (long)tq0 * DH, qok0, g);
+    load_row_operands<T, DH>(qreg1, qbase + (long)(qok1 ? tq1 : 0) * DH, qok1, g);
+
+    // score blocks of both query blocks against the K tile in stage `so`
+    auto scores = [&](int so, float16v& s0, float16v& s1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s0[r] = 0.f; s1[r] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            const typename E::opnd_t kop = load_km<T>(pkm[ks] + so);
+            s0 = E::mfma(kop, qreg0[ks], s0);
+            s1 = E::mfma(kop, qreg1[ks], s1);
+        }
+    };
+    // causal mask (tiles at a block's boundary only) and the row maxima of one block's scores
+    auto tile_max = [&](float16v& sc, int key0, int tq, int qb0) {
+        if (key0 + 31 > P + qb0) {           // wave-uniform
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                if (key0 + acc_row(j, g) > P + tq) sc[j] = -INFINITY;
+        }
+        float mt = sc[0];
+#pragma unroll
+        for (int j = 1; j < 16; ++j) mt = fmaxf(mt, sc[j]);
+        return fmaxf(mt, __shfl_xor(mt, 32, 64));
+    };
+    // exp(s - m) of one block, packed as the two MFMA operands; returns the lane's share of the row sums
+    auto exps = [&](const float16v& sc, float mneg, uint4* pop) {
+        float sv[16];
+        float psum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            sv[j] = fast_exp2(fmaf(sc[j], kLog2e, mneg));   // -inf -> 0
+            psum += sv[j];
+        }
+        pop[0] = pack8<T>(sv);
+        pop[1] = pack8<T>(sv + 8);
+        return psum;
+    };
+
+    float16v s0, s1;
+    if (nt > 0) {
+        if (nt > 1) wait_vmcnt<3 * NLD>(); else wait_vmcnt<NLD>();
+        scores(0, s0, s1);
+    }
+    // (the score MFMAs of "the next tile" also run behind a wave's last tile, on whatever the other stage holds:
+    // nothing reads their result, and the loop body stays one piece of code per stage)
+    auto body = [&](auto stage_c, int it) {
+        constexpr int st = decltype(stage_c)::value;
+        constexpr int so = st * 2 * TILE, son = (st ^ 1) * 2 * TILE;
+        const int key0 = (t_beg + it) * 32;
+        // -- between the straight-line blocks: row maxima, and the rare move of the reference --
+        // m0 / m1 are the rows' REFERENCE values of the exponentials, not their running maxima: a row keeps its
+        // reference while its scores stay below reference + kSlack (exponentials up to e^kSlack = 148, well inside
+        // fp16 and the fp32 sums), so that the accumulators are rescaled only when some row of the wave outgrows
+        // that -- on the first tile, and hardly ever again (a running maximum moves for some row of 64 on nearly
+        // every tile of a 2048-key range).  The row's log-sum-exp is reference + log(sum) either way.
+        constexpr float kSlack = 5.0f;
+        const float mt0 = tile_max(s0, key0, tq0, q0), mt1 = tile_max(s1, key0, tq1, q0 + 32);
+        float al0 = 1.0f, al1 = 1.0f;
+        if (__builtin_amdgcn_ballot_w64(mt0 > m0 + kSlack || mt1 > m1 + kSlack) != 0) {
+            const float mn0 = fmaxf(m0, mt0), mn1 = fmaxf(m1, mt1);
+            al0 = mn0 == -INFINITY ? 1.0f : fast_exp2((m0 - mn0) * kLog2e);
+            al1 = mn1 == -INFINITY ? 1.0f : fast_exp2((m1 - mn1) * kLog2e);
+            m0 = mn0; m1 = mn1;
+            // The accumulators stay in accumulation registers for the whole loop: a plain multiply here would make
+            // them vector registers everywhere (the vector ALU cannot address the other file) and the loop would
+            // spill.  The copies are explicit, with the wait states an MFMA result needs before it is read and a
+            // written register before an MFMA takes it as its addend.
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float t0, t1;
+                    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t0) : "a"(oacc0[db][r]));
+                    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t1) : "a"(oacc1[db][r]));
+                    t0 *= al0; t1 *= al1;
+                    asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(oacc0[db][r]) : "v"(t0));
+                    asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(oacc1[db][r]) : "v"(t1));
+                }
+            asm volatile("s_nop 7" ::: "memory");
+            l0 *= al0; l1 *= al1;
+        }
+        const float ms0 = m0 == -INFINITY ? 0.f : m0, ms1 = m1 == -INFINITY ? 0.f : m1;
+        if (it + 2 < nt) { issue(st, 0, t_beg + it + 2); wait_vmcnt<2 * NLD>(); }   // K(it) was read one body ago
+        else wait_vmcnt<0>();
+        // -- the block: exponentials and output MFMAs of this tile, score MFMAs of the next --
+        uint4 av[2][NDB];
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+                av[hs][db] = load_tr<T>(ptr0[db] + so + hs * 16 * DH, ptr1[db] + so + hs * 16 * DH);
+        float16v n0, n1;
+        scores(son, n0, n1);
+        uint4 p0[2], p1[2];
+        l0 += exps(s0, -ms0 * kLog2e, p0);
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) oacc0[db] = E::mfma(av[hs][db], p0[hs], oacc0[db]);
+        l1 += exps(s1, -ms1 * kLog2e, p1);
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) oacc1[db] = E::mfma(av[hs][db], p1[hs], oacc1[db]);
+        s0 = n0; s1 = n1;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the stage's V tile is in registers
+        if (it + 2 < nt) issue(st, 1, t_beg + it + 2);
+    };
+    for (int it = 0; it < nt; it += 2) {
+        body(std::integral_constant<int, 0>(), it);
+        if (it + 1 < nt) body(std::integral_constant<int, 1>(), it + 1);
+    }
+    wait_vmcnt<0>();
+
+    // merge of the NW partial (m, l, O) of a block through LDS, one block after the other in the same space
+    float* sM = reinterpret_cast<float*>(smem);
+    float* sL = sM + NW * 32;
+    float* ebuf = sL + NW * 32;
+    const bool partial = a.nsplit > 1;
+    constexpr int CPT = 32 * DH / (NW * 64);
+    static_assert(CPT % 4 == 0 && DH % CPT == 0, "bad reduction split");
+    auto finish = [&](float16v* oacc, float m, float lsum, int qb0, int tq, bool qok) {
+        __syncthreads();       // every wave is done with its ring (or with the previous block's merge)
+        const float lw = lsum + __shfl_xor(lsum, 32, 64);
+        if (g == 0) { sM[wave * 32 + li] = m; sL[wave * 32 + li] = lw; }
+        __syncthreads();
+        float m_tot = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) m_tot = fmaxf(m_tot, sM[w * 32 + li]);
+        const float m_ts = m_tot == -INFINITY ? 0.f : m_tot;
+        float L = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) L += sL[w * 32 + li] * fast_exp2((sM[w * 32 + li] - m_ts) * kLog2e);
+        const float f = L > 0.f ? fast_exp2((m - m_ts) * kLog2e) / L : 0.f;
+        // (the accumulators are read out of their accumulation registers explicitly, see the loop; layout as
+        // acc_to_lds_rows)
+        {
+            float* wbuf = ebuf + wave * 32 * EPI_LD;
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int jq = 0; jq < 4; ++jq) {
+                    float t[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[e]) : "a"(oacc[db][4 * jq + e]));
+                        t[e] *= f;
+                    }
+                    *reinterpret_cast<float4*>(wbuf + li * EPI_LD + db * 32 + 8 * jq + 4 * g) = make_float4(t[0], t[1], t[2], t[3]);
+                }
+        }
+        const long prow0 = ((long)blockIdx.y * (a.B * a.H) + bh) * T_;
+        if (wave == 0 && g == 0 && qok) {
+            const float lse_wg = L > 0.f ? m_tot + logf(L) : -INFINITY;
+            if (partial) a.part_lse[prow0 + tq] = lse_wg;
+            else a.lse[(long)bh * a.st_bhs + tq] = lse_wg;
+        }
+        __syncthreads();
+        const int row = tid / (DH / CPT), c0 = (tid % (DH / CPT)) * CPT;
+        if (qb0 + row < T_) {
+            T* dst = reinterpret_cast<T*>(a.o) + ((long)(qb0 + row) * a.B + b) * EE + (long)h * DH + c0;
+            float* pdst = a.part_o + (prow0 + qb0 + row) * DH + c0;
+#pragma unroll
+            for (int c = 0; c < CPT; c += 4) {
+                float4 acc4 = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int w = 0; w < NW; ++w) {
+                    const float4 v = *reinterpret_cast<const float4*>(ebuf + (w * 32 + row) * EPI_LD + c0 + c);
+                    acc4.x += v.x; acc4.y += v.y; acc4.z += v.z; acc4.w += v.w;
+                }
+                if (partial) *reinterpret_cast<float4*>(pdst + c) = acc4;
+                else store4<T>(dst + c, acc4.x, acc4.y, acc4.z, acc4.w);
+            }
+        }
+    };
+    finish(oacc0, m0, l0, q0, tq0, qok0);
+    if (two) finish(oacc1, m1, l1, q0 + 32, tq1, qok1);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1607,7 +1906,13 @@ static FwdPlan plan_fwd(const tp_attn_desc* d) {
     FwdPlan p;
     if (d->dtype != TP_F32 && tiled16(d->head_dim)) {
         // 16-bit: one workgroup per 32 queries whose four waves split the key range and merge in LDS
-        p.nw = 0; p.bn = 32; p.nsplit = 1; p.qblocks = (d->T + 31) / 32;
+        // slices of 64 queries and more: workgroups of 64 queries (attn_fwd3_kernel; p.bn = 64); reserved2 bit 3
+        // forces the 32-query workgroups
+        // -- when the pairs still give the chip enough workgroups (measured: ahead from 160 on, 5 to 20 %; behind
+        // at 64 to 120, where the 32-query form has twice the workgroups and eight waves each); bit 4 forces them
+        const bool pairs = d->T >= 64 && !(d->reserved2 & 8) &&
+                           ((long)d->batch * d->heads * ((d->T + 63) / 64) >= 160 || (d->reserved2 & 16));
+        p.nw = 0; p.bn = 32; p.nsplit = 1; p.qblocks = pairs ? (d->T + 63) / 64 : (d->T + 31) / 32;
         // A call with so few query blocks that over half of the CUs would get no workgroup, and a key range long
         // enough to share (16 tiles of 32 keys per share), spreads each block's keys over as many workgroups as fit
         // the chip; they leave fp32 partials in the workspace and the merge launch weighs them together.  Measured
@@ -1626,6 +1931,7 @@ static FwdPlan plan_fwd(const tp_attn_desc* d) {
         // from about twenty key tiles on (measured: 19 against 24 us at 2048 keys, 7.9 against 7.6 us at 256);
         // reserved2 bit 1 forces it, bit 2 forces four waves
         if (((long)d->cache_len + d->T >= 640 || (d->reserved2 & 2)) && !(d->reserved2 & 4)) p.bn = 8;
+        if (pairs) p.bn = 64;
         return p;
     }
     p.nw = d->T > 64 ? 4 : (d->T > 32 ? 2 : 1);
@@ -1667,7 +1973,8 @@ static void launch_fwd(const FwdPlan& p, const AttnArgs& a, hipStream_t s) {
     dim3 grid(p.qblocks, a.B * a.H, p.nsplit);
     if constexpr (sizeof(T) == 2 && (DH == 64 || DH == 128)) {
         const dim3 g2(xcd_grid(a.B * a.H, (a.T + 31) / 32), p.nsplit);
-        if (p.bn == 8) attn_fwd2_kernel<T, DH, 8, 1><<<g2, 512, 0, s>>>(a);
+        if (p.bn == 64) attn_fwd3_kernel<T, DH, 4><<<dim3(xcd_grid(a.B * a.H, (a.T + 63) / 64), p.nsplit), 256, 0, s>>>(a);
+        else if (p.bn == 8) attn_fwd2_kernel<T, DH, 8, 1><<<g2, 512, 0, s>>>(a);
         else attn_fwd2_kernel<T, DH, 4><<<g2, 256, 0, s>>>(a);
     } else {
         if (p.nw == 4) attn_fwd_kernel<T, DH, 4, 64><<<grid, 256, 0, s>>>(a);

@@ -416,8 +416,9 @@ def test_attn_prefix_fwd_bwd(dtype, T, B, H, Dh, P, L):
     assert_close(o, oref, dtype, "attn o")
     s = torch.bmm(q64, k64[:, :S].transpose(1, 2)) + oracle.causal_prefix_mask(T, P, torch.float64)
     assert_close(lse, torch.logsumexp(s, -1), torch.float32, "attn lse", 1e3 if dtype != torch.float32 else 10)
-    # both wave counts of the 16-bit forward, whatever the plan picks for this length
-    for variant in (2, 4):
+    # both wave counts of the 16-bit forward's 32-query workgroups and its 64-query workgroups (from 64 queries on),
+    # whatever the plan picks for this shape
+    for variant in (2 | 8, 4 | 8, 16):
         o_v, lse_v = ops.attn_prefix_fwd(qd, kd, vd, B, H, Dh, T, P, 1.0, variant=variant)
         assert_close(o_v, oref, dtype, "attn o, forward variant %d" % variant)
         assert_close(lse_v, torch.logsumexp(s, -1), torch.float32, "attn lse, forward variant %d" % variant,
@@ -550,7 +551,7 @@ def test_attn_fwd_keys_shared_by_workgroups(dtype, T, B, H, Dh, P, ns):
     q64, k64, v64 = q.double(), kc.double(), vc.double()
     oref = _attn_ref(q64, k64, v64, B, H, T, P)
     lse_ref = torch.logsumexp(torch.bmm(q64, k64.transpose(1, 2)) + oracle.causal_prefix_mask(T, P, torch.float64), -1)
-    for variant in (2, 4):
+    for variant in (2 | 8, 4 | 8, 16):
         o, lse = ops.attn_prefix_fwd(q.to(DEV), kc.to(DEV), vc.to(DEV), B, H, Dh, T, P, 1.0, nsplit=ns, variant=variant)
         assert_close(o, oref, dtype, "o, keys over %d workgroups, variant %d" % (ns, variant))
         assert_close(lse, lse_ref, torch.float32, "lse, keys over %d workgroups, variant %d" % (ns, variant), 1e3)
