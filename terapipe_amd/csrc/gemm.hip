@@ -520,10 +520,15 @@ static bool tile_cfg(int id, TileCfg& c) {
     case 38: c = {64, 128, 64, 8}; return true;    // 16 waves
     case 39: c = {128, 256, 64, 3}; return true;   // 8 waves
     case 40: c = {64, 256, 64, 4}; return true;    // 8 waves
+    // gemm_pipe_kernel again: row tiles that fit slices of 224 and of 160 / 320 rows (whole 16-row blocks, so
+    // nothing of a tile lies beyond the slice)
+    case 41: c = {224, 128, 64, 3}; return true;   // 2 x 2 waves of 112 x 64
+    case 42: c = {160, 128, 64, 3}; return true;   // 2 x 2 waves of 80 x 64
+    case 43: c = {224, 160, 64, 3}; return true;   // 2 x 2 waves of 112 x 80 (NT only, like 6 and 7)
     default: return false;
     }
 }
-static constexpr int kFirstStreamCfg = 21;
+static constexpr int kFirstStreamCfg = 21, kLastStreamCfg = 40;
 
 // Measured plans: for NT / NN the weight extents (N, K) match exactly and M (tokens of the slice) picks the
 // nearest measured M at or above it (at least half of it, so that a much shorter slice falls through to the
@@ -688,11 +693,13 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     if (forced_split) ns = forced_split;
     // the tall tiles load whole k-tiles only, and the 160 / 192 wide ones exist for the k-major weight (NT)
     // (a token-major tile 160 or 192 wide has no XOR swizzle: the chunk index would leave the row)
-    if ((cfg == 6 || cfg == 7) && (d->K % 64 || d->op != TP_GEMM_NT)) cfg = 5;
+    if ((cfg == 6 || cfg == 7 || cfg == 43) && (d->K % 64 || d->op != TP_GEMM_NT)) cfg = 5;
+    if ((cfg == 41 || cfg == 42) && (d->K % 64 || d->op == TP_GEMM_TN)) cfg = 5;
     if (((cfg >= 14 && cfg <= 20) || cfg == 2) && (d->K % 64 || (cfg == 17 && d->op != TP_GEMM_NT) || (cfg == 14 && d->op == TP_GEMM_TN))) cfg = 5;
     // the streaming kernel: NT and NN only, whole 64-wide k-tiles only; tiles whose width is not a power of two need
     // the k-major weight (NT)
-    if (cfg >= kFirstStreamCfg && (d->op == TP_GEMM_TN || d->K % 64 || ((cfg == 24 || cfg == 25) && d->op != TP_GEMM_NT))) cfg = 5;
+    if (cfg >= kFirstStreamCfg && cfg <= kLastStreamCfg &&
+        (d->op == TP_GEMM_TN || d->K % 64 || ((cfg == 24 || cfg == 25) && d->op != TP_GEMM_NT))) cfg = 5;
     p.cfg = cfg;
     tile_cfg(cfg, tc);
     p.gx = (d->N + tc.bn - 1) / tc.bn;
@@ -702,7 +709,7 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
 }
 
 // the tile configurations of gemm_pipe.hip
-static inline bool is_pipe_cfg(int cfg) { return cfg == 6 || cfg == 7 || (cfg >= 14 && cfg <= 16); }
+static inline bool is_pipe_cfg(int cfg) { return cfg == 6 || cfg == 7 || (cfg >= 14 && cfg <= 16) || (cfg >= 41 && cfg <= 43); }
 
 template <typename T, bool AKM, bool BKM>
 static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
@@ -731,7 +738,7 @@ static void launch_cfg(const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
 // false: the plan names a (tile configuration, op, dtype) that no kernel is built for -- nothing was launched
 template <typename T>
 static bool launch_gemm(const tp_gemm_desc* d, const GemmPlan& p, const GemmArgs& a, hipStream_t s) {
-    if (p.cfg >= kFirstStreamCfg) {
+    if (p.cfg >= kFirstStreamCfg && p.cfg <= kLastStreamCfg) {
         if (!launch_gemm_stream(p.cfg, d->op, d->dtype, dim3(p.gx, p.gy, p.nsplit), a, s)) return false;
     } else if (is_pipe_cfg(p.cfg) && d->dtype != TP_F32) {
         if (!launch_gemm_pipe(p.cfg, d->op, d->dtype, dim3(p.gx, p.gy, p.nsplit), a, s)) return false;

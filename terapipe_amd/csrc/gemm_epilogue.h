@@ -150,7 +150,7 @@ __device__ __forceinline__ void xcd_tile3(int t, int tx, int ty, int tz, int& ti
 }
 
 
-// The pipelined tiles of gemm_pipe.hip (tile configurations 6, 7, 14, 15, 16 of the plan): launches `cfg` on `grid` =
+// The pipelined tiles of gemm_pipe.hip (tile configurations 6, 7, 14, 15, 16, 41, 42, 43 of the plan): launches `cfg` on `grid` =
 // (column tiles, row tiles, k splits); false when cfg / op / dtype has no such kernel.
 bool launch_gemm_pipe(int cfg, int op, int dtype, dim3 grid, const GemmArgs& a, hipStream_t s);
 // A grouped launch (TN, token-major operands) of `tiles` workgroups on the pipelined 256 x 128 tile.

@@ -241,6 +241,9 @@ static bool launch_pipe_cfg(int cfg, dim3 grid, const GemmArgs& a, hipStream_t s
     case 14: if constexpr (AKM) { gemm_pipe_kernel<T, AKM, BKM, 192, 128, 2, 2, 3><<<grid, 256, 0, s>>>(a); return true; } return false;
     case 15: gemm_pipe_kernel<T, AKM, BKM, 256, 128, 4, 1, 3><<<grid, 256, 0, s>>>(a); return true;
     case 16: gemm_pipe_kernel<T, AKM, BKM, 128, 128, 2, 2, 3><<<grid, 256, 0, s>>>(a); return true;
+    case 41: if constexpr (AKM) { gemm_pipe_kernel<T, AKM, BKM, 224, 128, 2, 2, 3><<<grid, 256, 0, s>>>(a); return true; } return false;
+    case 42: if constexpr (AKM) { gemm_pipe_kernel<T, AKM, BKM, 160, 128, 2, 2, 3><<<grid, 256, 0, s>>>(a); return true; } return false;
+    case 43: if constexpr (AKM && BKM) { gemm_pipe_kernel<T, AKM, BKM, 224, 160, 2, 2, 3><<<grid, 256, 0, s>>>(a); return true; } return false;
     default: return false;
     }
 }

@@ -31,7 +31,7 @@ DEFAULT_GEOMETRIES = [
     "12288:49152:128:2048",                                 # 175B shape, 128-token slices
     "6144:24576:64:4096",                                   # 44B shape, 32-token slices x batch 2
 ]
-DMA_CFGS = [2, 3, 5, 6, 7, 8, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20]
+DMA_CFGS = [2, 3, 5, 6, 7, 8, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20, 41, 42, 43]
 # the weight-streaming kernel's configurations (NT and NN only; 24 and 25 NT only): cfg -> rows of its row tile
 STREAM_CFGS = {21: 192, 22: 256, 24: 192, 25: 256, 26: 128, 29: 256, 30: 192, 31: 192, 32: 256, 33: 192, 34: 256,
                35: 128, 36: 64, 37: 128, 38: 64}
@@ -132,6 +132,8 @@ def sweep(op, M, N, K, dtype, device, log, pair=False):
             if cfg in (2, 6, 7, 14, 15, 16) and (K % 64 or (cfg == 14 and op == "TN") or (cfg in (6, 7) and op != "NT") or
                                                  (cfg in (2, 6, 7, 14, 15) and M < 128)):
                 continue
+            if cfg in (41, 42, 43) and (K % 64 or op == "TN" or (cfg == 43 and op != "NT") or M < 128):
+                continue
             if cfg in STREAM_CFGS and ((cfg in (24, 25) and op != "NT") or STREAM_CFGS[cfg] < M // 2 or
                                        STREAM_CFGS[cfg] >= 2 * M):
                 continue
@@ -159,7 +161,7 @@ def shapes_of(geometry):
     return out
 
 
-def in_step(spec, dtype=torch.float16, log=sys.stderr, only_rows=None):
+def in_step(spec, dtype=torch.float16, log=sys.stderr, only_rows=None, only_cfgs=None):
     """Coordinate descent over the plans of the slice GEMMs (NT forward, NN data gradient) of one geometry,
     timing whole steps.  Returns [(op, M, N, K, cfg, nsplit)] for the shapes whose plan changed."""
     import time
@@ -207,12 +209,14 @@ def in_step(spec, dtype=torch.float16, log=sys.stderr, only_rows=None):
     for op, M, N, K in shapes:
         key = (OPS[op], M, N, K)
         trials = []
-        for cfg in DMA_CFGS:
+        for cfg in (only_cfgs or DMA_CFGS):
             for ns in IN_STEP_SPLITS:
-                if K // ns < 512 or (cfg >= 17 and (M < 192 or K % 64)) or (cfg == 17 and op != "NT"):
+                if K // ns < 512 or (17 <= cfg <= 20 and (M < 192 or K % 64)) or (cfg == 17 and op != "NT"):
                     continue
                 if cfg in (2, 6, 7, 14, 15, 16) and (K % 64 or (cfg in (6, 7) and op != "NT") or
                                                      (cfg in (2, 6, 7, 14, 15) and M < 128)):
+                    continue
+                if cfg in (41, 42, 43) and (K % 64 or (cfg == 43 and op != "NT") or M < 128):
                     continue
                 ops.GEMM_PLAN_OVERRIDE[key] = (cfg, ns)
                 try:
@@ -247,6 +251,8 @@ def main():
     ap.add_argument("--only-rows", metavar="M,M,...",
                     help="with --in-step: search only the slice GEMMs of these row counts (a whole geometry can take "
                          "longer than one sitting)")
+    ap.add_argument("--only-cfgs", metavar="C,C,...",
+                    help="with --in-step: try only these tile configurations (the incumbent plan stays the yardstick)")
     ap.add_argument("--pair", action="store_true",
                     help="time two concurrent chains of each GEMM on two streams (per-call time with a neighbour) "
                          "instead of one chain alone")
@@ -257,7 +263,8 @@ def main():
         sys.exit("tune_gemm: needs the GPU")
     if args.in_step:
         rows = {int(v) for v in args.only_rows.split(",")} if args.only_rows else None
-        for op, M, N, K, cfg, ns, ms in in_step(args.in_step, only_rows=rows):
+        cfgs = [int(v) for v in args.only_cfgs.split(",")] if args.only_cfgs else None
+        for op, M, N, K, cfg, ns, ms in in_step(args.in_step, only_rows=rows, only_cfgs=cfgs):
             print("{TP_GEMM_%s, %d, %d, %d, %d, %d},  // in-step search: step %.2f ms" % (op, M, N, K, cfg, ns, ms))
         return
     device = torch.device("cuda:0")

@@ -14,7 +14,7 @@ OPS = {"NT": _lib.TP_GEMM_NT, "NN": _lib.TP_GEMM_NN, "TN": _lib.TP_GEMM_TN}
 # tile configuration -> (rows, columns, workgroups that fit a CU)
 TILES = {0: (64, 64, 2), 2: (256, 256, 1), 6: (192, 160, 1), 7: (160, 160, 1), 3: (128, 256, 1), 5: (128, 128, 2), 8: (64, 64, 2), 10: (128, 128, 2), 11: (64, 256, 1),
          12: (64, 64, 2), 13: (128, 128, 1), 14: (192, 128, 1), 15: (256, 128, 1), 16: (128, 128, 1), 17: (256, 160, 1), 18: (256, 128, 1), 19: (256, 256, 1), 20: (256, 256, 1),
-         31: (192, 128, 1), 33: (192, 256, 1)}
+         31: (192, 128, 1), 33: (192, 256, 1), 41: (224, 128, 1), 42: (160, 128, 1), 43: (224, 160, 1)}
 
 
 def plan(op, M, N, K, dtype=_lib.TP_F16):
@@ -113,10 +113,11 @@ def test_forced_tiles_that_load_whole_k_tiles_fall_back_on_a_ragged_k():
     """A tile configuration forced through the descriptor's reserved field is replaced by the 128 x 128 register-
     free tile (5) when the kernel behind it cannot run the shape: the weight-streaming, pipelined and tall tiles
     load whole 64-wide k-tiles only, the weight-streaming tiles have no TN form."""
-    for cfg in (21, 26, 33, 40, 14, 15, 16, 19, 2):
+    for cfg in (21, 26, 33, 40, 14, 15, 16, 19, 2, 41, 42, 43):
         assert _forced_plan("NT", 128, 1024, 1024, cfg)[0] == cfg, cfg          # K % 64 == 0: taken as forced
         assert _forced_plan("NT", 128, 1024, 72, cfg)[0] == 5, cfg              # K = 72: would drop the k tail
         assert _forced_plan("NN", 128, 1024, 1096, cfg)[0] == 5, cfg
-    for cfg in (21, 33):
+    for cfg in (21, 33, 41, 42, 43):
         assert _forced_plan("TN", 1024, 1024, 1024, cfg)[0] == 5, cfg
     assert _forced_plan("NN", 128, 1024, 1024, 24)[0] == 5                      # 80-wide tiles: NT only
+    assert _forced_plan("NN", 224, 1024, 1024, 43)[0] == 5                      # 160-wide pipelined tile: NT only
