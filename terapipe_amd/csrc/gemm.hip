@@ -670,12 +670,17 @@ static GemmPlan plan_gemm(const tp_gemm_desc* d) {
     // The pipelined 16 x 16 x 32 tiles in place of the 32 x 32 ones the rules above name, where a sweep over other
     // geometries (hidden 3072, 4096, 8192; 128 to 512 rows; 144 slice products) has them ahead: 128 x 128 for
     // 128 x 128 (0.94 to 0.99 of the time), 192 x 128 for 128 x 256 at 129 to 192 rows and at 257 to 384 (0.83 to 0.91),
-    // 256 x 128 above 384 rows (0.92); a k-split stays within one round of workgroups of the new tile.
+    // 256 x 128 above 384 rows (0.92), and the 160- and 224-row tiles where they end with the slice (0.95 to 1.0 of
+    // the padded tile's time on the 13B shapes); a k-split stays within one round of workgroups of the new tile.
     if (d->op != TP_GEMM_TN && d->K % 64 == 0 && (cfg == 13 || cfg == 3)) {
         int bm = 128, bn = 128, to = 16;
         if (cfg == 3) {
-            if ((d->M > 128 && d->M <= 192) || (d->M > 256 && d->M <= 384)) { to = 14; bm = 192; }
-            else if (d->M > 384) { to = 15; bm = 256; }
+            // row tiles that end with the slice where whole 16-row blocks allow it: 160 (one or two tiles), 192 (one
+            // or two), 224 (one or two), else 256
+            if ((d->M > 128 && d->M <= 160) || (d->M > 256 && d->M <= 320)) { to = 42; bm = 160; }
+            else if ((d->M > 160 && d->M <= 192) || (d->M > 320 && d->M <= 384)) { to = 14; bm = 192; }
+            else if ((d->M > 192 && d->M <= 224) || (d->M > 384 && d->M <= 448)) { to = 41; bm = 224; }
+            else if (d->M > 448) { to = 15; bm = 256; }
             else to = 3;
         }
         if (to != 3) {

@@ -92,6 +92,10 @@ def test_rule_examples():
     assert plan("NT", 512, 20480, 4096) == (19, 1)         # two rows of 256 x 256 tiles
     assert plan("NN", 512, 4096, 16384) == (15, 4)         # 2 x 32 pipelined tiles of 256 x 128 on a long k
     assert plan("NT", 384, 16384, 4096) == (14, 1)         # two row tiles of 192 x 128
+    assert plan("NT", 224, 16384, 8192) == (41, 2)         # one row of 224 x 128 tiles: nothing of a tile beyond the slice
+    assert plan("NN", 448, 8192, 32768) == (41, 2)         # two of them
+    assert plan("NT", 320, 16384, 8192) == (42, 1)         # two row tiles of 160 x 128
+    assert plan("NT", 160, 32768, 8192) == (42, 1)         # one
     # fp32 keeps its own plan (64 x 64 register-staged tiles)
     assert plan("NT", 128, 4096, 4096, _lib.TP_F32)[0] == 0
 
