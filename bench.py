@@ -215,6 +215,32 @@ def box_constants(device, dtype=torch.float16):
                     "tp_gemm and torch.matmul"}
 
 
+def fill_path(device):
+    """What the global -> LDS path delivers when nothing else runs (tp_fill_probe): every workgroup's four waves
+    stream 8 KB batches into LDS, four batches in flight per wave and one 128 KB workgroup per CU -- the footprint
+    of a GEMM tile ring -- from a 4 GiB region that no two waves share a byte of (HBM: misses) and / or a 2 MiB
+    region (L2: hits), on 256, 128 and 64 CUs; a batch is 8 KB of consecutive bytes or a 64-row x 128-byte tile.  These rates bound every kernel here that stages operand tiles through LDS: a tile's bytes divided by the
+    rate of its hit : miss mix is the least time a k-tile can take, whatever the MFMA pipe could do meanwhile."""
+    from terapipe_amd import ops
+    big = torch.empty(1 << 30, dtype=torch.int32, device=device).random_(0, 7)
+    small = torch.empty(1 << 19, dtype=torch.int32, device=device).random_(0, 7)     # 2 MiB
+    rows = []
+    # consecutive bytes on 256, 128 and 64 CUs, then the tile walk of a GEMM's k loop (64 rows x 128 bytes, row pitch
+    # 10240 bytes = a k of 5120 16-bit elements) on 256 CUs
+    for wgs, stride in ((256, 0), (128, 0), (64, 0), (256, 10240)):
+        for hpm, name in ((-1, "all L2 hits"), (7, "7 hits : 1 HBM"), (3, "3 : 1"), (1, "1 : 1"), (0, "all HBM")):
+            batches = 512 if hpm != 0 else 256       # 256 workgroups x 4 waves x 512 batches x 8 KB = the 4 GiB
+            nbytes = wgs * 4 * batches * 8192
+            ms = _graph_ms([lambda: ops.fill_probe(big, small, hpm, wgs, batches, row_stride=stride)] * 3, 3) / 3
+            rate = nbytes / (ms * 1e-3)
+            hbm = rate * (0.0 if hpm < 0 else 1.0 / (hpm + 1))
+            rows.append({"workgroups": wgs, "pattern": "consecutive bytes" if stride == 0 else "64 x 128 B tiles, row pitch %d B" % stride,
+                         "mix": name, "us": round(ms * 1e3, 1), "GBps_per_CU": round(rate / wgs / 1e9, 1),
+                         "chip_TBps": round(rate / 1e12, 2), "of_which_HBM_TBps": round(hbm / 1e12, 2)})
+    return {"metric": "global -> LDS fill rate (global_load_lds_dwordx4, 128 KB of LDS and 16 batches of 8 KB in flight per CU)",
+            "unit": "GB/s per CU, TB/s chip-wide", "peak_HBM_TBps": PEAK_HBM / 1e12, "rows": rows}
+
+
 def in_step_picks():
     """{(op, M, N, K)} of the measured plan table's entries that were chosen by timing whole steps on the slice
     streams rather than the launch alone (their comments in gemm_tuned.inc say so): alone on the chip, as the
@@ -642,6 +668,9 @@ def main():
                     help="leave out the vendor library's times on the same GEMM shapes (context beside the per-GEMM table)")
     ap.add_argument("--attention-grid", action="store_true",
                     help="print the (T, P) micro-grid of the prefix-attention kernels instead of the step benchmark")
+    ap.add_argument("--fill-path", action="store_true",
+                    help="print what the global -> LDS path of the CUs delivers (hits, misses and mixes) instead of the "
+                         "step benchmark")
     ap.add_argument("--two-launch-attn-bwd", action="store_true",
                     help="issue dQ and the one-pass dK/dV of a slice as two launches instead of one (comparison)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -673,6 +702,9 @@ def main():
     torch.cuda.set_device(device)
     if args.attention_grid:
         print(json.dumps(attention_grid(device)))
+        return
+    if args.fill_path:
+        print(json.dumps(fill_path(device)))
         return
     if args.graph and (args.eager or args.slice_streams != 1):
         print("bench.py: --graph replays a single-stream capture; use it with --slice-streams 1 and without --eager",

@@ -343,6 +343,17 @@ int tp_accum_cast(void* dst, const float* src, int64_t n, int accumulate, int dt
 int tp_colsum_acc(const void* x, int64_t ldx, float* acc, int M, int N, int dtype, void* stream);
 /* fills n 32-bit words with zero (a kernel, so it can be recorded into a HIP graph) */
 int tp_zero_words(void* dst, int64_t n_words, void* stream);
+/* Measurement aid, no counterpart in the reference: `workgroups` workgroups of four waves each stream
+   batches_per_wave batches of 8192 bytes per wave into LDS with global_load_lds_dwordx4 (128 KB of LDS and four
+   batches in flight per wave: one workgroup per CU) and do nothing else.  hits_per_miss < 0: every batch from
+   small_region (which the L2 holds); 0: every batch from the wave's own stretch of big (HBM); n > 0: one batch of
+   big after every n of small_region.  row_stride 0: a batch is 8192 consecutive bytes; else a batch is a tile of 64
+   rows x 128 bytes of a row-major matrix with row_stride bytes between rows, and consecutive batches of a source
+   walk along the rows -- the access pattern of a GEMM's k loop over a k-major operand.  Bytes moved:
+   workgroups * 4 * batches_per_wave * 8192.  bench.py --fill-path times it: the rates bound every kernel here that
+   stages operand tiles through LDS. */
+int tp_fill_probe(const void* big, int64_t big_bytes, const void* small_region, int64_t small_bytes,
+                  int hits_per_miss, int workgroups, int batches_per_wave, int64_t row_stride, void* stream);
 
 #ifdef __cplusplus
 }

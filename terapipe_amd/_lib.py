@@ -130,6 +130,7 @@ SYMBOLS = {
     "tp_accum_cast": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "tp_colsum_acc": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_void_p]),
     "tp_zero_words": (c_int, [c_void_p, c_int64, c_void_p]),
+    "tp_fill_probe": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_int64, c_void_p]),
 }
 
 _lock = threading.Lock()

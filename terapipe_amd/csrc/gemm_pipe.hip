@@ -220,12 +220,16 @@ void gemm_pipe_kernel(typename std::conditional<GROUPED, GemmGroupArgs, GemmArgs
         tile_steady(std::integral_constant<int, 0>{});
         if constexpr (STAGES > 1) tile_steady(std::integral_constant<int, 1>{});
         if constexpr (STAGES > 2) tile_steady(std::integral_constant<int, 2>{});
+        if constexpr (STAGES > 3) tile_steady(std::integral_constant<int, 3>{});
+        if constexpr (STAGES > 4) tile_steady(std::integral_constant<int, 4>{});
     }
     for (; kt0 < nk; kt0 += STAGES) {
         if (kt0 + 0 < nk) tile(std::integral_constant<int, 0>{}, kt0);
         if constexpr (STAGES > 1) { if (kt0 + 1 < nk) tile(std::integral_constant<int, 1>{}, kt0 + 1); }
         if constexpr (STAGES > 2) { if (kt0 + 2 < nk) tile(std::integral_constant<int, 2>{}, kt0 + 2); }
-        static_assert(STAGES <= 3, "at most three stages");
+        if constexpr (STAGES > 3) { if (kt0 + 3 < nk) tile(std::integral_constant<int, 3>{}, kt0 + 3); }
+        if constexpr (STAGES > 4) { if (kt0 + 4 < nk) tile(std::integral_constant<int, 4>{}, kt0 + 4); }
+        static_assert(STAGES <= 5, "at most five stages");
     }
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();

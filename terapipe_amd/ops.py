@@ -441,6 +441,18 @@ def zero_(t):
     return t
 
 
+def fill_probe(big, small, hits_per_miss, workgroups, batches_per_wave, row_stride=0):
+    """Launches the library's global -> LDS streaming probe (tp_fill_probe) on the current stream; returns the bytes
+    it moves.  big / small: contiguous device tensors whose byte sizes are multiples of 8192.  row_stride (bytes):
+    0 = consecutive bytes, else 64-row x 128-byte tiles of a matrix with that row pitch."""
+    _require_cuda(big, small)
+    lib = _lib.load()
+    nb, ns = big.numel() * big.element_size(), small.numel() * small.element_size()
+    _lib.check(lib.tp_fill_probe(_p(big), nb, _p(small), ns, int(hits_per_miss), int(workgroups), int(batches_per_wave),
+                                 int(row_stride), _stream()), "tp_fill_probe")
+    return workgroups * 4 * batches_per_wave * 8192
+
+
 def embedding_fwd(ids, weight, out=None):
     """ids int64 [M] -> out [M, E] = weight[ids]."""
     _require_cuda(ids, weight)

@@ -83,6 +83,9 @@ def test_argument_errors_without_gpu(lib):
     assert b"head_dim" in lib.tp_last_error()
     assert lib.tp_layernorm_fwd(None, None, None, None, None, None, 4, 64, 1e-5, 0, None) == 1
     assert lib.tp_zero_words(None, 4, None) == 1
+    assert lib.tp_fill_probe(None, 8192, None, 8192, 0, 1, 1, 0, None) == 1
+    assert lib.tp_fill_probe(4096, 8192, 4096, 100, 0, 1, 1, 0, None) == 1   # region not a multiple of 8192 bytes
+    assert lib.tp_fill_probe(4096, 8192, 4096, 8192, 0, 1, 1, 1024, None) == 1   # 64 rows of that pitch do not fit
 
 
 def test_every_head_dimension_of_the_model_table_is_accepted(lib):

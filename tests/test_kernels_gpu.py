@@ -719,6 +719,21 @@ def test_vec_param_grads_one_launch(dtype):
         assert_close(accs[5 + 2 * k] - 0.5, dy.double().sum(0), torch.float32, "dbeta %d" % k, 1e2 * tol)
 
 
+def test_fill_probe_runs_every_mix():
+    """The global -> LDS streaming probe behind `bench.py --fill-path`: every hit : miss mix launches, completes and
+    leaves its source regions as they were (it only reads)."""
+    ops = _ops()
+    big = torch.arange(1 << 22, dtype=torch.int32, device=DEV)       # 16 MiB
+    small = torch.arange(1 << 18, dtype=torch.int32, device=DEV)     # 1 MiB
+    for hpm in (-1, 0, 1, 3, 7):
+        for stride in (0, 2048, 10240):
+            moved = ops.fill_probe(big, small, hpm, 64, 16, row_stride=stride)
+            assert moved == 64 * 4 * 16 * 8192
+    torch.cuda.synchronize()
+    assert torch.equal(big, torch.arange(1 << 22, dtype=torch.int32, device=DEV))
+    assert torch.equal(small, torch.arange(1 << 18, dtype=torch.int32, device=DEV))
+
+
 def test_error_paths():
     """Bad arguments come back as status codes with a message; nothing is launched."""
     import ctypes
