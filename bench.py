@@ -368,7 +368,7 @@ def measure_workload(name, args, device, detail):
            "ms_per_step": elapsed * 1e3 / steps, "tokens_per_s": w["L"] * w["B"] * steps / elapsed,
            "ms_per_step_std": (sum((t - mean) ** 2 for t in per_step) / steps) ** 0.5,
            "ms_per_step_min": min(per_step), "ms_per_step_max": max(per_step)}
-    if args.slice_streams > 1 and not args.graph:
+    if args.slice_streams > 1 and not args.graph and not args.no_one_stream:
         # the same step with ONE slice stream: slice i+1 starts when slice i has left the stack, as on a pipeline
         # stage that receives its slices from an upstream stage (terapipe.py:249-264); recorded launches re-issued
         runner.slice_streams = 1
@@ -660,6 +660,8 @@ def main():
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="with the default workload C3 the line also carries the prefix-attention roofline measured on C5 "
                          "(32-token slices) and short figures for C2, C4 and C5; this leaves them out")
+    ap.add_argument("--no-one-stream", action="store_true",
+                    help="leave out the timing of the same step on one slice stream")
     ap.add_argument("--no-layer-surface", action="store_true",
                     help="leave out the timing of the layer-level surface under the reference's own slice loop")
     ap.add_argument("--no-box-constants", action="store_true",
