@@ -160,7 +160,7 @@ def timed_steps(step, warmup, steps):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
-def layer_surface_step(layers, x, R, w):
+def layer_surface_step(layers, x, R, w, in_place=False):
     """One step through the layer-level surface under the reference's own loop (terapipe.py:249-264 forward,
     :182-191 backward): per slice ``layers(x_i, cache, cache_len)`` with the caches detached and marked
     requires_grad, then in reverse ``autograd.backward([y_i] + cache_out_i, [dy_i] + da_{i+1})`` with
@@ -169,6 +169,8 @@ def layer_surface_step(layers, x, R, w):
     import terapipe_amd as ta
     for p in layers.parameters():
         p.grad = None
+    for layer in layers.layers:
+        layer.accumulate_grads_in_place = in_place
     ss, B = w["slices"], w["B"]
     xs = ta.grid_slice_batch_and_sequence(x, [B], ss, requires_grad=True)
     dys = ta.grid_slice_batch_and_sequence(R, [B], ss)
@@ -382,11 +384,16 @@ def measure_workload(name, args, device, detail):
         runner.slice_streams = args.slice_streams
     if detail and w["dtype"] != "f32" and not args.no_layer_surface:
         msl = timed_steps(lambda: layer_surface_step(layers, x, R, w), 2, 4)
+        msi = timed_steps(lambda: layer_surface_step(layers, x, R, w, in_place=True), 2, 4)
+        for layer in layers.layers:
+            layer.accumulate_grads_in_place = False
         res["layer_surface"] = {
             "ms_per_step": msl, "tokens_per_s": w["L"] * w["B"] / (msl * 1e-3),
+            "ms_per_step_grads_in_place": msi, "tokens_per_s_grads_in_place": w["L"] * w["B"] / (msi * 1e-3),
             "what": "ModelParallelTransformerLayer.forward per slice under the reference's own loop and autograd "
                     "(terapipe.py:249-264, :182-191): per-slice parameter-gradient GEMMs, gradient caches, one stream, "
-                    "every launch issued from Python"}
+                    "every launch issued from Python; grads_in_place: with accumulate_grads_in_place=True, the "
+                    "slices after the first add their parameter gradients to .grad inside the gradient kernels"}
     if args.no_roofline:
         return res, (layers, runner, x, R)
 
@@ -668,6 +675,11 @@ def main():
                     help="leave out the timing of the same step on one slice stream")
     ap.add_argument("--no-layer-surface", action="store_true",
                     help="leave out the timing of the layer-level surface under the reference's own slice loop")
+    ap.add_argument("--layer-surface-only", action="store_true",
+                    help="time only the layer-level surface (the reference's per-slice loop under autograd) for "
+                         "--steps steps after --warmup and print its line: the run to put under a kernel trace")
+    ap.add_argument("--grads-in-place", action="store_true",
+                    help="with --layer-surface-only: set accumulate_grads_in_place on the layers")
     ap.add_argument("--no-box-constants", action="store_true",
                     help="leave out the measured copy bandwidth and 8192^3 GEMM rate of this box")
     ap.add_argument("--no-vendor-gemm", action="store_true",
@@ -721,6 +733,14 @@ def main():
               file=sys.stderr)
         sys.exit(2)
     w = WORKLOADS[args.workload]
+    if args.layer_surface_only:
+        layers, runner, x, R = build_model(w, device)
+        del runner
+        ms = timed_steps(lambda: layer_surface_step(layers, x, R, w, args.grads_in_place), args.warmup, args.steps)
+        print(json.dumps({"workload": "%s: %s" % (args.workload, w["desc"]), "layer_surface_ms_per_step": ms,
+                          "accumulate_grads_in_place": args.grads_in_place,
+                          "tokens_per_s": w["L"] * w["B"] / (ms * 1e-3), "steps": args.steps, "warmup": args.warmup}))
+        return
     if args.copy_calibration:
         src = torch.ones(64 << 20, dtype=torch.int32, device=device)
         dst = torch.empty_like(src)

@@ -14,7 +14,7 @@ import torch.nn as nn
 
 from . import _layer_core as core
 from . import ops
-from ._lib import TP_EPI_BIAS, TP_EPI_STORE, TP_GEMM_NN, TP_GEMM_NT, TP_GEMM_TN
+from ._lib import TP_EPI_ACCUMULATE, TP_EPI_BIAS, TP_EPI_STORE, TP_GEMM_NN, TP_GEMM_NT, TP_GEMM_TN
 
 # reference transformer_models.py:16 -- kept for callers that import it; the kernels mask by index.
 NEG_INF = -65504
@@ -177,21 +177,27 @@ def _temp_cache(B, H, T, Dh, like):
             torch.empty(B * H, T, Dh, dtype=like.dtype, device=like.device))
 
 
-def _small_grads(acc_views, w):
-    out = {}
-    for name in core.SMALL_PARAMS:
-        g = torch.empty_like(w[name])
-        ops.accum_cast(g, acc_views[name], False)
-        out[name] = g
-    return out
+def _grads_can_go_in_place(w):
+    """Every parameter of the layer already has a dense .grad of its own dtype to add to."""
+    for p in w.values():
+        g = p.grad
+        if g is None or g.dtype != p.dtype or g.shape != p.shape or not g.is_contiguous():
+            return False
+    return True
 
 
 class _LayerFunction(torch.autograd.Function):
     """One whole layer over one slice.  Inputs: x, k_cache, v_cache (or None, None), then the 12
-    parameters in core.PARAM_NAMES order.  Outputs: out, and the two caches when given."""
+    parameters in core.PARAM_NAMES order.  Outputs: out, and the two caches when given.
+
+    Backward of a slice: the data gradients (core.layer_bwd), then the four weight gradients of the slice as one
+    grouped library call and its eight vector-parameter gradients as one launch.  grads_in_place: where every
+    parameter already has a .grad, add this slice's gradients to it inside those launches (the GEMM's accumulate
+    epilogue, one rounding) and hand autograd None for them, instead of returning twelve tensors that autograd
+    adds to .grad one elementwise kernel each."""
 
     @staticmethod
-    def forward(ctx, heads, cache_len, activation, x, k_cache, v_cache, *params):
+    def forward(ctx, heads, cache_len, activation, grads_in_place, x, k_cache, v_cache, *params):
         w = dict(zip(core.PARAM_NAMES, params))
         T, B, E = x.shape
         Dh = E // heads
@@ -200,6 +206,7 @@ class _LayerFunction(torch.autograd.Function):
             k_cache, v_cache = _temp_cache(B, heads, T, Dh, x)
         out, st = core.layer_fwd(w, x.contiguous(), heads, k_cache, v_cache, cache_len, activation)
         ctx.st, ctx.w, ctx.heads, ctx.activation = st, w, heads, activation
+        ctx.grads_in_place = bool(grads_in_place)
         ctx.set_materialize_grads(False)
         if ctx.has_cache:
             # the caches were written through their raw pointers (as `cache.data[index] = value` does,
@@ -223,16 +230,40 @@ class _LayerFunction(torch.autograd.Function):
                 has_incoming = True
             else:
                 gk, gv = torch.zeros_like(st.k_cache), torch.zeros_like(st.v_cache)
-        acc = torch.zeros(core.small_acc_numel(E, F), dtype=torch.float32, device=dout.device)
-        views = core.small_acc_views(acc, E, F)
-        wgrad = {n: torch.empty_like(w[n]) for n in core.BIG_PARAMS}
-        dx = core.layer_bwd(w, st, dout.contiguous(), heads, gk, gv, wgrad, False, views,
+        M, dt, dev = st.T * st.B, st.x.dtype, dout.device
+        dout = dout.contiguous()
+        dout2d = dout.view(M, E)
+        new = lambda n: torch.empty(M, n, dtype=dt, device=dev)
+        buf = core.Bufs(dz1=new(F), dhn=new(E), dh=new(E), dqkv=new(3 * E), dxn=new(E))
+        dx = core.layer_bwd(w, st, dout, heads, gk, gv, None, False, None,
                             accumulate_prefix=True, has_incoming=has_incoming, zero_slice_rows=has_incoming,
-                            activation=ctx.activation)
-        grads = _small_grads(views, w)
-        grads.update(wgrad)
+                            activation=ctx.activation, buf=buf)
+        in_place = ctx.grads_in_place and _grads_can_go_in_place(w)
+        epi = TP_EPI_ACCUMULATE if in_place else TP_EPI_STORE
+        wgrad = {n: (w[n].grad if in_place else torch.empty_like(w[n])) for n in core.BIG_PARAMS}
+        ops.gemm_grouped([(TP_GEMM_TN, buf.dqkv, st.xn, 3 * E, E, M, wgrad["attn.in_proj.weight"], epi),
+                          (TP_GEMM_TN, buf.dh, st.o.view(M, E), E, E, M, wgrad["attn.out_proj.weight"], epi),
+                          (TP_GEMM_TN, buf.dz1, st.hn, F, E, M, wgrad["fc1.weight"], epi),
+                          (TP_GEMM_TN, dout2d, st.a, E, F, M, wgrad["fc2.weight"], epi)])
+        acc = torch.zeros(core.small_acc_numel(E, F), dtype=torch.float32, device=dev)
+        sv = core.small_acc_views(acc, E, F)
+        ops.vec_param_grads([(buf.dqkv, sv["attn.in_proj.bias"]),
+                             (buf.dh, sv["attn.out_proj.bias"]),
+                             (buf.dz1, sv["fc1.bias"]),
+                             (dout2d, sv["fc2.bias"]),
+                             (buf.dxn, st.x, st.mean1, st.rstd1, sv["attn_ln.weight"], sv["attn_ln.bias"]),
+                             (buf.dhn, st.h, st.mean2, st.rstd2, sv["fc_ln.weight"], sv["fc_ln.bias"])])
+        if in_place:
+            for n in core.SMALL_PARAMS:
+                ops.accum_cast(w[n].grad, sv[n], True)
+            grads = dict.fromkeys(core.PARAM_NAMES)
+        else:
+            flat = torch.empty(acc.numel(), dtype=dt, device=dev)
+            ops.accum_cast(flat, acc, False)
+            grads = core.small_acc_views(flat, E, F)
+            grads.update(wgrad)
         ctx.st = None
-        return (None, None, None, dx, gk, gv) + tuple(grads[n] for n in core.PARAM_NAMES)
+        return (None, None, None, None, dx, gk, gv) + tuple(grads[n] for n in core.PARAM_NAMES)
 
 
 class _AttentionFunction(torch.autograd.Function):
@@ -343,6 +374,12 @@ class TransformerLayer(nn.Module):
     """Reference transformer_models.py:264-285: pre-LN block with a ReLU MLP.  (The reference's plain
     class omits `checkpoint_gradients` and cannot run; here it defaults to False.)"""
 
+    # Set True (per instance or on the class) to have the backward of a slice add its parameter gradients to
+    # existing .grad tensors inside the gradient kernels instead of returning them to autograd.  Same sums with one
+    # rounding fewer; only for loops that call .backward() / autograd.backward (as the reference's does):
+    # torch.autograd.grad would see None for the parameters, and post-accumulate-grad hooks do not fire.
+    accumulate_grads_in_place = False
+
     def __init__(self, embedding_dim, ffn_embedding_dim, num_attention_heads, device="cpu",
                  checkpoint_gradients=False, activation="relu"):
         super().__init__()
@@ -372,8 +409,8 @@ class TransformerLayer(nn.Module):
         else:
             assert cache_len == 0
         p = self.param_dict()
-        res = _LayerFunction.apply(self.attn.num_heads, cache_len, self.activation, x, k, v,
-                                   *[p[n] for n in core.PARAM_NAMES])
+        res = _LayerFunction.apply(self.attn.num_heads, cache_len, self.activation, self.accumulate_grads_in_place,
+                                   x, k, v, *[p[n] for n in core.PARAM_NAMES])
         if full_cache is not None:
             return res[0], (res[1], res[2])
         return res, None

@@ -227,10 +227,12 @@ def _reference_style_loop(layers, x, dy, batch_slices, seq_slices):
     return y, dx, finals, cg
 
 
+@pytest.mark.parametrize("in_place", [False, True], ids=["autograd-accumulates", "grads-in-place"])
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
-def test_reference_style_slice_loop(dtype):
+def test_reference_style_slice_loop(dtype, in_place):
     """Layer-level autograd contract: detach()/requires_grad_() caches per slice, backward with the
-    cache-output gradients of the next slice, cache-input .grad as hand-off."""
+    cache-output gradients of the next slice, cache-input .grad as hand-off.  in_place: the slices after the
+    first add their parameter gradients to .grad inside the gradient kernels (accumulate_grads_in_place)."""
     ta = _mods()
     n_layers, E, H, L, B = 2, 256, 4, 64, 2
     Fd = 4 * E
@@ -245,6 +247,8 @@ def test_reference_style_slice_loop(dtype):
     yo, dxo, fco, cgo = oracle.terapipe_forward_backward(leaf, x.float(), dy.float(), H, bs, ss,
                                                          return_cache_grads=True, activation=act)
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps, act)
+    for layer in layers.layers:
+        layer.accumulate_grads_in_place = in_place
     y, dx, finals, cg = _reference_style_loop(layers, x.to(DEV), dy.to(DEV), bs, ss)
     assert_close(y, yo, dtype, "y")
     assert_close(dx, dxo, dtype, "dx")
@@ -255,6 +259,30 @@ def test_reference_style_slice_loop(dtype):
                 P = sum(ss[:i])
                 assert_close(cg[b][i][j], cgo[b][i][j], dtype, "cache grad b%d slice %d tensor %d" % (b, i, j))
                 assert (cg[b][i][j][:, P:] == 0).all(), "rows >= P of the cache gradient are zero"
+    _check_param_grads(_param_grads(layers), [{k: v.grad for k, v in p.items()} for p in leaf], dtype, "ref loop")
+
+
+@pytest.mark.parametrize("in_place", [False, True], ids=["autograd-accumulates", "grads-in-place"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_reference_style_slice_loop_on_64_row_multiples(dtype, in_place):
+    """The same loop on slices of 128 / 64 / 192 tokens at hidden 512: a slice's four weight gradients meet
+    the conditions of the grouped launch (k a multiple of 64), with the store and the accumulate epilogue."""
+    ta = _mods()
+    n_layers, E, H, L, B = 2, 512, 4, 384, 1
+    Fd = 4 * E
+    bs, ss = [1], [128, 64, 192]
+    ps = make_params(n_layers, E, Fd, dtype, seed=3)
+    g = torch.Generator().manual_seed(11)
+    x, dy = torch.randn(L, B, E, generator=g).to(dtype), torch.randn(L, B, E, generator=g).to(dtype)
+    leaf = [{k: v.clone().requires_grad_(True) for k, v in p.items()} for p in ps]
+    yo, dxo, fco, cgo = oracle.terapipe_forward_backward(leaf, x.float(), dy.float(), H, bs, ss,
+                                                         return_cache_grads=True, activation="gelu")
+    layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps, "gelu")
+    for layer in layers.layers:
+        layer.accumulate_grads_in_place = in_place
+    y, dx, finals, cg = _reference_style_loop(layers, x.to(DEV), dy.to(DEV), bs, ss)
+    assert_close(y, yo, dtype, "y")
+    assert_close(dx, dxo, dtype, "dx")
     _check_param_grads(_param_grads(layers), [{k: v.grad for k, v in p.items()} for p in leaf], dtype, "ref loop")
 
 
