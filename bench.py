@@ -160,7 +160,7 @@ def timed_steps(step, warmup, steps):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
-def layer_surface_step(layers, x, R, w, in_place=False):
+def layer_surface_step(layers, x, R, w, in_place=False, defer=False):
     """One step through the layer-level surface under the reference's own loop (terapipe.py:249-264 forward,
     :182-191 backward): per slice ``layers(x_i, cache, cache_len)`` with the caches detached and marked
     requires_grad, then in reverse ``autograd.backward([y_i] + cache_out_i, [dy_i] + da_{i+1})`` with
@@ -171,6 +171,7 @@ def layer_surface_step(layers, x, R, w, in_place=False):
         p.grad = None
     for layer in layers.layers:
         layer.accumulate_grads_in_place = in_place
+        layer.defer_weight_grads = defer
     ss, B = w["slices"], w["B"]
     xs = ta.grid_slice_batch_and_sequence(x, [B], ss, requires_grad=True)
     dys = ta.grid_slice_batch_and_sequence(R, [B], ss)
@@ -385,15 +386,20 @@ def measure_workload(name, args, device, detail):
     if detail and w["dtype"] != "f32" and not args.no_layer_surface:
         msl = timed_steps(lambda: layer_surface_step(layers, x, R, w), 2, 4)
         msi = timed_steps(lambda: layer_surface_step(layers, x, R, w, in_place=True), 2, 4)
+        msd = timed_steps(lambda: layer_surface_step(layers, x, R, w, defer=True), 2, 4)
         for layer in layers.layers:
-            layer.accumulate_grads_in_place = False
+            layer.accumulate_grads_in_place = layer.defer_weight_grads = False
         res["layer_surface"] = {
             "ms_per_step": msl, "tokens_per_s": w["L"] * w["B"] / (msl * 1e-3),
             "ms_per_step_grads_in_place": msi, "tokens_per_s_grads_in_place": w["L"] * w["B"] / (msi * 1e-3),
+            "ms_per_step_deferred_weight_grads": msd,
+            "tokens_per_s_deferred_weight_grads": w["L"] * w["B"] / (msd * 1e-3),
             "what": "ModelParallelTransformerLayer.forward per slice under the reference's own loop and autograd "
                     "(terapipe.py:249-264, :182-191): per-slice parameter-gradient GEMMs, gradient caches, one stream, "
                     "every launch issued from Python; grads_in_place: with accumulate_grads_in_place=True, the "
-                    "slices after the first add their parameter gradients to .grad inside the gradient kernels"}
+                    "slices after the first add their parameter gradients to .grad inside the gradient kernels; "
+                    "deferred_weight_grads: with defer_weight_grads=True, a sequence's weight gradients are taken once, "
+                    "in the backward of its first slice, over all its rows"}
     if args.no_roofline:
         return res, (layers, runner, x, R)
 
@@ -680,6 +686,8 @@ def main():
                          "--steps steps after --warmup and print its line: the run to put under a kernel trace")
     ap.add_argument("--grads-in-place", action="store_true",
                     help="with --layer-surface-only: set accumulate_grads_in_place on the layers")
+    ap.add_argument("--defer-weight-grads", action="store_true",
+                    help="with --layer-surface-only: set defer_weight_grads on the layers")
     ap.add_argument("--no-box-constants", action="store_true",
                     help="leave out the measured copy bandwidth and 8192^3 GEMM rate of this box")
     ap.add_argument("--no-vendor-gemm", action="store_true",
@@ -736,9 +744,11 @@ def main():
     if args.layer_surface_only:
         layers, runner, x, R = build_model(w, device)
         del runner
-        ms = timed_steps(lambda: layer_surface_step(layers, x, R, w, args.grads_in_place), args.warmup, args.steps)
+        ms = timed_steps(lambda: layer_surface_step(layers, x, R, w, args.grads_in_place, args.defer_weight_grads),
+                         args.warmup, args.steps)
         print(json.dumps({"workload": "%s: %s" % (args.workload, w["desc"]), "layer_surface_ms_per_step": ms,
                           "accumulate_grads_in_place": args.grads_in_place,
+                          "defer_weight_grads": args.defer_weight_grads,
                           "tokens_per_s": w["L"] * w["B"] / (ms * 1e-3), "steps": args.steps, "warmup": args.warmup}))
         return
     if args.copy_calibration:

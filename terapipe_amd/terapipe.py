@@ -33,11 +33,12 @@ def uniform_slice(length, n_slices):
 class TransformerLayers(nn.Module):
     """Reference terapipe.py:52-95.  mixed_precision selects fp16 as the reference does
     (``layer.half()``, terapipe.py:67); ``dtype`` overrides it (bf16 for the 175B/44B shapes).
-    accumulate_grads_in_place: see TransformerLayer.accumulate_grads_in_place (layer-level surface only; the
-    fused runner takes its parameter gradients once per step either way)."""
+    accumulate_grads_in_place, defer_weight_grads: see TransformerLayer (layer-level surface only; the fused
+    runner takes its parameter gradients once per step either way)."""
 
     def __init__(self, n_layers, embedding_dim, ffn_embedding_dim, num_attention_heads, mixed_precision=True,
-                 dtype=None, device="cuda", activation="relu", accumulate_grads_in_place=False):
+                 dtype=None, device="cuda", activation="relu", accumulate_grads_in_place=False,
+                 defer_weight_grads=False):
         super().__init__()
         self.n_layers = n_layers
         self.embedding_dim = embedding_dim
@@ -51,6 +52,7 @@ class TransformerLayers(nn.Module):
             layer = ModelParallelTransformerLayer(embedding_dim, ffn_embedding_dim, num_attention_heads,
                                                   device=device, activation=activation)
             layer.accumulate_grads_in_place = accumulate_grads_in_place
+            layer.defer_weight_grads = defer_weight_grads
             layers.append(layer.to(self.dtype))
         self.layers = nn.ModuleList(layers)
 

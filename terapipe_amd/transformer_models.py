@@ -186,18 +186,44 @@ def _grads_can_go_in_place(w):
     return True
 
 
+class _GradOptions:
+    """How a layer's backward hands its parameter gradients to autograd (TransformerLayer's two switches) and,
+    for deferred weight gradients, the sequences whose backward is under way (keyed by their K cache)."""
+    __slots__ = ("in_place", "defer", "pending")
+
+    def __init__(self):
+        self.in_place, self.defer, self.pending = False, False, {}
+
+
+class _PendingGrads:
+    """Deferred weight gradients of one sequence in one layer: the output gradients and inputs of the four
+    linears for every position whose slice has run its backward (rows [low, rows); the reverse-slice order
+    fills them from the end), and the fp32 sums of the vector-parameter gradients so far."""
+    __slots__ = ("rows", "low", "dqkv", "dh", "dz1", "dout", "xn", "o", "hn", "a", "acc")
+
+    def __init__(self, rows, E, F, dtype, device):
+        new = lambda n: torch.empty(rows, n, dtype=dtype, device=device)
+        self.rows = self.low = rows
+        self.dqkv, self.dh, self.dz1, self.dout = new(3 * E), new(E), new(F), new(E)
+        self.xn, self.o, self.hn, self.a = new(E), new(E), new(E), new(F)
+        self.acc = torch.zeros(core.small_acc_numel(E, F), dtype=torch.float32, device=device)
+
+
 class _LayerFunction(torch.autograd.Function):
     """One whole layer over one slice.  Inputs: x, k_cache, v_cache (or None, None), then the 12
     parameters in core.PARAM_NAMES order.  Outputs: out, and the two caches when given.
 
-    Backward of a slice: the data gradients (core.layer_bwd), then the four weight gradients of the slice as one
-    grouped library call and its eight vector-parameter gradients as one launch.  grads_in_place: where every
-    parameter already has a .grad, add this slice's gradients to it inside those launches (the GEMM's accumulate
-    epilogue, one rounding) and hand autograd None for them, instead of returning twelve tensors that autograd
-    adds to .grad one elementwise kernel each."""
+    Backward of a slice: the data gradients (core.layer_bwd), then the four weight gradients as one grouped
+    library call and the eight vector-parameter gradients as one launch.  opts (_GradOptions):
+    in_place -- where every parameter already has a .grad, add the gradients to it inside those launches (the
+    GEMM's accumulate epilogue, one rounding) and hand autograd None, instead of returning twelve tensors that
+    autograd adds to .grad one elementwise kernel each;
+    defer -- keep the slice's dY / X rows and take the weight gradients once per sequence, over all its rows, in
+    the backward of the slice at position 0 (the last one the reverse-slice order reaches); the slices before
+    it hand autograd None for the parameters."""
 
     @staticmethod
-    def forward(ctx, heads, cache_len, activation, grads_in_place, x, k_cache, v_cache, *params):
+    def forward(ctx, heads, cache_len, activation, opts, x, k_cache, v_cache, *params):
         w = dict(zip(core.PARAM_NAMES, params))
         T, B, E = x.shape
         Dh = E // heads
@@ -206,7 +232,7 @@ class _LayerFunction(torch.autograd.Function):
             k_cache, v_cache = _temp_cache(B, heads, T, Dh, x)
         out, st = core.layer_fwd(w, x.contiguous(), heads, k_cache, v_cache, cache_len, activation)
         ctx.st, ctx.w, ctx.heads, ctx.activation = st, w, heads, activation
-        ctx.grads_in_place = bool(grads_in_place)
+        ctx.opts = opts
         ctx.set_materialize_grads(False)
         if ctx.has_cache:
             # the caches were written through their raw pointers (as `cache.data[index] = value` does,
@@ -216,7 +242,7 @@ class _LayerFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, dk_out=None, dv_out=None):
-        st, w, heads = ctx.st, ctx.w, ctx.heads
+        st, w, heads, opts = ctx.st, ctx.w, ctx.heads, ctx.opts
         E = st.x.shape[1]
         F = w["fc1.weight"].shape[0]
         if dout is None:
@@ -234,18 +260,24 @@ class _LayerFunction(torch.autograd.Function):
         dout = dout.contiguous()
         dout2d = dout.view(M, E)
         new = lambda n: torch.empty(M, n, dtype=dt, device=dev)
-        buf = core.Bufs(dz1=new(F), dhn=new(E), dh=new(E), dqkv=new(3 * E), dxn=new(E))
+        pend = None
+        if opts.defer and ctx.has_cache:
+            # rows [r0, r1) of the sequence's position-indexed gradient buffers
+            r0, r1 = st.cache_len * st.B, (st.cache_len + st.T) * st.B
+            key = st.k_cache.data_ptr()
+            pend = opts.pending.get(key)
+            if pend is None or pend.low != r1:
+                # the last slice of a sequence opens it (an entry that does not end where this slice begins
+                # belongs to a sequence whose backward was abandoned)
+                pend = opts.pending[key] = _PendingGrads(r1, E, F, dt, dev)
+            buf = core.Bufs(dz1=pend.dz1[r0:r1], dhn=new(E), dh=pend.dh[r0:r1], dqkv=pend.dqkv[r0:r1], dxn=new(E))
+        else:
+            buf = core.Bufs(dz1=new(F), dhn=new(E), dh=new(E), dqkv=new(3 * E), dxn=new(E))
         dx = core.layer_bwd(w, st, dout, heads, gk, gv, None, False, None,
                             accumulate_prefix=True, has_incoming=has_incoming, zero_slice_rows=has_incoming,
                             activation=ctx.activation, buf=buf)
-        in_place = ctx.grads_in_place and _grads_can_go_in_place(w)
-        epi = TP_EPI_ACCUMULATE if in_place else TP_EPI_STORE
-        wgrad = {n: (w[n].grad if in_place else torch.empty_like(w[n])) for n in core.BIG_PARAMS}
-        ops.gemm_grouped([(TP_GEMM_TN, buf.dqkv, st.xn, 3 * E, E, M, wgrad["attn.in_proj.weight"], epi),
-                          (TP_GEMM_TN, buf.dh, st.o.view(M, E), E, E, M, wgrad["attn.out_proj.weight"], epi),
-                          (TP_GEMM_TN, buf.dz1, st.hn, F, E, M, wgrad["fc1.weight"], epi),
-                          (TP_GEMM_TN, dout2d, st.a, E, F, M, wgrad["fc2.weight"], epi)])
-        acc = torch.zeros(core.small_acc_numel(E, F), dtype=torch.float32, device=dev)
+        acc = pend.acc if pend is not None else torch.zeros(core.small_acc_numel(E, F), dtype=torch.float32,
+                                                            device=dev)
         sv = core.small_acc_views(acc, E, F)
         ops.vec_param_grads([(buf.dqkv, sv["attn.in_proj.bias"]),
                              (buf.dh, sv["attn.out_proj.bias"]),
@@ -253,17 +285,38 @@ class _LayerFunction(torch.autograd.Function):
                              (dout2d, sv["fc2.bias"]),
                              (buf.dxn, st.x, st.mean1, st.rstd1, sv["attn_ln.weight"], sv["attn_ln.bias"]),
                              (buf.dhn, st.h, st.mean2, st.rstd2, sv["fc_ln.weight"], sv["fc_ln.bias"])])
+        ctx.st = None
+        no_param_grads = (None, None, None, None, dx, gk, gv) + (None,) * len(core.PARAM_NAMES)
+        if pend is not None:
+            pend.dout[r0:r1].copy_(dout2d)
+            pend.xn[r0:r1].copy_(st.xn)
+            pend.o[r0:r1].copy_(st.o.view(M, E))
+            pend.hn[r0:r1].copy_(st.hn)
+            pend.a[r0:r1].copy_(st.a)
+            pend.low = r0
+            if r0 > 0:
+                return no_param_grads
+            del opts.pending[key]
+            K = pend.rows
+            pairs = ((pend.dqkv, pend.xn), (pend.dh, pend.o), (pend.dz1, pend.hn), (pend.dout, pend.a))
+        else:
+            K = M
+            pairs = ((buf.dqkv, st.xn), (buf.dh, st.o.view(M, E)), (buf.dz1, st.hn), (dout2d, st.a))
+        in_place = opts.in_place and _grads_can_go_in_place(w)
+        epi = TP_EPI_ACCUMULATE if in_place else TP_EPI_STORE
+        wgrad = {n: (w[n].grad if in_place else torch.empty_like(w[n])) for n in core.BIG_PARAMS}
+        ops.gemm_grouped([(TP_GEMM_TN, dy, xin, wgrad[n].shape[0], wgrad[n].shape[1], K, wgrad[n], epi)
+                          for n, (dy, xin) in zip(("attn.in_proj.weight", "attn.out_proj.weight", "fc1.weight",
+                                                   "fc2.weight"), pairs)])
         if in_place:
             for n in core.SMALL_PARAMS:
                 ops.accum_cast(w[n].grad, sv[n], True)
-            grads = dict.fromkeys(core.PARAM_NAMES)
-        else:
-            flat = torch.empty(acc.numel(), dtype=dt, device=dev)
-            ops.accum_cast(flat, acc, False)
-            grads = core.small_acc_views(flat, E, F)
-            grads.update(wgrad)
-        ctx.st = None
-        return (None, None, None, None, dx, gk, gv) + tuple(grads[n] for n in core.PARAM_NAMES)
+            return no_param_grads
+        flat = torch.empty(acc.numel(), dtype=dt, device=dev)
+        ops.accum_cast(flat, acc, False)
+        grads = core.small_acc_views(flat, E, F)
+        grads.update(wgrad)
+        return no_param_grads[:7] + tuple(grads[n] for n in core.PARAM_NAMES)
 
 
 class _AttentionFunction(torch.autograd.Function):
@@ -374,17 +427,22 @@ class TransformerLayer(nn.Module):
     """Reference transformer_models.py:264-285: pre-LN block with a ReLU MLP.  (The reference's plain
     class omits `checkpoint_gradients` and cannot run; here it defaults to False.)"""
 
-    # Set True (per instance or on the class) to have the backward of a slice add its parameter gradients to
-    # existing .grad tensors inside the gradient kernels instead of returning them to autograd.  Same sums with one
-    # rounding fewer; only for loops that call .backward() / autograd.backward (as the reference's does):
-    # torch.autograd.grad would see None for the parameters, and post-accumulate-grad hooks do not fire.
+    # Two switches for loops that call .backward() / autograd.backward slice by slice, as the reference's does
+    # (torch.autograd.grad would see None for the parameters, and post-accumulate-grad hooks may not fire):
+    # accumulate_grads_in_place -- the backward of a slice adds its parameter gradients to existing .grad tensors
+    # inside the gradient kernels instead of returning them to autograd (same sums, one rounding fewer);
+    # defer_weight_grads -- with a cache, the weight gradients of a sequence are taken once, over all its rows, in
+    # the backward of the slice at cache_len 0, which the reverse-slice order reaches last; .grad is complete when
+    # that backward returns, and every slice of the sequence must run its backward, last slice first.
     accumulate_grads_in_place = False
+    defer_weight_grads = False
 
     def __init__(self, embedding_dim, ffn_embedding_dim, num_attention_heads, device="cpu",
                  checkpoint_gradients=False, activation="relu"):
         super().__init__()
         self.checkpoint_gradients = checkpoint_gradients
         self.activation = activation
+        self._grad_options = _GradOptions()
         self.attn_ln = nn.LayerNorm(embedding_dim).to(device)
         self.attn = MultiheadLMAttentionWithCache(embedding_dim, num_attention_heads, device=device)
         self.fc_ln = nn.LayerNorm(embedding_dim).to(device)
@@ -409,7 +467,9 @@ class TransformerLayer(nn.Module):
         else:
             assert cache_len == 0
         p = self.param_dict()
-        res = _LayerFunction.apply(self.attn.num_heads, cache_len, self.activation, self.accumulate_grads_in_place,
+        opts = self._grad_options
+        opts.in_place, opts.defer = bool(self.accumulate_grads_in_place), bool(self.defer_weight_grads)
+        res = _LayerFunction.apply(self.attn.num_heads, cache_len, self.activation, opts,
                                    x, k, v, *[p[n] for n in core.PARAM_NAMES])
         if full_cache is not None:
             return res[0], (res[1], res[2])

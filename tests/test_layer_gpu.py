@@ -227,12 +227,14 @@ def _reference_style_loop(layers, x, dy, batch_slices, seq_slices):
     return y, dx, finals, cg
 
 
-@pytest.mark.parametrize("in_place", [False, True], ids=["autograd-accumulates", "grads-in-place"])
+@pytest.mark.parametrize("in_place,defer", [(False, False), (True, False), (False, True), (True, True)],
+                         ids=["autograd-accumulates", "grads-in-place", "deferred", "deferred-in-place"])
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
-def test_reference_style_slice_loop(dtype, in_place):
+def test_reference_style_slice_loop(dtype, in_place, defer):
     """Layer-level autograd contract: detach()/requires_grad_() caches per slice, backward with the
     cache-output gradients of the next slice, cache-input .grad as hand-off.  in_place: the slices after the
-    first add their parameter gradients to .grad inside the gradient kernels (accumulate_grads_in_place)."""
+    first add their parameter gradients to .grad inside the gradient kernels (accumulate_grads_in_place);
+    defer: a sequence's weight gradients are taken once, in the backward of its first slice (defer_weight_grads)."""
     ta = _mods()
     n_layers, E, H, L, B = 2, 256, 4, 64, 2
     Fd = 4 * E
@@ -248,7 +250,7 @@ def test_reference_style_slice_loop(dtype, in_place):
                                                          return_cache_grads=True, activation=act)
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps, act)
     for layer in layers.layers:
-        layer.accumulate_grads_in_place = in_place
+        layer.accumulate_grads_in_place, layer.defer_weight_grads = in_place, defer
     y, dx, finals, cg = _reference_style_loop(layers, x.to(DEV), dy.to(DEV), bs, ss)
     assert_close(y, yo, dtype, "y")
     assert_close(dx, dxo, dtype, "dx")
@@ -262,9 +264,10 @@ def test_reference_style_slice_loop(dtype, in_place):
     _check_param_grads(_param_grads(layers), [{k: v.grad for k, v in p.items()} for p in leaf], dtype, "ref loop")
 
 
-@pytest.mark.parametrize("in_place", [False, True], ids=["autograd-accumulates", "grads-in-place"])
+@pytest.mark.parametrize("in_place,defer", [(False, False), (True, False), (False, True), (True, True)],
+                         ids=["autograd-accumulates", "grads-in-place", "deferred", "deferred-in-place"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
-def test_reference_style_slice_loop_on_64_row_multiples(dtype, in_place):
+def test_reference_style_slice_loop_on_64_row_multiples(dtype, in_place, defer):
     """The same loop on slices of 128 / 64 / 192 tokens at hidden 512: a slice's four weight gradients meet
     the conditions of the grouped launch (k a multiple of 64), with the store and the accumulate epilogue."""
     ta = _mods()
@@ -279,7 +282,7 @@ def test_reference_style_slice_loop_on_64_row_multiples(dtype, in_place):
                                                          return_cache_grads=True, activation="gelu")
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps, "gelu")
     for layer in layers.layers:
-        layer.accumulate_grads_in_place = in_place
+        layer.accumulate_grads_in_place, layer.defer_weight_grads = in_place, defer
     y, dx, finals, cg = _reference_style_loop(layers, x.to(DEV), dy.to(DEV), bs, ss)
     assert_close(y, yo, dtype, "y")
     assert_close(dx, dxo, dtype, "dx")
