@@ -17,7 +17,7 @@ import pytest
 import torch
 
 import oracle
-from tests.util import assert_close, load_params_into
+from tests.util import assert_close, load_params_into, reference_style_loop
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -117,6 +117,42 @@ def test_full_width_against_the_oracle(name, streams):
     frac = _check_active_sets(name, masks, preacts)
     print("  ReLU decisions that differ from the oracle's: %.2e of all units" % frac, flush=True)
     _compare_step(name, "eager", runner, layers, y, xd, yo, dxo, fco, leaf, dtype)
+
+
+@pytest.mark.parametrize("in_place,defer", [(False, False), (True, True)], ids=["autograd-accumulates", "deferred-in-place"])
+def test_full_width_layer_surface_against_the_oracle(in_place, defer):
+    """Config 3's width and slice list through the LAYER-LEVEL surface under the reference's own loop (one
+    autograd graph per slice, cache-gradient hand-off through gradient caches), two steps so that the second
+    finds .grad tensors to add to: with per-slice parameter gradients handed to autograd, and with a sequence's
+    weight gradients deferred to the backward of its first slice and added to .grad inside the kernels.  The smooth
+    activation keeps 16-bit sign flips of the ReLU out of the bound (this surface does not expose its active set)."""
+    import terapipe_amd as ta
+    n_layers, E, H, Fd, L, B, dtype, ss, std = FULL_WIDTH["C3"]
+    print("layer-level surface at C3's width: in_place=%s defer=%s" % (in_place, defer), flush=True)
+    ps = _params(n_layers, E, Fd, dtype, std, seed=59)
+    g = torch.Generator().manual_seed(61)
+    x = torch.randn(L, B, E, generator=g).to(dtype)
+    dy = torch.randn(L, B, E, generator=g).to(dtype)
+    layers = ta.TransformerLayers(n_layers, E, Fd, H, dtype=dtype, device=DEV, activation="gelu",
+                                  accumulate_grads_in_place=in_place, defer_weight_grads=defer)
+    load_params_into(layers, ps, dtype)
+    for step in (1, 2):
+        y, dx, finals, cg = reference_style_loop(layers, x.to(DEV), dy.to(DEV), [B], ss)
+    torch.cuda.synchronize()
+    leaf = [{k: v.clone().requires_grad_(True) for k, v in p.items()} for p in ps]
+    yo, dxo, fco, cgo = oracle.terapipe_forward_backward(leaf, x.float(), dy.float(), H, [B], ss,
+                                                         return_cache_grads=True, activation="gelu")
+    assert_close(y, yo, dtype, "y")
+    assert_close(dx, dxo, dtype, "dx")
+    for j in range(2 * n_layers):
+        assert_close(finals[0][j], fco[0][j], dtype, "final cache %d" % j)
+        for i in range(1, len(ss)):
+            assert_close(cg[0][i][j], cgo[0][i][j], dtype, "cache grad slice %d tensor %d" % (i, j))
+    for l, (layer, p) in enumerate(zip(layers.layers, leaf)):
+        for n, t in layer.param_dict().items():
+            # two identical steps accumulated into .grad
+            assert_close(t.grad, 2.0 * p[n].grad, dtype, "layer %d d(%s) over two steps" % (l, n))
+    assert all(not layer._grad_options.pending for layer in layers.layers), "a deferred sequence was left open"
 
 
 @pytest.mark.parametrize("name", ["C4-full", "C5-full"])

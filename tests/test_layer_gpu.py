@@ -18,7 +18,7 @@ import torch
 import torch.nn.functional as F
 
 import oracle
-from tests.util import TOL, assert_close, load_params_into, make_params, oracle_run, rel_err
+from tests.util import TOL, assert_close, load_params_into, make_params, oracle_run, reference_style_loop, rel_err
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -194,39 +194,6 @@ def test_attention_module_without_bias(dtype):
     assert_close(attn.out_proj.weight.grad, p32["attn.out_proj.weight"].grad, dtype, "d out_proj.weight")
 
 
-def _reference_style_loop(layers, x, dy, batch_slices, seq_slices):
-    """The slice loop of the reference's TeraPipe.forward + TeraPipeBackwardPassHook.backward
-    (terapipe.py:249-264, :182-191) driven through the layer-level autograd surface."""
-    ta = _mods()
-    xs = ta.grid_slice_batch_and_sequence(x, batch_slices, seq_slices, requires_grad=True)
-    dys = ta.grid_slice_batch_and_sequence(dy, batch_slices, seq_slices)
-    nb, ns = len(batch_slices), len(seq_slices)
-    cache_inputs = np.empty((nb, ns), dtype="O")
-    cache_outputs = np.empty((nb, ns), dtype="O")
-    outputs = np.empty((nb, ns), dtype="O")
-    finals = []
-    for b in range(nb):
-        cache = layers.create_cache(batch_slices[b], x.size(0))
-        cache_len = 0
-        for i in range(ns):
-            cache = [c.detach().requires_grad_() for c in cache]
-            y, cache_out = layers(xs[b, i], cache, cache_len)
-            cache_inputs[b, i], cache_outputs[b, i], outputs[b, i] = cache, cache_out, y
-            cache = cache_out
-            cache_len += seq_slices[i]
-        finals.append([c.detach() for c in cache])
-    for b in reversed(range(nb)):
-        da = []
-        for i in reversed(range(ns)):
-            a = list(cache_outputs[b, i]) if i < ns - 1 else []
-            torch.autograd.backward([outputs[b, i]] + a, [dys[b, i]] + da)
-            da = [t.grad for t in cache_inputs[b, i]]
-    y = torch.cat([torch.cat(list(outputs[b]), 0) for b in range(nb)], 1).detach()
-    dx = torch.cat([torch.cat([xs[b, i].grad for i in range(ns)], 0) for b in range(nb)], 1)
-    cg = [[[t.grad for t in cache_inputs[b, i]] for i in range(ns)] for b in range(nb)]
-    return y, dx, finals, cg
-
-
 @pytest.mark.parametrize("in_place,defer", [(False, False), (True, False), (False, True), (True, True)],
                          ids=["autograd-accumulates", "grads-in-place", "deferred", "deferred-in-place"])
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
@@ -251,7 +218,7 @@ def test_reference_style_slice_loop(dtype, in_place, defer):
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps, act)
     for layer in layers.layers:
         layer.accumulate_grads_in_place, layer.defer_weight_grads = in_place, defer
-    y, dx, finals, cg = _reference_style_loop(layers, x.to(DEV), dy.to(DEV), bs, ss)
+    y, dx, finals, cg = reference_style_loop(layers, x.to(DEV), dy.to(DEV), bs, ss)
     assert_close(y, yo, dtype, "y")
     assert_close(dx, dxo, dtype, "dx")
     for b in range(len(bs)):
@@ -283,7 +250,7 @@ def test_reference_style_slice_loop_on_64_row_multiples(dtype, in_place, defer):
     layers = _build_layers(ta, n_layers, E, Fd, H, dtype, ps, "gelu")
     for layer in layers.layers:
         layer.accumulate_grads_in_place, layer.defer_weight_grads = in_place, defer
-    y, dx, finals, cg = _reference_style_loop(layers, x.to(DEV), dy.to(DEV), bs, ss)
+    y, dx, finals, cg = reference_style_loop(layers, x.to(DEV), dy.to(DEV), bs, ss)
     assert_close(y, yo, dtype, "y")
     assert_close(dx, dxo, dtype, "dx")
     _check_param_grads(_param_grads(layers), [{k: v.grad for k, v in p.items()} for p in leaf], dtype, "ref loop")

@@ -1,4 +1,5 @@
 """Helpers shared by the GPU parity tests."""
+import numpy as np
 import torch
 
 import oracle
@@ -56,3 +57,36 @@ def oracle_run(ps, x, dy, heads, batch_slices, seq_slices, dtype64=False):
     y, dx, caches = oracle.terapipe_forward_backward(leaf, x.to(dt), dy.to(dt), heads, batch_slices, seq_slices)
     grads = [{k: v.grad for k, v in p.items()} for p in leaf]
     return y, dx, caches, grads
+
+
+def reference_style_loop(layers, x, dy, batch_slices, seq_slices):
+    """The slice loop of the reference's TeraPipe.forward + TeraPipeBackwardPassHook.backward
+    (terapipe.py:249-264, :182-191) driven through the layer-level autograd surface."""
+    import terapipe_amd as ta
+    xs = ta.grid_slice_batch_and_sequence(x, batch_slices, seq_slices, requires_grad=True)
+    dys = ta.grid_slice_batch_and_sequence(dy, batch_slices, seq_slices)
+    nb, ns = len(batch_slices), len(seq_slices)
+    cache_inputs = np.empty((nb, ns), dtype="O")
+    cache_outputs = np.empty((nb, ns), dtype="O")
+    outputs = np.empty((nb, ns), dtype="O")
+    finals = []
+    for b in range(nb):
+        cache = layers.create_cache(batch_slices[b], x.size(0))
+        cache_len = 0
+        for i in range(ns):
+            cache = [c.detach().requires_grad_() for c in cache]
+            y, cache_out = layers(xs[b, i], cache, cache_len)
+            cache_inputs[b, i], cache_outputs[b, i], outputs[b, i] = cache, cache_out, y
+            cache = cache_out
+            cache_len += seq_slices[i]
+        finals.append([c.detach() for c in cache])
+    for b in reversed(range(nb)):
+        da = []
+        for i in reversed(range(ns)):
+            a = list(cache_outputs[b, i]) if i < ns - 1 else []
+            torch.autograd.backward([outputs[b, i]] + a, [dys[b, i]] + da)
+            da = [t.grad for t in cache_inputs[b, i]]
+    y = torch.cat([torch.cat(list(outputs[b]), 0) for b in range(nb)], 1).detach()
+    dx = torch.cat([torch.cat([xs[b, i].grad for i in range(ns)], 0) for b in range(nb)], 1)
+    cg = [[[t.grad for t in cache_inputs[b, i]] for i in range(ns)] for b in range(nb)]
+    return y, dx, finals, cg
