@@ -7,8 +7,8 @@ libterapipe_hip.so through terapipe_amd.ops.
 import torch
 
 from . import ops
-from ._lib import (TP_EPI_ACCUMULATE, TP_EPI_BIAS_GELU, TP_EPI_BIAS_RELU, TP_EPI_BIAS_RESIDUAL, TP_EPI_GELU_GRAD,
-                   TP_EPI_QKV_SCATTER, TP_EPI_RELU_GRAD, TP_EPI_STORE, TP_GEMM_NN, TP_GEMM_NT, TP_GEMM_TN)
+from ._lib import (TP_EPI_BIAS_GELU, TP_EPI_BIAS_RELU, TP_EPI_BIAS_RESIDUAL, TP_EPI_GELU_GRAD, TP_EPI_QKV_SCATTER,
+                   TP_EPI_RELU_GRAD, TP_GEMM_NN, TP_GEMM_NT)
 
 # order of the small (vector) parameters inside one layer's fp32 gradient accumulator
 SMALL_PARAMS = ("attn_ln.weight", "attn_ln.bias", "attn.in_proj.bias", "attn.out_proj.bias",
@@ -137,20 +137,14 @@ def layer_fwd(w, x, heads, k_cache, v_cache, cache_len, activation="relu", need_
     return out.view(T, B, E), st
 
 
-def _wgrad(target, accumulate, A, Bm, M_, N_, K_):
-    """target[M_, N_] (+)= A[K_, M_]^T . Bm[K_, N_]"""
-    ops.gemm(TP_GEMM_TN, A, Bm, M_, N_, K_, C=target, epilogue=TP_EPI_ACCUMULATE if accumulate else TP_EPI_STORE)
+def layer_bwd(w, st, dout, heads, gk, gv, accumulate_prefix, has_incoming, zero_slice_rows, activation="relu",
+              buf=_NOBUF, suffix=None):
+    """Backward of layer_fwd for one slice: the data gradients.
 
-
-def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, accumulate_prefix, has_incoming,
-              zero_slice_rows, activation="relu", buf=_NOBUF, suffix=None):
-    """Backward of layer_fwd for one slice.
-
-    dout [T, B, E]; gk / gv gradient caches (see tp_attn_desc).  wgrad maps the four weight names to
-    gradient tensors that are overwritten (accumulate_wgrad False) or added to; small_acc maps the vector
-    parameter names to fp32 accumulators that are added to.  With wgrad None / small_acc None the weight
-    / vector-parameter gradients of this slice are NOT computed: the caller keeps the intermediate
-    gradients this call leaves in `buf` (dz1, dhn, dh, dqkv, dxn) and reduces over all slices at once.
+    dout [T, B, E]; gk / gv gradient caches (see tp_attn_desc).  The parameter gradients are the caller's: it
+    keeps the intermediate gradients this call leaves in `buf` (dz1, dhn, dh, dqkv, dxn; dout is fc2's) and
+    reduces them against the saved inputs -- per slice (the layer-level surface) or over all slices of a step at
+    once (the runner): four TN products and eight column reductions (ops.gemm_grouped, ops.vec_param_grads).
     suffix: None, or dict(q_all, d_o_all, lse_all, delta_all, q_end) of position-indexed buffers that hold
     every slice processed so far (buf.d_o and buf.delta are then views of them at this slice): dK/dV of
     the slice's keys are computed in one pass over all later query positions and gk / gv are not used.
@@ -164,34 +158,25 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
     Dh = E // heads
     dt, dev = dout.dtype, dout.device
     dout2d = dout.reshape(M, E)
-    sa = small_acc if small_acc is not None else {}
     # MLP
     dz1 = _buf(buf.dz1, (M, F), dt, dev)
     if activation == "relu":
-        ops.gemm(TP_GEMM_NN, dout2d, w["fc2.weight"], M, F, E, C=dz1, epilogue=TP_EPI_RELU_GRAD, aux=st.a,
-                 colsum_acc=sa.get("fc1.bias"))
+        ops.gemm(TP_GEMM_NN, dout2d, w["fc2.weight"], M, F, E, C=dz1, epilogue=TP_EPI_RELU_GRAD, aux=st.a)
     else:
-        ops.gemm(TP_GEMM_NN, dout2d, w["fc2.weight"], M, F, E, C=dz1, epilogue=TP_EPI_GELU_GRAD, aux=st.z,
-                 colsum_acc=sa.get("fc1.bias"))
-    if wgrad is not None:
-        _wgrad(wgrad["fc2.weight"], accumulate_wgrad, dout2d, st.a, E, F, M)
+        ops.gemm(TP_GEMM_NN, dout2d, w["fc2.weight"], M, F, E, C=dz1, epilogue=TP_EPI_GELU_GRAD, aux=st.z)
     dhn = _buf(buf.dhn, (M, E), dt, dev)
-    if wgrad is not None:
-        _wgrad(wgrad["fc1.weight"], accumulate_wgrad, dz1, st.hn, F, E, M)
     # a k-split data-gradient GEMM leaves its partial sums to the LayerNorm backward that follows directly
     dhn_in = ops.gemm(TP_GEMM_NN, dz1, w["fc1.weight"], M, E, F, C=dhn, defer_reduce=True)
-    dh = ops.layernorm_bwd(dhn_in, st.h, st.mean2, st.rstd2, w["fc_ln.weight"], dout2d, sa.get("fc_ln.weight"),
-                           sa.get("fc_ln.bias"), sa.get("fc2.bias"), sa.get("attn.out_proj.bias"), out=buf.dh)
+    dh = ops.layernorm_bwd(dhn_in, st.h, st.mean2, st.rstd2, w["fc_ln.weight"], dout2d, None, None, None, None,
+                           out=buf.dh)
     # attention
     d_o = _buf(buf.d_o, (M, E), dt, dev)
     ops.gemm(TP_GEMM_NN, dh, w["attn.out_proj.weight"], M, E, E, C=d_o)
-    if wgrad is not None:
-        _wgrad(wgrad["attn.out_proj.weight"], accumulate_wgrad, dh, st.o, E, E, M)
     dqkv = _buf(buf.dqkv, (M, 3 * E), dt, dev)
     if suffix is None:
         ops.attn_prefix_bwd(st.q, st.k_cache, st.v_cache, st.o, st.lse, d_o, dqkv, gk, gv, B, heads, Dh, T,
                             st.cache_len, float(Dh) ** -0.5, accumulate_prefix, has_incoming, zero_slice_rows,
-                            colsum_dqkv_acc=sa.get("attn.in_proj.bias"), delta=buf.delta,
+                            delta=buf.delta,
                             q_bh_rows=st.q_bh_rows, stat_bh_rows=st.stat_bh_rows)
     elif suffix.get("fused"):
         # dQ of the slice and dK / dV of its keys over all later positions as one launch.  The dK/dV half takes delta
@@ -205,8 +190,6 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
                            float(Dh) ** -0.5, buf.delta, suffix["q_all"], suffix["d_o_all"], suffix["lse_all"],
                            suffix["delta_all"], suffix["o_all"], suffix["q_end"], suffix["own_end"],
                            q_bh_rows=st.q_bh_rows, stat_bh_rows=st.stat_bh_rows)
-        if "attn.in_proj.bias" in sa:
-            ops.colsum_acc(dqkv, sa["attn.in_proj.bias"])
     else:
         ops.attn_prefix_bwd(st.q, st.k_cache, st.v_cache, st.o, st.lse, d_o, dqkv, None, None, B, heads, Dh, T,
                             st.cache_len, float(Dh) ** -0.5, False, False, False, delta=buf.delta,
@@ -215,12 +198,8 @@ def layer_bwd(w, st, dout, heads, gk, gv, wgrad, accumulate_wgrad, small_acc, ac
             buf.sync()
         ops.attn_suffix_dkdv(st.k_cache, st.v_cache, suffix["q_all"], suffix["d_o_all"], suffix["lse_all"],
                              suffix["delta_all"], dqkv, B, heads, Dh, st.cache_len, T, suffix["q_end"])
-        if "attn.in_proj.bias" in sa:
-            ops.colsum_acc(dqkv, sa["attn.in_proj.bias"])
     dxn = _buf(buf.dxn, (M, E), dt, dev)
-    if wgrad is not None:
-        _wgrad(wgrad["attn.in_proj.weight"], accumulate_wgrad, dqkv, st.xn, 3 * E, E, M)
     dxn_in = ops.gemm(TP_GEMM_NN, dqkv, w["attn.in_proj.weight"], M, E, 3 * E, C=dxn, defer_reduce=True)
-    dx = ops.layernorm_bwd(dxn_in, st.x, st.mean1, st.rstd1, w["attn_ln.weight"], dh, sa.get("attn_ln.weight"),
-                           sa.get("attn_ln.bias"), None, None, out=buf.dx)
+    dx = ops.layernorm_bwd(dxn_in, st.x, st.mean1, st.rstd1, w["attn_ln.weight"], dh, None, None, None, None,
+                           out=buf.dx)
     return dx.view(T, B, E)

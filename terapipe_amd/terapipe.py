@@ -385,7 +385,7 @@ def _backward_body(runner, ws, act, bufs, states):
                                        d_o=pb["d_o"][l][r0:r1], dqkv=pb["dqkv"][l][r0:r1], dxn=pb["dxn"][l][r0:r1],
                                        dx=pb["dx"][l][r0:r1], delta=pb["delta"][l][:, P:], sync=sync)
                         core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), H, None, None,
-                                       None, False, None, False, False, False, activation=act[l], buf=bf,
+                                       False, False, False, activation=act[l], buf=bf,
                                        suffix=dict(q_all=pb["q"][l], d_o_all=pb["d_o"][l], lse_all=pb["lse"][l],
                                                    delta_all=pb["delta"][l], q_end=L,
                                                    o_all=pb["o"][l].view(L, Bs, E) if bufs.fused_attn_bwd else None,
@@ -413,7 +413,7 @@ def _backward_body(runner, ws, act, bufs, states):
                 # the gradient caches need no zero fill: the last slice (processed first) writes every
                 # prefix row with '=', the earlier ones add to rows that were written before
                 core.layer_bwd(ws[l], states[b, i][l], pb["dx"][l + 1][r0:r1].view(T, Bs, E), H,
-                               gc[2 * l], gc[2 * l + 1], None, False, None, accumulate_prefix=not last,
+                               gc[2 * l], gc[2 * l + 1], accumulate_prefix=not last,
                                has_incoming=not last, zero_slice_rows=False, activation=act[l], buf=bf)
             if runner.slice_timing is not None:
                 runner.slice_timing["bwd"].append(_timing_event(main))

@@ -8,6 +8,8 @@ the head dimension is one of 16, 32, 64, 80, 96, 128 (every entry of MODEL_CONFI
 a separate _AssignCache op, with the same in-place, alias-returning semantics and the same gradient
 contract (reference transformer_models.py:177-193).
 """
+import warnings
+
 import numpy as np
 import torch
 import torch.nn as nn
@@ -267,15 +269,17 @@ class _LayerFunction(torch.autograd.Function):
             key = st.k_cache.data_ptr()
             pend = opts.pending.get(key)
             if pend is None or pend.low != r1:
-                # the last slice of a sequence opens it (an entry that does not end where this slice begins
-                # belongs to a sequence whose backward was abandoned)
+                # the last slice of a sequence opens it; an entry that does not end where this slice begins belongs
+                # to a sequence whose backward was abandoned or skipped a slice
+                if pend is not None and pend.low < pend.rows:
+                    warnings.warn("defer_weight_grads: the backward of a sequence stopped at row %d and never reached "
+                                  "its first slice; its weight gradients are dropped" % pend.low)
                 pend = opts.pending[key] = _PendingGrads(r1, E, F, dt, dev)
             buf = core.Bufs(dz1=pend.dz1[r0:r1], dhn=new(E), dh=pend.dh[r0:r1], dqkv=pend.dqkv[r0:r1], dxn=new(E))
         else:
             buf = core.Bufs(dz1=new(F), dhn=new(E), dh=new(E), dqkv=new(3 * E), dxn=new(E))
-        dx = core.layer_bwd(w, st, dout, heads, gk, gv, None, False, None,
-                            accumulate_prefix=True, has_incoming=has_incoming, zero_slice_rows=has_incoming,
-                            activation=ctx.activation, buf=buf)
+        dx = core.layer_bwd(w, st, dout, heads, gk, gv, accumulate_prefix=True, has_incoming=has_incoming,
+                            zero_slice_rows=has_incoming, activation=ctx.activation, buf=buf)
         acc = pend.acc if pend is not None else torch.zeros(core.small_acc_numel(E, F), dtype=torch.float32,
                                                             device=dev)
         sv = core.small_acc_views(acc, E, F)
