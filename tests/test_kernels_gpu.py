@@ -456,6 +456,57 @@ def test_attn_prefix_fwd_bwd(dtype, T, B, H, Dh, P, L):
             assert_close(acc, dqkv.double().sum(0), dtype, "dqkv colsum" + tag)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("T,B,H,Dh,P,L,drift", [(128, 1, 4, 128, 896, 1024, 0.0), (160, 1, 4, 128, 352, 512, 0.0),
+                                                (32, 2, 3, 64, 480, 512, 0.0), (128, 1, 4, 128, 896, 1024, 0.05),
+                                                (64, 2, 2, 64, 448, 512, 0.1)])
+def test_attn_peaked_and_drifting_scores(dtype, T, B, H, Dh, P, L, drift):
+    """Scores with a standard deviation near 17 (Dh 128) / 12 (Dh 64), so that a row's softmax sits on a few keys and
+    its largest score keeps being overtaken along the key range: the forward kernels take exponentials against a
+    per-row reference that moves only when a row outgrows it by e^5, and this is the input on which it moves often.
+    drift adds a ramp along the key position (later keys score higher), the order in which the reference is
+    overtaken tile after tile.  All forward forms against the fp64 restatement, and without the ramp the backward
+    too (with it the keys carry a common component of up to 50, which dQ = dS K cancels -- the rows of dS sum to
+    zero -- so that the 16-bit rounding of dS alone exceeds the bound on any implementation)."""
+    ops = _ops()
+    S, E, BH = P + T, H * Dh, B * H
+    g = torch.Generator().manual_seed(T + P + Dh)
+    q = _rnd((BH, T, Dh), dtype, g, 1.0)
+    k32 = torch.randn(BH, L, Dh, generator=g) * 1.5
+    if drift:
+        # a component along q's mean direction that grows with the key position
+        k32 = k32 + drift * torch.arange(L).view(1, L, 1) * torch.sign(q.float().mean(1, keepdim=True))
+    kc, vc = k32.to(dtype), _rnd((BH, L, Dh), dtype, g)
+    d_o = _rnd((T, B, E), dtype, g)
+    qd, kd, vd = q.to(DEV), kc.to(DEV), vc.to(DEV)
+    q64 = q.double().requires_grad_(True)
+    k64, v64 = kc.double().requires_grad_(True), vc.double().requires_grad_(True)
+    oref = _attn_ref(q64, k64, v64, B, H, T, P)
+    s = torch.bmm(q64, k64[:, :S].transpose(1, 2)) + oracle.causal_prefix_mask(T, P, torch.float64)
+    lse_ref = torch.logsumexp(s, -1)
+    o, lse = ops.attn_prefix_fwd(qd, kd, vd, B, H, Dh, T, P, 1.0)
+    assert_close(o, oref, dtype, "attn o")
+    assert_close(lse, lse_ref, torch.float32, "attn lse", 1e3)
+    for variant in (2 | 8, 4 | 8, 16):
+        o_v, lse_v = ops.attn_prefix_fwd(qd, kd, vd, B, H, Dh, T, P, 1.0, variant=variant)
+        assert_close(o_v, oref, dtype, "attn o, forward variant %d" % variant)
+        assert_close(lse_v, lse_ref, torch.float32, "attn lse, forward variant %d" % variant, 1e3)
+    if drift:
+        return
+    oref.backward(d_o.double())
+    gk = torch.zeros(BH, L, Dh, dtype=torch.float32, device=DEV)
+    gv = torch.zeros(BH, L, Dh, dtype=torch.float32, device=DEV)
+    dqkv = torch.empty(T * B, 3 * E, dtype=dtype, device=DEV)
+    ops.attn_prefix_bwd(qd, kd, vd, o, lse, d_o.to(DEV), dqkv, gk, gv, B, H, Dh, T, P, 1.0,
+                        accumulate_prefix=False, has_incoming=False, zero_slice_rows=False)
+    dq, dk, dv = oracle.split_qkv(dqkv.view(T, B, 3 * E).double().cpu(), H)
+    assert_close(dq, q64.grad, dtype, "dq")
+    assert_close(dk, k64.grad[:, P:S], dtype, "dk slice")
+    assert_close(dv, v64.grad[:, P:S], dtype, "dv slice")
+    assert_close(gk[:, :P], k64.grad[:, :P], dtype, "gk prefix")
+    assert_close(gv[:, :P], v64.grad[:, :P], dtype, "gv prefix")
+
+
 SUFFIX_CASES = [
     # B, H, Dh, L (cache rows), slices
     (2, 2, 64, 96, [32, 32, 32]),
