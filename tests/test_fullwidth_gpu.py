@@ -1,4 +1,4 @@
-"""Oracle parity at the real width of BASELINE configs 2-5: hidden size, head count, FFN size, dtype and
+"""Oracle parity at the real width of benchmark configs 2-5: hidden size, head count, FFN size, dtype and
 slice list as the configs state them, on one or two layers of the stack (the CPU oracle's time bounds the
 layer count).  test_full_width_against_the_oracle runs configs 4 and 5 on a prefix of the sequence (the first
 1024 of 2048 positions = 8 of 16 slices of 128 tokens; the first 512 = 16 of 64 slices of 32 tokens, batch 2)

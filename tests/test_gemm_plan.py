@@ -1,5 +1,5 @@
 """The GEMM plan (tile configuration + k splits) that tp_gemm picks, asked through tp_gemm_plan: host code, so these
-run without a GPU.  The measured table must give every shape of the four BASELINE geometries exactly its entry, and
+run without a GPU.  The measured table must give every shape of the four benchmark geometries exactly its entry, and
 the rules for slice GEMMs outside the table must give plans that are valid and that follow the stated principles
 (one round of workgroups when k is split, no split that leaves less than 1536 of k)."""
 import ctypes
@@ -50,7 +50,7 @@ def test_every_table_entry_is_the_plan_of_its_shape():
 
 
 def test_the_baseline_geometries_are_covered_by_exact_entries():
-    """Every 16-bit GEMM of BASELINE configs 2-5 (slice linears at each slice length, parameter gradients of a step)
+    """Every 16-bit GEMM of benchmark configs 2-5 (slice linears at each slice length, parameter gradients of a step)
     has its own entry, so that a revision of the rules cannot move a benchmark shape."""
     have = {e[:4] for e in _table()}
     geos = [(2048, 8192, [256], 2048), (5120, 20480, [512, 384, 320, 256, 224, 192, 160], 2048),

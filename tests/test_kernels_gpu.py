@@ -379,7 +379,7 @@ ATTN_CASES = [
     (7, 1, 1, 64, 5, 12),
     (1, 1, 1, 64, 0, 1),
     (64, 1, 2, 128, 0, 64),        # two waves
-    (32, 2, 48, 128, 2016, 2048),  # BASELINE config 5's last slice: 96 (batch, head) pairs, 32 queries, 2048 keys
+    (32, 2, 48, 128, 2016, 2048),  # benchmark config 5's last slice: 96 (batch, head) pairs, 32 queries, 2048 keys
     (128, 1, 96, 128, 1920, 2048), # config 4's last slice
     (160, 1, 40, 128, 1888, 2048), # config 3's last slice
     # head dimensions other than 64 and 128 (the reference's model table has 80, 96 and 16, transformer_models.py:33-49):
@@ -514,7 +514,7 @@ SUFFIX_CASES = [
     (1, 3, 128, 200, [40, 7, 100, 33]),      # ragged: nothing aligned to the 32-row blocks
     (2, 1, 64, 64, [5, 1, 20]),              # caches longer than the sequence
     (1, 2, 128, 512, [128, 128, 128, 128]),
-    (2, 48, 128, 1024, [32] * 32),                             # BASELINE config 5's heads and slices (half its length)
+    (2, 48, 128, 1024, [32] * 32),                             # benchmark config 5's heads and slices (half its length)
     (1, 96, 128, 1024, [128] * 8),                             # config 4's
     (1, 40, 128, 2048, [512, 384, 320, 256, 224, 192, 160]),   # config 3's, whole
 ]
@@ -592,7 +592,7 @@ def test_attn_position_indexed_and_suffix_dkdv(dtype, B, H, Dh, L, slices):
 def test_attn_fwd_keys_shared_by_workgroups(dtype, T, B, H, Dh, P, ns):
     """The 16-bit forward with the key range of every query block forced onto `ns` workgroups whose fp32 partials
     the merge launch weighs together -- what the plan does by itself for calls with few blocks and long key ranges
-    (BASELINE config 5's later slices in ATTN_CASES).  Shares that come out empty (more workgroups than tiles) and
+    (benchmark config 5's later slices in ATTN_CASES).  Shares that come out empty (more workgroups than tiles) and
     ragged last tiles are part of the cases.  Checked against the fp64 attention."""
     ops = _ops()
     S, E, BH = P + T, H * Dh, B * H

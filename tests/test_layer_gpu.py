@@ -271,7 +271,7 @@ def _run_terapipe(ta, layers, x, dy, B, L, bs, ss, keep_states=False, **kw):
 
 @pytest.mark.parametrize("fp32gc", [True, False])
 def test_terapipe_c1_tiny_fp32(fp32gc):
-    """BASELINE config 1 (layer stack part): 4 layers, hidden 256, 4 heads, FFN 1024, seq 128, batch 2,
+    """benchmark config 1 (layer stack part): 4 layers, hidden 256, 4 heads, FFN 1024, seq 128, batch 2,
     fp32, 8 slices of 16, reverse-slice backward, tolerance 1e-5."""
     ta = _mods()
     n_layers, E, H, Fd, L, B = 4, 256, 4, 1024, 128, 2
@@ -290,7 +290,7 @@ def test_terapipe_c1_tiny_fp32(fp32gc):
 
 
 def test_terapipe_c1_tokens_and_cross_entropy():
-    """BASELINE config 1 end to end: token ids -> embedding -> sliced stack -> LM head -> mean cross
+    """benchmark config 1 end to end: token ids -> embedding -> sliced stack -> LM head -> mean cross
     entropy on random next-token targets.  The embedding / LM head / loss are harness-owned torch ops on
     both sides; the stack between them is the HIP path vs the oracle."""
     ta = _mods()
@@ -340,7 +340,7 @@ def test_terapipe_c1_tokens_and_cross_entropy():
 
 
 def test_terapipe_c1_end_to_end_native_embedding_and_loss():
-    """BASELINE config 1 end to end with nothing but the HIP path between the token ids and the loss:
+    """benchmark config 1 end to end with nothing but the HIP path between the token ids and the loss:
     VocabParallelEmbedding -> sliced stack -> tied LM head -> vocab_parallel_cross_entropy -> mean, against
     the oracle (embedding, stack, cross-entropy restatements) in fp32 at 1e-5."""
     ta = _mods()
@@ -388,7 +388,7 @@ def test_terapipe_c1_end_to_end_native_embedding_and_loss():
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
 @pytest.mark.parametrize("case", ["uniform", "nonuniform", "fine", "batch_sliced"])
 def test_terapipe_16bit_reduced_shapes(dtype, case):
-    """Reduced-size versions of BASELINE configs 2-5 (head dim 128, N(0,1) inputs, random-projection
+    """Reduced-size versions of benchmark configs 2-5 (head dim 128, N(0,1) inputs, random-projection
     loss): uniform 256-token slices, the non-uniform DP-style slice list, 32-token slices, and a batch
     of 2 cut into two batch slices."""
     ta = _mods()
@@ -457,7 +457,7 @@ def test_terapipe_other_head_dims(dtype, Dh):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
 def test_slicing_invariance_full_width(dtype):
-    """Size-independent property at a BASELINE width (hidden 2048, 16 heads, seq 2048): gradients with 8
+    """Size-independent property at a benchmark width (hidden 2048, 16 heads, seq 2048): gradients with 8
     slices equal gradients with one slice (the invariant of test_transformer_terapipe.py:333-352),
     computed entirely by the HIP path."""
     ta = _mods()
@@ -794,7 +794,7 @@ def test_replay_survives_a_larger_workspace_on_the_same_stream():
 
 @pytest.mark.parametrize("n_layers,steps", [(2, 5), (24, 4)])
 def test_default_runner_matches_single_stream_at_c2_shape(n_layers, steps):
-    """BASELINE config 2's geometry (hidden 2048, 16 heads, FFN 8192, sequence 2048 as 8 x 256, fp16) on two
+    """benchmark config 2's geometry (hidden 2048, 16 heads, FFN 8192, sequence 2048 as 8 x 256, fp16) on two
     layers and on all 24: the constructor's defaults (three slice streams, launch replay) against one stream
     launched from Python, several steps -- the first as written, the second recorded, the rest re-issued.  Same
     kernels on the same data: outputs and input gradients are bit-identical; the parameter gradients (fp32
