@@ -3,8 +3,8 @@ slice list as the configs state them, on one or two layers of the stack (the CPU
 layer count).  test_full_width_against_the_oracle runs configs 4 and 5 on a prefix of the sequence (the first
 1024 of 2048 positions = 8 of 16 slices of 128 tokens; the first 512 = 16 of 64 slices of 32 tokens, batch 2)
 with the eager runner on one and on three streams; test_full_length_default_runner_against_the_oracle runs
-both at all 2048 positions, and config 3 with all five layers of its stage (the workload the benchmark times),
-through the runner as it is constructed by default (three slice streams, launch replay) and compares the first
+both at all 2048 positions, and configs 2 and 3 with all their layers (24 and 5: the workloads as the benchmark times
+them), through the runner as it is constructed by default (three slice streams, launch replay) and compares the first
 step (eager) and the third (re-issued from the recorded launches).
 
 Compared per tensor (max |got - ref| / max |ref| <= 2e-2): the output, the input gradient, the final K/V
@@ -31,8 +31,9 @@ FULL_WIDTH = {
     "C5": (1, 6144, 48, 24576, 512, 2, torch.bfloat16, [32] * 16, 0.02),
     "C4-full": (1, 12288, 96, 49152, 2048, 1, torch.bfloat16, [128] * 16, 0.006),
     "C5-full": (1, 6144, 48, 24576, 2048, 2, torch.bfloat16, [32] * 64, 0.02),
-    # the benchmark's default workload as it is timed: all five layers of the stage
+    # configs 3 and 2 as the benchmark times them: every layer
     "C3-full": (5, 5120, 40, 20480, 2048, 1, torch.float16, [512, 384, 320, 256, 224, 192, 160], 0.02),
+    "C2-full": (24, 2048, 16, 8192, 2048, 1, torch.float16, [256] * 8, 0.02),
 }
 
 
@@ -158,10 +159,10 @@ def test_full_width_layer_surface_against_the_oracle(in_place, defer):
     assert all(not layer._grad_options.pending for layer in layers.layers), "a deferred sequence was left open"
 
 
-@pytest.mark.parametrize("name", ["C4-full", "C5-full", "C3-full"])
+@pytest.mark.parametrize("name", ["C4-full", "C5-full", "C3-full", "C2-full"])
 def test_full_length_default_runner_against_the_oracle(name):
-    """All 2048 positions of configs 4 and 5 (one layer) and of config 3 with all five layers of its stage -- the
-    workload the benchmark times -- through the runner as constructed by default (three slice streams,
+    """All 2048 positions of configs 4 and 5 (one layer) and of configs 2 and 3 with all their layers (24 and 5) -- the
+    workloads as the benchmark times them -- through the runner as constructed by default (three slice streams,
     launch replay): inside the runner this is what reaches the forward's key split (from 1024 keys on), the
     one-pass dK/dV over a tail of up to 2016 positions, and (config 5) the fused attention backward on lanes.
     Step 1 runs eagerly, step 2 records, step 3 is re-issued from the record; steps 1 and 3 are each compared
